@@ -1,0 +1,18 @@
+"""MI355X-native attention hot path for Daisy.
+
+Hand-written gfx950 HIP kernels (``daisy_amd/csrc``, C ABI in
+``include/daisy_hip.h``) behind the reference's own Python interfaces:
+``CausalSelfAttention``, ``KVCache``, ``Generator``, ``chunk_kda`` and
+``fused_kda_gate``.
+"""
+from .attention import (CausalSelfAttention, Rotary, WindowMask, build_window_mask,  # noqa: F401
+                        dense_mask_to_window, doc_start_from_ids)
+from .functional import norm  # noqa: F401
+from .generate import Generator  # noqa: F401
+from .kda import chunk_kda, fused_kda_gate  # noqa: F401
+from .kv_cache import KVCache, RingContext  # noqa: F401
+
+__all__ = [
+    "CausalSelfAttention", "Rotary", "WindowMask", "build_window_mask", "dense_mask_to_window",
+    "doc_start_from_ids", "norm", "Generator", "chunk_kda", "fused_kda_gate", "KVCache", "RingContext",
+]

@@ -1,0 +1,271 @@
+"""Drop-in ``CausalSelfAttention`` / ``Rotary`` backed by the gfx950 kernels.
+
+Mirrors models/daisy/attention.py of the reference: same constructor, same
+state-dict keys (``qkvo_w``, optional ``g_ve``), same ``forward`` / ``prefill`` /
+``step`` / ``reset_history`` signatures, shapes and dtypes.  The QKV and output
+projections and the weightless RMS norms stay PyTorch library calls; RoPE, the
+mask and the attention itself run in ``libdaisy_hip.so``.  Inference only: the
+kernels have no backward.
+
+Masks.  The reference passes a dense additive ``[1, 1, T, T]`` mask built by
+``build_attn_mask`` (models/daisy/daisy_core.py:53-69).  Here the mask is the
+light descriptor ``WindowMask(window, doc_start)``; ``build_window_mask`` makes
+one from token ids.  A dense reference mask is still accepted and converted
+(each row must allow one contiguous run of keys ending at the query).
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import Optional, Union
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from . import ops
+from .functional import init_linear, norm
+from .kv_cache import RingContext
+
+
+@dataclass
+class WindowMask:
+    """``0 <= q - k < window`` and ``k >= doc_start[q]``.
+
+    ``window``: keys visible per query including itself (``None`` = unlimited).
+    ``doc_start``: int32 ``[T]`` on the GPU, first position of each query's
+    document, or ``None`` for a single document.
+    """
+    window: Optional[int]
+    doc_start: Optional[Tensor] = None
+
+
+def doc_start_from_ids(input_seq: Tensor, eos_token_id: int) -> Tensor:
+    """int32 ``[T]``: position of the latest EOS at or before each token (0 if none).
+
+    The reference numbers documents with ``cumsum(ids == eos)``
+    (models/daisy/daisy_core.py:60), so an EOS token opens its own document.
+    """
+    ids = input_seq.reshape(-1)
+    pos = torch.arange(ids.numel(), device=ids.device, dtype=torch.int32)
+    marks = torch.where(ids == eos_token_id, pos, torch.zeros_like(pos))
+    return torch.cummax(marks, dim=0).values.to(torch.int32).contiguous()
+
+
+def build_window_mask(input_seq: Tensor, window_size: Optional[int], eos_token_id: Optional[int]) -> WindowMask:
+    """Descriptor equivalent of the reference's ``build_attn_mask`` (no T x T tensor)."""
+    ds = None if eos_token_id is None else doc_start_from_ids(input_seq, eos_token_id)
+    return WindowMask(window_size, ds)
+
+
+def dense_mask_to_window(attn_mask: Tensor) -> WindowMask:
+    """Converts a reference-style additive mask ``[..., T, T]`` to a ``WindowMask``.
+
+    Raises if some row is not a single run of allowed keys ending at the query.
+    """
+    m = attn_mask.reshape(-1, attn_mask.shape[-2], attn_mask.shape[-1])
+    torch._assert(m.shape[0] == 1, "a dense attn_mask must broadcast over batch and heads")
+    allowed = m[0] == 0
+    T = allowed.shape[0]
+    pos = torch.arange(T, device=allowed.device)
+    first = torch.argmax(allowed.to(torch.int8), dim=1)
+    count = allowed.sum(dim=1)
+    band = (pos[None, :] >= first[:, None]) & (pos[None, :] <= pos[:, None])
+    if not bool((count == pos - first + 1).all()) or not bool((allowed == band).all()):
+        raise ValueError("attn_mask is not a causal band per row; only window/document masks are supported")
+    return WindowMask(None, first.to(torch.int32).contiguous())
+
+
+MaskLike = Union[None, WindowMask, Tensor]
+
+
+def _as_window_mask(attn_mask: MaskLike) -> WindowMask:
+    if attn_mask is None:
+        return WindowMask(None, None)
+    if isinstance(attn_mask, WindowMask):
+        return attn_mask
+    if isinstance(attn_mask, Tensor):
+        return dense_mask_to_window(attn_mask)
+    raise TypeError(f"unsupported attn_mask type {type(attn_mask).__name__}")
+
+
+def _apply_rope(x_BTHD: Tensor, cos: Tensor, sin: Tensor) -> Tensor:
+    # Used for single-token tensors only; the prefill kernel rotates in registers.
+    x1, x2 = x_BTHD.to(dtype=torch.float32).chunk(2, dim=-1)
+    y1 = x1 * cos + x2 * sin
+    y2 = x1 * (-sin) + x2 * cos
+    return torch.cat((y1, y2), dim=-1).type_as(x_BTHD)
+
+
+class Rotary(nn.Module):
+    """Half-truncated RoPE tables (models/daisy/attention.py:26-70).
+
+    The first ``dim // 4`` frequencies are ``(1/1024) ** linspace(0, 1, dim // 4)``,
+    the remaining ``dim // 4`` are zero; ``dim < 4`` keeps all ``dim // 2``.  Tables
+    are fp32 ``[max_seq_len, dim // 2]`` non-persistent buffers.
+    """
+
+    def __init__(self, dim: int, max_seq_len: int):
+        super().__init__()
+        half, keep = dim // 2, dim // 4
+        base = 1024
+        if keep == 0:
+            angular_freq = (1 / base) ** torch.linspace(0, 1, steps=half, dtype=torch.float32)
+        else:
+            active = (1 / base) ** torch.linspace(0, 1, steps=keep, dtype=torch.float32)
+            angular_freq = torch.cat([active, active.new_zeros(half - keep)])
+        self.inv_freq = nn.Buffer(angular_freq, persistent=False)
+        theta = torch.outer(torch.arange(max_seq_len, dtype=torch.float32), angular_freq)
+        self.cos = nn.Buffer(theta.cos(), persistent=False)
+        self.sin = nn.Buffer(theta.sin(), persistent=False)
+        self._max_seq_len = int(max_seq_len)
+
+    def _get_cos_sin(self, L):
+        torch._assert(L <= self.cos.shape[0], f"Rotary buffers too small {self.cos.shape[0]} < {L}")
+        return self.cos.narrow(0, 0, L), self.sin.narrow(0, 0, L)
+
+    def forward(self, x_BTHD: Tensor):
+        cos, sin = self._get_cos_sin(x_BTHD.size(-3))
+        return _apply_rope(x_BTHD, cos[None, :, None, :], sin[None, :, None, :])
+
+    def step(self, x_BTHD: Tensor, pos: int):
+        torch._assert(x_BTHD.size(1) == 1, "step() requires single position only")
+        cos, sin = self._get_cos_sin(pos + 1)
+        return _apply_rope(x_BTHD, cos[None, pos:pos + 1, None, :], sin[None, pos:pos + 1, None, :])
+
+
+class CausalSelfAttention(nn.Module):
+    """Merged-QKVO sliding-window causal self-attention (models/daisy/attention.py:73-202)."""
+
+    def __init__(self, dim: int, num_heads: int, head_dim, receives_ve: bool = False,
+                 layer_idx: Optional[int] = None, max_seq_len: int = 131072):
+        super().__init__()
+        torch._assert(dim % num_heads == 0, "dim must be divisible by num_heads")
+        self.num_heads = num_heads
+        self.head_dim: int = head_dim
+        self.m_dim = dim
+        self.qkvo_w = nn.Parameter(init_linear(torch.empty(4, dim, dim)).bfloat16())
+        if os.getenv("DISABLE_O_ZERO_INIT", "") != "1":
+            self.qkvo_w.detach()[3].zero_()
+        self.rotary = Rotary(head_dim, max_seq_len)
+        self.attn_scale = 0.12
+        self.last_q = None
+        self.last_k = None
+        self.receives_ve = receives_ve
+        if receives_ve:
+            # Gate logits per layer as in the reference (attention.py:94-106).
+            ve_init_logits = {0: 0.3228, 1: 0.0, 2: -1.5163, 21: -2.4423, 22: -2.9444, 23: 10.0}
+            init_val = ve_init_logits.get(layer_idx, 0.0) if layer_idx is not None else 0.0
+            self.g_ve = nn.Parameter(torch.tensor(init_val))
+        else:
+            self.g_ve = None
+        self.debug_logging = False
+        # Set to True to rotate keys while they are staged into LDS instead of in a pre-pass.
+        self.rotate_k_in_kernel = False
+
+    def reset_history(self):
+        self.last_q = None
+        self.last_k = None
+
+    # -- shared pieces -------------------------------------------------------
+    def _project_qkv(self, x: Tensor):
+        """QKV projection + RMS norm of q, k and v (no RoPE); ``[B, T, H, D]`` views."""
+        B, T = x.size(0), x.size(1)
+        x = x.to(self.qkvo_w.dtype)
+        qkv = F.linear(x, self.qkvo_w[:3].flatten(end_dim=1)).view(B, T, 3 * self.num_heads, self.head_dim)
+        q, k, v = qkv.chunk(3, dim=-2)
+        return norm(q), norm(k), norm(v)
+
+    def _mix_ve(self, v: Tensor, ve: Optional[Tensor]) -> Tensor:
+        if not self.receives_ve:
+            return v
+        torch._assert(ve is not None, "ve must be provided when receives_ve=True")
+        g_x = torch.sigmoid(self.g_ve).to(v.dtype)
+        return g_x * v + (1.0 - g_x) * ve.view_as(v).to(v.dtype)
+
+    def _kernel_dtype(self, t: Tensor) -> Tensor:
+        # The kernels compute on bf16 operands; fp32 parameters (as some tests
+        # use) are rounded here and the result is widened again by the caller.
+        return t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)
+
+    def _attend(self, x: Tensor, ve: Optional[Tensor], attn_mask: MaskLike):
+        B, T = x.size(0), x.size(1)
+        mask = _as_window_mask(attn_mask)
+        q, k, v = self._project_qkv(x)
+        dtype = q.dtype
+        v = self._mix_ve(v, ve)
+        cos, sin = self.rotary._get_cos_sin(T)
+        o, k_rot = ops.prefill_attention(
+            self._kernel_dtype(q), self._kernel_dtype(k), self._kernel_dtype(v),
+            window=mask.window, scale=self.attn_scale, cos=cos, sin=sin, doc_start=mask.doc_start,
+            rotate_k_in_kernel=self.rotate_k_in_kernel)
+        y = o.view(B, T, self.m_dim).to(dtype)
+        y = F.linear(y, self.qkvo_w[3])
+        return y, k_rot.to(dtype), v
+
+    # -- reference interface -----------------------------------------------
+    def forward(self, x: Tensor, ve: Optional[Tensor], block_mask=None, attn_mask: MaskLike = None):
+        if block_mask is not None and not isinstance(block_mask, WindowMask):
+            raise NotImplementedError(
+                "flex_attention BlockMask objects (training) are not supported; pass a WindowMask")
+        y, _, _ = self._attend(x, ve, block_mask if block_mask is not None else attn_mask)
+        return y
+
+    def forward_sdpa(self, x: Tensor, ve: Optional[Tensor], attn_mask: MaskLike = None):
+        return self.forward(x, ve, attn_mask=attn_mask)
+
+    def prefill(self, x: Tensor, ve: Optional[Tensor], attn_mask: MaskLike = None, debug: bool = False):
+        """Returns ``y [B, T, dim]``, ``k [B, H, T, D]`` (normed + rotated), ``v [B, H, T, D]``."""
+        y, k, v = self._attend(x, ve, attn_mask)
+        if debug:
+            self.last_k = k
+        return y, k.transpose(1, 2), v.transpose(1, 2)
+
+    def step(self, x, k_ctx: Union[Tensor, RingContext], v_ctx: Union[Tensor, RingContext], pos: int,
+             ve: Optional[Tensor], window: Optional[int]):
+        """One token: returns ``y [B, 1, dim]``, ``k [B, 1, H, D]``, ``v [B, 1, H, D]``.
+
+        ``k_ctx``/``v_ctx`` are either the chronological cached rows
+        ``[B, n, H, D]`` (the reference's calling convention) or the
+        ``RingContext`` of a ``KVCache`` layer, in which case the kernel streams
+        the ring in place and appends the new row itself.
+        """
+        B = x.size(0)
+        torch._assert(x.size(1) == 1, "step() requires single position only")
+        q, k, v = self._project_qkv(x)
+        dtype = q.dtype
+        v = self._mix_ve(v, ve)
+        cos, sin = self.rotary._get_cos_sin(pos + 1)
+        cos_row, sin_row = cos[pos], sin[pos]
+        qk, kk, vk = (self._kernel_dtype(t)[:, 0] for t in (q, k, v))  # [B, H, D]
+
+        ring = k_ctx if isinstance(k_ctx, RingContext) else None
+        if ring is not None and (window != ring.W or ring.k.dtype != torch.bfloat16 or pos != ring.t):
+            # Not the layout the in-place path streams; use the chronological rows.
+            k_ctx, v_ctx = ring.cache.view(ring.layer)
+            ring = None
+        if ring is not None:
+            W, t = ring.W, ring.t
+            slot = t % W
+            o = ops.decode_attention(qk, kk, vk, ring.k, ring.v, n_rows=min(t + 1, W), new_idx=slot,
+                                     write_back=True, scale=self.attn_scale, cos_row=cos_row, sin_row=sin_row)
+            ring.mark_written()
+            k_new = ring.k[:, :, slot, :].unsqueeze(1)
+            v_new = ring.v[:, :, slot, :].unsqueeze(1)
+        else:
+            n = k_ctx.size(1)
+            r = n if window is None else min(n, max(window - 1, 0))
+            k_new = _apply_rope(self._kernel_dtype(k), cos_row[None, None, None, :], sin_row[None, None, None, :])
+            v_new = self._kernel_dtype(v)
+            q_rot = _apply_rope(self._kernel_dtype(q), cos_row[None, None, None, :], sin_row[None, None, None, :])
+            if r > 0:
+                kc = self._kernel_dtype(k_ctx)[:, n - r:n].transpose(1, 2)  # [B, H, r, D] view
+                vc = self._kernel_dtype(v_ctx)[:, n - r:n].transpose(1, 2)
+            else:
+                kc = vc = None
+            o = ops.decode_attention(q_rot[:, 0], k_new[:, 0], v_new[:, 0], kc, vc, n_rows=r + 1, new_idx=r,
+                                     write_back=False, scale=self.attn_scale)
+            k_new, v_new = k_new.to(dtype), v_new.to(dtype)
+        y = o.reshape(B, 1, self.m_dim).to(dtype)
+        y = F.linear(y, self.qkvo_w[3])
+        return y, k_new, v_new

@@ -1,0 +1,368 @@
+// Kernel 2: split-K single-token decode over a bf16 KV cache (gfx950).
+//
+// One workgroup (4 wavefronts) streams a contiguous range of cache rows of one
+// (batch, head).  A row of D bf16 is covered by D/8 lanes with one 16-byte
+// load each, so a wavefront load instruction fetches 64*16 = 1 KiB of
+// consecutive cache bytes.  Every group of D/8 lanes keeps its own online
+// softmax state (max, sum, 8 output channels); the groups of a wavefront are
+// merged with cross-lane moves, the wavefronts of a workgroup through LDS, and
+// the splits of a (batch, head) -- when there are several -- by a second tiny
+// kernel over fp32 partials in the caller's workspace.
+//
+// HBM traffic per step is the K and V rows once: B*H*n_rows*D*2*2 bytes.
+#include "common.h"
+
+namespace daisy {
+
+struct DecodeParams {
+  const uint16_t* q; int64_t q_sb, q_sh;
+  const uint16_t* k_new; int64_t kn_sb, kn_sh;
+  const uint16_t* v_new; int64_t vn_sb, vn_sh;
+  uint16_t* kc; int64_t kc_sb, kc_sh, kc_sr;
+  uint16_t* vc; int64_t vc_sb, vc_sh, vc_sr;
+  const float* cos_row; const float* sin_row;
+  uint16_t* o; int64_t o_sb, o_sh;
+  float* partials;  // [B, H, nsplit, D + 2] when nsplit > 1
+  int B, H, n_rows, new_idx, write_back, nsplit, rows_per_split;
+  float scale_log2e;
+};
+
+constexpr int kDecodeThreads = 256;
+constexpr int kDecodeWaves = kDecodeThreads / 64;
+constexpr int kDecodeUnroll = 8;  // 16-byte loads in flight per lane and tensor
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+  int y = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false);
+  return x + __int_as_float(y);
+}
+
+// Sum over the LPR consecutive lanes that share a cache row; every lane of the
+// group ends with the total.
+template <int LPR>
+__device__ __forceinline__ float group_sum(float x) {
+  x = dpp_add<0xB1>(x);                     // quad_perm [1,0,3,2]   (xor 1)
+  x = dpp_add<0x4E>(x);                     // quad_perm [2,3,0,1]   (xor 2)
+  if (LPR >= 8) x = dpp_add<0x141>(x);      // row_half_mirror       (joins the two quads of 8 lanes)
+  if (LPR >= 16) x = dpp_add<0x128>(x);     // row_ror 8             (joins the two halves of 16 lanes)
+  return x;
+}
+
+// Loads this lane's 8 channels of a [D] bf16 vector, optionally rotates them
+// with the position's cos/sin row (pairs (i, i + D/2)), rounds to bf16 like the
+// reference does after RoPE, and returns them as floats.
+template <int D>
+__device__ __forceinline__ void load_vec_rot(const uint16_t* vec, int dl, const float* cos_row, const float* sin_row,
+                                             float* out) {
+  u32x4 own = *reinterpret_cast<const u32x4*>(vec + dl);
+  unpack8(own, out);
+  if (cos_row != nullptr) {
+    constexpr int HALF = D / 2;
+    const bool lower = dl < HALF;
+    const int pl = lower ? dl + HALF : dl - HALF;
+    u32x4 par = *reinterpret_cast<const u32x4*>(vec + pl);
+    float pf[8];
+    unpack8(par, pf);
+    const int tl = lower ? dl : dl - HALF;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float c = cos_row[tl + i], s = sin_row[tl + i];
+      const float y = lower ? rope_lo(out[i], pf[i], c, s) : rope_hi(pf[i], out[i], c, s);
+      out[i] = round_bf16(y);
+    }
+  }
+}
+
+struct SoftmaxState {
+  float m, l;
+  float acc[8];
+};
+
+// Merges `b` into `a` (both may be empty, i.e. m == -inf).
+__device__ __forceinline__ void merge_state(SoftmaxState& a, const SoftmaxState& b) {
+  const float m = fmaxf(a.m, b.m);
+  const float mu = (m == -INFINITY) ? 0.f : m;
+  const float sa = fast_exp2(a.m - mu), sb = fast_exp2(b.m - mu);
+  a.l = a.l * sa + b.l * sb;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a.acc[i] = a.acc[i] * sa + b.acc[i] * sb;
+  a.m = m;
+}
+
+template <int D>
+__global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) {
+  constexpr int LPR = D / 8;        // lanes per cache row
+  constexpr int RPW = 64 / LPR;     // rows per wavefront load
+  constexpr int U = kDecodeUnroll;
+  constexpr int RB = RPW * U;       // rows per wavefront iteration
+
+  const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int sub = lane / LPR;
+  const int dl = (lane % LPR) * 8;
+
+  float qf[8], knf[8];
+  load_vec_rot<D>(p.q + b * p.q_sb + h * p.q_sh, dl, p.cos_row, p.sin_row, qf);
+  load_vec_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_row, p.sin_row, knf);
+  const u32x4 vn_packed = *reinterpret_cast<const u32x4*>(p.v_new + b * p.vn_sb + h * p.vn_sh + dl);
+  const u32x4 kn_packed = pack8(knf);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) qf[i] *= p.scale_log2e;
+
+  const int r0 = split * p.rows_per_split;
+  const int r1 = min(r0 + p.rows_per_split, p.n_rows);
+  uint16_t* kbase = p.kc + b * p.kc_sb + h * p.kc_sh + dl;
+  uint16_t* vbase = p.vc + b * p.vc_sb + h * p.vc_sh + dl;
+
+  SoftmaxState st;
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) st.acc[i] = 0.f;
+
+  // Lanes whose row is past the range, or is the new token's slot, load a row
+  // that is always readable instead (and are masked / overwritten below).
+  const int safe_row = (r0 != p.new_idx) ? r0 : r0 + 1;
+  const uint16_t* k_safe = (safe_row < r1) ? kbase + (int64_t)safe_row * p.kc_sr : p.k_new + b * p.kn_sb + h * p.kn_sh + dl;
+  const uint16_t* v_safe = (safe_row < r1) ? vbase + (int64_t)safe_row * p.vc_sr : p.v_new + b * p.vn_sb + h * p.vn_sh + dl;
+
+  for (int base = r0 + wave * RB; base < r1; base += kDecodeWaves * RB) {
+    u32x4 kr[U], vr[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int row = base + u * RPW + sub;
+      const uint16_t* a = (row < r1 && row != p.new_idx) ? kbase + (int64_t)row * p.kc_sr : k_safe;
+      kr[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int row = base + u * RPW + sub;
+      const uint16_t* a = (row < r1 && row != p.new_idx) ? vbase + (int64_t)row * p.vc_sr : v_safe;
+      vr[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a));
+    }
+
+    float s[U];
+    float mblk = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int row = base + u * RPW + sub;
+      if (row == p.new_idx && row < r1) {
+        kr[u] = kn_packed;
+        vr[u] = vn_packed;
+        if (p.write_back) {
+          *reinterpret_cast<u32x4*>(kbase + (int64_t)row * p.kc_sr) = kn_packed;
+          *reinterpret_cast<u32x4*>(vbase + (int64_t)row * p.vc_sr) = vn_packed;
+        }
+      }
+      float kf[8];
+      unpack8(kr[u], kf);
+      float d = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) d = fmaf(qf[i], kf[i], d);
+      d = group_sum<LPR>(d);
+      s[u] = (row < r1) ? d : -INFINITY;
+      mblk = fmaxf(mblk, s[u]);
+    }
+
+    const float mnew = fmaxf(st.m, mblk);
+    const float mu = (mnew == -INFINITY) ? 0.f : mnew;
+    const float alpha = fast_exp2(st.m - mu);
+    st.m = mnew;
+    st.l *= alpha;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) st.acc[i] *= alpha;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float pu = fast_exp2(s[u] - mu);
+      st.l += pu;
+      float vf[8];
+      unpack8(vr[u], vf);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) st.acc[i] = fmaf(pu, vf[i], st.acc[i]);
+    }
+  }
+
+  // Merge the row groups of this wavefront (lanes that differ above bit log2(LPR)).
+#pragma unroll
+  for (int off = LPR; off < 64; off <<= 1) {
+    SoftmaxState o;
+    o.m = __shfl_xor(st.m, off);
+    o.l = __shfl_xor(st.l, off);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o.acc[i] = __shfl_xor(st.acc[i], off);
+    merge_state(st, o);
+  }
+
+  // Merge the wavefronts through LDS.
+  __shared__ float sm_m[kDecodeWaves], sm_l[kDecodeWaves];
+  __shared__ float sm_acc[kDecodeWaves][D];
+  if (lane < LPR) {
+    if (lane == 0) {
+      sm_m[wave] = st.m;
+      sm_l[wave] = st.l;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sm_acc[wave][dl + i] = st.acc[i];
+  }
+  __syncthreads();
+  if (wave == 0 && lane < LPR) {
+#pragma unroll
+    for (int w = 1; w < kDecodeWaves; ++w) {
+      SoftmaxState o;
+      o.m = sm_m[w];
+      o.l = sm_l[w];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o.acc[i] = sm_acc[w][dl + i];
+      merge_state(st, o);
+    }
+    if (p.nsplit == 1) {
+      const float inv = 1.f / st.l;
+      float of[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) of[i] = st.acc[i] * inv;
+      *reinterpret_cast<u32x4*>(p.o + b * p.o_sb + h * p.o_sh + dl) = pack8(of);
+    } else {
+      float* part = p.partials + (((int64_t)b * p.H + h) * p.nsplit + split) * (D + 2);
+      if (lane == 0) {
+        part[0] = st.m;
+        part[1] = st.l;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) part[2 + dl + i] = st.acc[i];
+    }
+  }
+}
+
+// Combines the per-split partials of one (batch, head); one thread per channel.
+template <int D>
+__global__ __launch_bounds__(D) void decode_combine_kernel(DecodeParams p) {
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const float* part = p.partials + ((int64_t)b * p.H + h) * p.nsplit * (D + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < p.nsplit; ++s) m = fmaxf(m, part[s * (D + 2)]);
+  float l = 0.f, acc = 0.f;
+  for (int s = 0; s < p.nsplit; ++s) {
+    const float w = fast_exp2(part[s * (D + 2)] - m);
+    l += part[s * (D + 2) + 1] * w;
+    acc += part[s * (D + 2) + 2 + d] * w;
+  }
+  const float r = acc / l;
+  p.o[b * p.o_sb + h * p.o_sh + d] = (uint16_t)(pack_bf16x2(r, 0.f) & 0xffffu);
+}
+
+static int choose_nsplit(int B, int H, int n_rows) {
+  // Aim for about 2048 workgroups on the 256 compute units, keep at least 256
+  // rows per workgroup so every wavefront has two full iterations.
+  const int bh = B * H;
+  int ns = (2048 + bh - 1) / bh;
+  const int max_by_rows = n_rows / 256 > 0 ? n_rows / 256 : 1;
+  if (ns > max_by_rows) ns = max_by_rows;
+  if (ns < 1) ns = 1;
+  if (ns > 64) ns = 64;
+  return ns;
+}
+
+static int resolve_nsplit(int B, int H, int n_rows, int nsplit) {
+  if (nsplit <= 0) nsplit = choose_nsplit(B, H, n_rows);
+  if (nsplit > n_rows) nsplit = n_rows;
+  if (nsplit < 1) nsplit = 1;
+  const int rps = (n_rows + nsplit - 1) / nsplit;
+  // Drop splits that would be empty after rounding rows_per_split up.
+  return (n_rows + rps - 1) / rps;
+}
+
+}  // namespace daisy
+
+using namespace daisy;
+
+extern "C" size_t daisy_decode_workspace_bytes(int B, int H, int D, int n_rows, int nsplit) {
+  if (B <= 0 || H <= 0 || D <= 0 || n_rows <= 0) return 0;
+  const int ns = resolve_nsplit(B, H, n_rows, nsplit);
+  if (ns == 1) return 0;
+  return (size_t)B * H * ns * (D + 2) * sizeof(float);
+}
+
+extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
+                                const void* k_new, const int64_t* k_new_strides,
+                                const void* v_new, const int64_t* v_new_strides,
+                                void* k_cache, const int64_t* k_cache_strides,
+                                void* v_cache, const int64_t* v_cache_strides,
+                                const float* cos_row, const float* sin_row,
+                                void* o, const int64_t* o_strides,
+                                int B, int H, int D,
+                                int n_rows, int new_idx, int write_back,
+                                float scale, int nsplit,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  DAISY_CHECK_ARG(q && k_new && v_new && o, "decode: q, k_new, v_new and o must be non-NULL");
+  DAISY_CHECK_ARG(q_strides && k_new_strides && v_new_strides && o_strides, "decode: stride arrays must be non-NULL");
+  DAISY_CHECK_ARG(B > 0 && H > 0, "decode: B=%d and H=%d must be positive", B, H);
+  DAISY_CHECK_ARG(B <= 65535 && H <= 65535, "decode: B=%d and H=%d must each be <= 65535", B, H);
+  DAISY_CHECK_SUPPORTED(D == 64 || D == 128, "decode: head_dim %d not supported (64 or 128)", D);
+  DAISY_CHECK_ARG(n_rows >= 1, "decode: n_rows=%d must be >= 1 (the new token is always attended)", n_rows);
+  DAISY_CHECK_ARG(new_idx >= 0 && new_idx < n_rows, "decode: new_idx=%d outside [0, %d)", new_idx, n_rows);
+  DAISY_CHECK_ARG((cos_row == nullptr) == (sin_row == nullptr), "decode: cos_row and sin_row must both be given or both NULL");
+  DAISY_CHECK_ARG(n_rows == 1 || (k_cache && v_cache && k_cache_strides && v_cache_strides),
+                  "decode: cache pointers and strides are required when n_rows > 1");
+  DAISY_CHECK_ARG(!write_back || (k_cache && v_cache), "decode: write_back needs cache pointers");
+  auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+  DAISY_CHECK_ARG(al16(q) && al16(k_new) && al16(v_new) && al16(o) && al16(k_cache) && al16(v_cache),
+                  "decode: tensors must be 16-byte aligned");
+  static const int64_t zero3[3] = {0, 0, 0};
+  if (!k_cache_strides) k_cache_strides = zero3;
+  if (!v_cache_strides) v_cache_strides = zero3;
+  for (int i = 0; i < 2; ++i) {
+    DAISY_CHECK_ARG(q_strides[i] % 8 == 0 && k_new_strides[i] % 8 == 0 && v_new_strides[i] % 8 == 0 && o_strides[i] % 8 == 0,
+                    "decode: vector strides must be multiples of 8 elements");
+  }
+  for (int i = 0; i < 3; ++i) {
+    DAISY_CHECK_ARG(k_cache_strides[i] % 8 == 0 && v_cache_strides[i] % 8 == 0,
+                    "decode: cache strides must be multiples of 8 elements");
+  }
+
+  DecodeParams p;
+  p.q = (const uint16_t*)q; p.q_sb = q_strides[0]; p.q_sh = q_strides[1];
+  p.k_new = (const uint16_t*)k_new; p.kn_sb = k_new_strides[0]; p.kn_sh = k_new_strides[1];
+  p.v_new = (const uint16_t*)v_new; p.vn_sb = v_new_strides[0]; p.vn_sh = v_new_strides[1];
+  p.kc = (uint16_t*)k_cache; p.kc_sb = k_cache_strides[0]; p.kc_sh = k_cache_strides[1]; p.kc_sr = k_cache_strides[2];
+  p.vc = (uint16_t*)v_cache; p.vc_sb = v_cache_strides[0]; p.vc_sh = v_cache_strides[1]; p.vc_sr = v_cache_strides[2];
+  if (n_rows == 1 && !k_cache) {
+    // Only the new row exists; give the kernel a readable dummy row.
+    p.kc = (uint16_t*)k_new; p.kc_sb = k_new_strides[0]; p.kc_sh = k_new_strides[1]; p.kc_sr = 0;
+    p.vc = (uint16_t*)v_new; p.vc_sb = v_new_strides[0]; p.vc_sh = v_new_strides[1]; p.vc_sr = 0;
+    write_back = 0;
+  }
+  p.cos_row = cos_row; p.sin_row = sin_row;
+  p.o = (uint16_t*)o; p.o_sb = o_strides[0]; p.o_sh = o_strides[1];
+  p.B = B; p.H = H; p.n_rows = n_rows; p.new_idx = new_idx; p.write_back = write_back;
+  p.nsplit = resolve_nsplit(B, H, n_rows, nsplit);
+  p.rows_per_split = (n_rows + p.nsplit - 1) / p.nsplit;
+  p.scale_log2e = scale * kLog2e;
+  p.partials = nullptr;
+  if (p.nsplit > 1) {
+    const size_t need = (size_t)B * H * p.nsplit * (D + 2) * sizeof(float);
+    if (!workspace || workspace_bytes < need) {
+      set_error("decode: workspace of %zu bytes needed for %d splits, got %zu", need, p.nsplit, workspace_bytes);
+      return DAISY_ERR_WORKSPACE;
+    }
+    p.partials = (float*)workspace;
+  }
+
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(p.nsplit, H, B);
+  if (D == 128) {
+    hipLaunchKernelGGL(decode_kernel<128>, grid, dim3(kDecodeThreads), 0, s, p);
+    DAISY_CHECK_LAUNCH("decode_kernel");
+    if (p.nsplit > 1) {
+      hipLaunchKernelGGL(decode_combine_kernel<128>, dim3(H, B), dim3(128), 0, s, p);
+      DAISY_CHECK_LAUNCH("decode_combine_kernel");
+    }
+  } else {
+    hipLaunchKernelGGL(decode_kernel<64>, grid, dim3(kDecodeThreads), 0, s, p);
+    DAISY_CHECK_LAUNCH("decode_kernel");
+    if (p.nsplit > 1) {
+      hipLaunchKernelGGL(decode_combine_kernel<64>, dim3(H, B), dim3(64), 0, s, p);
+      DAISY_CHECK_LAUNCH("decode_combine_kernel");
+    }
+  }
+  return DAISY_OK;
+}

@@ -1,0 +1,21 @@
+"""Elementwise helpers that stay in PyTorch (library routines on either side)."""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor
+
+
+def norm(x: Tensor) -> Tensor:
+    """Weightless RMS norm over the last dim, eps = finfo(dtype).eps.
+
+    Same call as the reference's ``norm`` (models/daisy/functional.py:6-7).
+    """
+    return F.rms_norm(x, (x.size(-1),))
+
+
+@torch.no_grad()
+def init_linear(w: Tensor) -> Tensor:
+    """Uniform init with std 0.5 / sqrt(fan_in) (models/daisy/functional.py:10-14)."""
+    bound = (3 ** 0.5) * 0.5 * (w.size(-1) ** -0.5)
+    return w.uniform_(-bound, bound)

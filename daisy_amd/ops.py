@@ -1,0 +1,212 @@
+"""Tensor-level entry points over the C ABI (one function per kernel).
+
+These take and return ``torch`` tensors on an AMD GPU and do nothing but
+validate, allocate outputs and pass raw pointers to ``libdaisy_hip.so``.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+ATTN_SCALE = 0.12  # the reference's constant softmax scale (models/daisy/attention.py:88)
+
+
+def _check_bf16(name: str, t: torch.Tensor, ndim: int) -> None:
+    if t.dtype != torch.bfloat16:
+        raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
+    if t.dim() != ndim:
+        raise ValueError(f"{name} must have {ndim} dims, got shape {tuple(t.shape)}")
+    if t.stride(-1) != 1:
+        raise ValueError(f"{name} must be contiguous in its last dim")
+
+
+def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *,
+                      window: Optional[int], scale: float = ATTN_SCALE,
+                      cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                      doc_start: Optional[torch.Tensor] = None,
+                      out: Optional[torch.Tensor] = None, k_out: Optional[torch.Tensor] = None,
+                      rotate_k_in_kernel: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Sliding-window causal attention over ``[B, T, H, D]`` bf16 tensors.
+
+    ``cos``/``sin`` (fp32 ``[>=T, D/2]``) rotate q and k inside the call;
+    ``doc_start`` (int32 ``[T]``) confines each query to its document; ``window``
+    counts the visible keys including the query itself (``None``/``<=0`` = full
+    causal).  Returns ``(o, k_rot)``: ``o`` is ``[B, T, H, D]`` bf16 and ``k_rot``
+    the rotated keys (``None`` without ``cos``/``sin``).
+    """
+    dev = _lib.require_gpu(q, k, v, cos, sin, doc_start, out, k_out)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_bf16(name, t, 4)
+    B, T, H, D = q.shape
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError(f"q, k, v shapes differ: {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    if (cos is None) != (sin is None):
+        raise ValueError("cos and sin must be given together")
+    if cos is not None:
+        for name, t in (("cos", cos), ("sin", sin)):
+            if t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != D // 2 or not t.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous fp32 [rows, {D // 2}] table, got {tuple(t.shape)} {t.dtype}")
+            torch._assert(T <= t.shape[0], f"Rotary buffers too small {t.shape[0]} < {T}")
+    if doc_start is not None:
+        if doc_start.dtype != torch.int32 or doc_start.shape != (T,) or not doc_start.is_contiguous():
+            raise ValueError("doc_start must be a contiguous int32 [T] tensor")
+    if out is None:
+        out = torch.empty((B, T, H, D), dtype=torch.bfloat16, device=dev)
+    else:
+        _check_bf16("out", out, 4)
+    if cos is not None and k_out is None:
+        k_out = torch.empty((B, T, H, D), dtype=torch.bfloat16, device=dev)
+    if k_out is not None:
+        _check_bf16("k_out", k_out, 4)
+        if cos is None:
+            raise ValueError("k_out is only produced when cos/sin are given")
+    w = 0 if window is None else int(window)
+    flags = _lib.PREFILL_ROTATE_K_IN_KERNEL if rotate_k_in_kernel else 0
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.daisy_prefill_fwd(
+            q.data_ptr(), _lib.strides(q, (0, 1, 2)),
+            k.data_ptr(), _lib.strides(k, (0, 1, 2)),
+            v.data_ptr(), _lib.strides(v, (0, 1, 2)),
+            _lib.ptr(cos), _lib.ptr(sin), _lib.ptr(doc_start),
+            out.data_ptr(), _lib.strides(out, (0, 1, 2)),
+            _lib.ptr(k_out), None if k_out is None else _lib.strides(k_out, (0, 1, 2)),
+            B, T, H, D, w, float(scale), flags, _lib.current_stream(dev))
+    _lib.check(rc, "daisy_prefill_fwd")
+    return out, k_out
+
+
+def decode_workspace_bytes(B: int, H: int, D: int, n_rows: int, nsplit: int = 0) -> int:
+    return int(_lib.load().daisy_decode_workspace_bytes(B, H, D, n_rows, nsplit))
+
+
+def decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
+                     k_rows: Optional[torch.Tensor], v_rows: Optional[torch.Tensor], *,
+                     n_rows: int, new_idx: int, write_back: bool,
+                     scale: float = ATTN_SCALE,
+                     cos_row: Optional[torch.Tensor] = None, sin_row: Optional[torch.Tensor] = None,
+                     out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+                     nsplit: int = 0) -> torch.Tensor:
+    """One decode step for every (batch, head).
+
+    ``q``, ``k_new``, ``v_new``: bf16 ``[B, H, D]`` (any batch/head strides).
+    ``k_rows``/``v_rows``: bf16 tensors addressed as ``[B, H, rows, D]`` through
+    their strides (dims 0, 1, 2); logical rows ``0..n_rows-1`` are attended,
+    except that row ``new_idx`` is taken from ``k_new``/``v_new`` (after RoPE
+    with ``cos_row``/``sin_row``) and stored back when ``write_back``.
+    Returns ``o`` bf16 ``[B, H, D]``.
+    """
+    dev = _lib.require_gpu(q, k_new, v_new, k_rows, v_rows, cos_row, sin_row, out, workspace)
+    for name, t in (("q", q), ("k_new", k_new), ("v_new", v_new)):
+        _check_bf16(name, t, 3)
+    B, H, D = q.shape
+    if k_new.shape != q.shape or v_new.shape != q.shape:
+        raise ValueError("q, k_new, v_new must all be [B, H, D]")
+    if k_rows is not None:
+        _check_bf16("k_rows", k_rows, 4)
+        _check_bf16("v_rows", v_rows, 4)
+    if out is None:
+        out = torch.empty((B, H, D), dtype=torch.bfloat16, device=dev)
+    else:
+        _check_bf16("out", out, 3)
+    lib = _lib.load()
+    need = int(lib.daisy_decode_workspace_bytes(B, H, D, n_rows, nsplit))
+    if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(dev):
+        rc = lib.daisy_decode_fwd(
+            q.data_ptr(), _lib.strides(q, (0, 1)),
+            k_new.data_ptr(), _lib.strides(k_new, (0, 1)),
+            v_new.data_ptr(), _lib.strides(v_new, (0, 1)),
+            _lib.ptr(k_rows), None if k_rows is None else _lib.strides(k_rows, (0, 1, 2)),
+            _lib.ptr(v_rows), None if v_rows is None else _lib.strides(v_rows, (0, 1, 2)),
+            _lib.ptr(cos_row), _lib.ptr(sin_row),
+            out.data_ptr(), _lib.strides(out, (0, 1)),
+            B, H, D, int(n_rows), int(new_idx), 1 if write_back else 0,
+            float(scale), int(nsplit),
+            _lib.ptr(workspace), ws_bytes, _lib.current_stream(dev))
+    _lib.check(rc, "daisy_decode_fwd")
+    return out
+
+
+def kda_workspace_bytes(B: int, T: int, H: int, Dk: int, Dv: int, chunk: int = 64) -> int:
+    return int(_lib.load().daisy_kda_workspace_bytes(B, T, H, Dk, Dv, chunk))
+
+
+def kda_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, *,
+                  scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
+                  output_final_state: bool = False, use_qk_l2norm_in_kernel: bool = True,
+                  l2_eps: float = 1e-6, chunk: int = 64,
+                  workspace: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Chunked KDA forward; see ``daisy_kda_chunk_fwd`` in ``include/daisy_hip.h``."""
+    dev = _lib.require_gpu(q, k, v, g, beta, initial_state, workspace)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_bf16(name, t, 4)
+    B, T, H, Dk = q.shape
+    Dv = v.shape[-1]
+    if k.shape != q.shape or g.shape != q.shape or v.shape[:3] != q.shape[:3] or beta.shape != (B, T, H):
+        raise ValueError("kda: expected q,k,g [B,T,H,Dk], v [B,T,H,Dv], beta [B,T,H]")
+    if g.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"g must be fp32 or bf16, got {g.dtype}")
+    q, k, v, g = q.contiguous(), k.contiguous(), v.contiguous(), g.contiguous()
+    beta = beta.to(torch.float32).contiguous()
+    if scale is None:
+        scale = Dk ** -0.5
+    if initial_state is not None:
+        if initial_state.shape != (B, H, Dk, Dv):
+            raise ValueError(f"initial_state must be [B,H,Dk,Dv], got {tuple(initial_state.shape)}")
+        initial_state = initial_state.to(torch.float32).contiguous()
+    o = torch.empty((B, T, H, Dv), dtype=torch.bfloat16, device=dev)
+    final = torch.empty((B, H, Dk, Dv), dtype=torch.float32, device=dev) if output_final_state else None
+    lib = _lib.load()
+    need = int(lib.daisy_kda_workspace_bytes(B, T, H, Dk, Dv, chunk))
+    if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(dev):
+        rc = lib.daisy_kda_chunk_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(),
+            g.data_ptr(), 1 if g.dtype == torch.bfloat16 else 0, beta.data_ptr(),
+            _lib.ptr(initial_state), o.data_ptr(), _lib.ptr(final),
+            B, T, H, Dk, Dv, int(chunk), float(scale), 1 if use_qk_l2norm_in_kernel else 0, float(l2_eps),
+            _lib.ptr(workspace), ws_bytes, _lib.current_stream(dev))
+    _lib.check(rc, "daisy_kda_chunk_fwd")
+    return o, final
+
+
+def kda_gate_fwd(g: torch.Tensor, A_log: torch.Tensor, head_k_dim: int,
+                 g_bias: Optional[torch.Tensor] = None, beta: float = 1.0, threshold: float = 20.0) -> torch.Tensor:
+    """``-exp(A_log[h]) * softplus(g + bias)``; ``g [..., H*Dk]`` -> ``[..., H, Dk]`` in ``g.dtype``."""
+    dev = _lib.require_gpu(g, A_log, g_bias)
+    if g.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"g must be fp32 or bf16, got {g.dtype}")
+    last = g.shape[-1]
+    if last % head_k_dim != 0:
+        raise RuntimeError("last dim must be divisible by head_k_dim")
+    H = last // head_k_dim
+    if A_log.numel() != H:
+        raise RuntimeError(f"A_log must be shape [H] or [1,1,H,1]; got {tuple(A_log.shape)} with H={H}")
+    a = A_log.detach().reshape(H).to(device=dev, dtype=torch.float32).contiguous()
+    bias = None
+    if g_bias is not None:
+        b = g_bias.detach().to(device=dev, dtype=torch.float32)
+        if b.numel() == H * head_k_dim:
+            bias = b.reshape(H, head_k_dim).contiguous()
+        elif b.numel() == H:
+            bias = b.reshape(H, 1).expand(H, head_k_dim).contiguous()
+        else:
+            raise RuntimeError(f"g_bias must be one of [(H*D,), (H,D), (1,1,H,D), (H,)]; got {tuple(b.shape)}")
+    gc = g.contiguous()
+    out = torch.empty((*g.shape[:-1], H, head_k_dim), dtype=g.dtype, device=dev)
+    rows = gc.numel() // last
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.daisy_kda_gate_fwd(gc.data_ptr(), a.data_ptr(), _lib.ptr(bias), out.data_ptr(),
+                                    rows, H, head_k_dim, 1 if g.dtype == torch.bfloat16 else 0,
+                                    float(beta), float(threshold), _lib.current_stream(dev))
+    _lib.check(rc, "daisy_kda_gate_fwd")
+    return out

@@ -1,0 +1,169 @@
+/*
+ * daisy_hip.h -- C ABI of libdaisy_hip.so, the gfx950 (MI355X) kernels behind
+ * Daisy's attention hot path.
+ *
+ * Conventions
+ *   - All tensor pointers are device pointers, borrowed for the duration of the
+ *     call.  The library never allocates or frees device memory and keeps no
+ *     tensor state; scratch space is passed in as `workspace`.
+ *   - bf16 tensors are passed as `void*` (2-byte elements, the last dimension
+ *     contiguous); strides are counted in ELEMENTS, not bytes.
+ *   - Every launch is asynchronous on `stream` (a hipStream_t passed as void*;
+ *     NULL is the default stream).  No call synchronises the host.
+ *   - Return value: DAISY_OK (0) or a negative error code; the text of the last
+ *     error on the calling thread is returned by daisy_last_error().  No C++
+ *     exception crosses this boundary.
+ *
+ * The reference is pure Python and has no FFI; each entry point names the
+ * reference call it stands in for (paths relative to the reference checkout).
+ */
+#ifndef DAISY_HIP_H
+#define DAISY_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DAISY_OK 0
+#define DAISY_ERR_INVALID_ARGUMENT (-1)
+#define DAISY_ERR_UNSUPPORTED (-2)
+#define DAISY_ERR_WORKSPACE (-3)
+#define DAISY_ERR_LAUNCH (-4)
+
+/* Text of the last error raised on this thread ("" if none). */
+const char* daisy_last_error(void);
+
+/* ABI version of this header (bumped on any signature change). */
+int daisy_abi_version(void);
+
+/* ---------------------------------------------------------------------------
+ * Kernel 1: sliding-window causal flash-attention prefill with fused RoPE.
+ *
+ * Replaces, in CausalSelfAttention._sdpa_common / prefill
+ * (models/daisy/attention.py:141-150,173-179):
+ *   rotary(q), rotary(k)            (attention.py:16-20,57-62,122-125)
+ *   build_attn_mask(...)            (models/daisy/daisy_core.py:53-69)
+ *   F.scaled_dot_product_attention  (attention.py:145,147)
+ *
+ *   o[b,t,h,:] = sum_k softmax_k(scale * <rope(q[b,t,h]), rope(k[b,k,h])>) v[b,k,h,:]
+ *   over keys k with  max(t - window + 1, doc_start[t]) <= k <= t.
+ *
+ * q, k, v, o : bf16, logical shape [B, T, H, D]; *_strides = {batch, token, head}
+ *              element strides (D contiguous).  D must be 64 or 128 for the MFMA
+ *              kernel; any other even D <= 256 runs a scalar kernel.
+ * cos, sin   : fp32 [>= T, D/2] row-major rotation tables, or both NULL when
+ *              q and k are already rotated.  Row t rotates position t with
+ *              y1 = x1*cos + x2*sin, y2 = -x1*sin + x2*cos on pairs (i, i+D/2).
+ * doc_start  : int32 [T] or NULL; doc_start[t] = index of the first token of the
+ *              document containing t (non-decreasing).  Shared by all batches,
+ *              like the reference's [1,1,T,T] mask.
+ * k_out      : bf16 [B, T, H, D] with its own strides, or NULL.  When cos/sin
+ *              are given, receives the rotated keys (what the reference's
+ *              prefill returns for the KV cache, attention.py:179); the
+ *              attention kernel then reads keys from k_out instead of rotating
+ *              them again for every query block.
+ * window     : keys visible per query INCLUDING itself; <= 0 means full causal.
+ * flags      : 0, or DAISY_PREFILL_ROTATE_K_IN_KERNEL to rotate the keys while
+ *              they are staged into LDS instead of in a pre-pass (k_out, when
+ *              given, is still written).  That is also what happens when
+ *              cos/sin are given and k_out is NULL.
+ */
+#define DAISY_PREFILL_ROTATE_K_IN_KERNEL 1
+int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
+                      const void* k, const int64_t* k_strides,
+                      const void* v, const int64_t* v_strides,
+                      const float* cos, const float* sin,
+                      const int32_t* doc_start,
+                      void* o, const int64_t* o_strides,
+                      void* k_out, const int64_t* k_out_strides,
+                      int B, int T, int H, int D,
+                      int window, float scale, int flags, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Kernel 2: split-K single-token decode over a bf16 KV cache.
+ *
+ * Replaces, in CausalSelfAttention.step (attention.py:181-202) together with
+ * KVCache.view / write (inference/kv_cache.py:26-51):
+ *   rotary.step(q, pos), rotary.step(k, pos)       (attention.py:64-70,123)
+ *   torch.cat([k_ctx[:, n-r:n], k], 1) ... SDPA    (attention.py:192-199)
+ *   cache.k[layer, :, :, t % W] = k_new             (kv_cache.py:44-51)
+ *
+ * The cache tensors are addressed as rows: row r of (b, h) starts at
+ * base + b*strides[0] + h*strides[1] + r*strides[2].  The step attends
+ * `n_rows` logical rows 0..n_rows-1; logical row `new_idx` is NOT read from the
+ * cache but taken from k_new / v_new (after RoPE), and is stored into the cache
+ * at that row when `write_back` is non-zero.  Row order is irrelevant to the
+ * result, so a ring buffer is streamed in physical order:
+ *   ring of W slots at time t:  n_rows = min(t+1, W), new_idx = t % W, write_back = 1
+ *   chronological context [B,n,H,D], r = min(n, window-1) live rows starting at
+ *   row n-r:  base += (n-r)*strides[2], n_rows = r+1, new_idx = r, write_back = 0
+ *
+ * q, k_new, v_new, o : bf16 [B, H, D]; strides = {batch, head}.
+ * cos_row, sin_row   : fp32 [D/2] rows of the rotation tables for this position
+ *                      (applied to q and k_new), or both NULL.
+ * workspace          : >= daisy_decode_workspace_bytes(...) bytes, 256-byte
+ *                      aligned; may be NULL when that function returns 0.
+ * nsplit             : number of sequence splits per (b, h); 0 = choose.
+ * D must be 64 or 128.
+ */
+size_t daisy_decode_workspace_bytes(int B, int H, int D, int n_rows, int nsplit);
+
+int daisy_decode_fwd(const void* q, const int64_t* q_strides,
+                     const void* k_new, const int64_t* k_new_strides,
+                     const void* v_new, const int64_t* v_new_strides,
+                     void* k_cache, const int64_t* k_cache_strides,
+                     void* v_cache, const int64_t* v_cache_strides,
+                     const float* cos_row, const float* sin_row,
+                     void* o, const int64_t* o_strides,
+                     int B, int H, int D,
+                     int n_rows, int new_idx, int write_back,
+                     float scale, int nsplit,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * Kernel 3: chunked Kimi Delta Attention forward.
+ *
+ * Replaces the call  chunk_kda(q, k, v, g, beta, initial_state=...,
+ * output_final_state=..., use_qk_l2norm_in_kernel=True)  at
+ * models/daisy/attention_kimi.py:133-134 (the implementation is in the absent
+ * third-party package flash-linear-attention).  Per (b, h), with fp32 state
+ * S [Dk, Dv]:
+ *   S <- diag(exp(g_t)) S;  S <- S + beta_t k_t (v_t - S^T k_t)^T;  o_t = scale * S^T q_t
+ *
+ * q, k  : bf16 [B, T, H, Dk] contiguous.     v, o : bf16 [B, T, H, Dv] contiguous.
+ * g     : log-decay [B, T, H, Dk] contiguous, fp32 (g_is_bf16 = 0) or bf16 (1); <= 0.
+ * beta  : fp32 [B, T, H] contiguous.
+ * initial_state : fp32 [B, H, Dk, Dv] or NULL (zeros).
+ * final_state   : fp32 [B, H, Dk, Dv] or NULL (not wanted).
+ * Dk = Dv = 128 and chunk = 64 are the supported shapes.  T is arbitrary.
+ * l2norm_qk : normalise q and k rows as x / sqrt(sum(x^2) + l2_eps) first.
+ * workspace : >= daisy_kda_workspace_bytes(...) bytes, 256-byte aligned.
+ */
+size_t daisy_kda_workspace_bytes(int B, int T, int H, int Dk, int Dv, int chunk);
+
+int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
+                        const void* g, int g_is_bf16, const float* beta,
+                        const float* initial_state, void* o, float* final_state,
+                        int B, int T, int H, int Dk, int Dv, int chunk,
+                        float scale, int l2norm_qk, float l2_eps,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------
+ * KDA log-decay gate:  out[..., h, d] = -exp(A_log[h]) * softplus(g[..., h, d] + bias[h, d])
+ * (softplus is the identity above `threshold`).  Replaces fused_kda_gate
+ * (models/daisy/fla_custom_ops.py:71-103,190-200), forward only.
+ *
+ * g, out : [rows, H, Dk] contiguous, both bf16 (io_is_bf16 = 1) or both fp32 (0).
+ * A_log  : fp32 [H].   bias : fp32 [H, Dk] or NULL.
+ */
+int daisy_kda_gate_fwd(const void* g, const float* A_log, const float* bias, void* out,
+                       int64_t rows, int H, int Dk, int io_is_bf16,
+                       float softplus_beta, float threshold, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DAISY_HIP_H */

@@ -1,0 +1,101 @@
+"""Kernel 2 parity: HIP split-K decode vs the fp32 oracle (through the C ABI)."""
+import pytest
+import torch
+
+import oracle
+from daisy_amd import ops
+from helpers import assert_close_bf16, say
+
+pytestmark = pytest.mark.gpu
+
+
+def _ref_decode(q, k_rows, v_rows, scale=0.12):
+    """q [B,H,D]; rows [B,H,N,D] (already holding the new row) -> fp32 [B,H,D]."""
+    return oracle.sdpa(q[:, :, None, :], k_rows, v_rows, None, scale)[:, :, 0, :]
+
+
+@pytest.mark.parametrize("B,H,D,W,t,nsplit", [
+    (2, 3, 128, 64, 10, 0),      # ring not yet wrapped
+    (2, 3, 128, 64, 63, 0),      # last free slot
+    (2, 3, 128, 64, 64, 0),      # first wrap: new row overwrites slot 0
+    (1, 2, 128, 1024, 5000, 0),  # wrapped several times, auto split
+    (1, 2, 128, 1024, 5000, 1),  # same, one workgroup per (b, h)
+    (1, 2, 128, 1024, 5000, 4),
+    (3, 2, 64, 200, 777, 0),     # D = 64, W not a multiple of the row block
+    (3, 2, 64, 200, 777, 3),
+    (1, 1, 128, 1, 9, 0),        # W = 1: only the new row
+    (4, 8, 128, 4096, 8192, 0),  # the benchmark's ring shape at small batch
+])
+def test_decode_ring_matches_oracle(B, H, D, W, t, nsplit):
+    say(f"decode ring case B{B} H{H} D{D} W{W} t{t} nsplit{nsplit}")
+    g = torch.Generator().manual_seed(W + t)
+    kc = torch.randn(B, H, W, D, generator=g).bfloat16()
+    vc = torch.randn(B, H, W, D, generator=g).bfloat16()
+    q, kn, vn = (torch.randn(B, H, D, generator=g).bfloat16() for _ in range(3))
+    cos, sin = oracle.rope_tables(D, t + 1)
+    q_rot = oracle.apply_rope(q[:, None], cos[t:t + 1], sin[t:t + 1])[:, 0]
+    k_rot = oracle.apply_rope(kn[:, None], cos[t:t + 1], sin[t:t + 1])[:, 0]
+    n_rows, slot = min(t + 1, W), t % W
+    k_exp, v_exp = kc.clone(), vc.clone()
+    k_exp[:, :, slot] = k_rot
+    v_exp[:, :, slot] = vn
+    ref = _ref_decode(q_rot, k_exp[:, :, :n_rows], v_exp[:, :, :n_rows])
+
+    dkc, dvc = kc.cuda(), vc.cuda()
+    o = ops.decode_attention(q.cuda(), kn.cuda(), vn.cuda(), dkc, dvc, n_rows=n_rows, new_idx=slot,
+                             write_back=True, cos_row=cos[t].cuda(), sin_row=sin[t].cuda(), nsplit=nsplit)
+    torch.cuda.synchronize()
+    assert_close_bf16(o, ref, "o")
+    assert torch.equal(dkc.cpu(), k_exp), "cache K after the step (only the new slot may change)"
+    assert torch.equal(dvc.cpu(), v_exp), "cache V after the step"
+
+
+@pytest.mark.parametrize("n,window", [(0, 8), (5, 8), (20, 8), (20, None), (300, 257)])
+def test_decode_chronological_context(n, window):
+    """The reference's calling convention: k_ctx [B, n, H, D] + new row, last window-1 rows live."""
+    B, H, D = 2, 2, 128
+    say(f"decode ctx case n{n} window{window}")
+    g = torch.Generator().manual_seed(n)
+    k_ctx = torch.randn(B, n, H, D, generator=g).bfloat16()
+    v_ctx = torch.randn(B, n, H, D, generator=g).bfloat16()
+    q, kn, vn = (torch.randn(B, H, D, generator=g).bfloat16() for _ in range(3))
+    r = n if window is None else min(n, max(window - 1, 0))
+    k_all = torch.cat([k_ctx[:, n - r:], kn[:, None]], 1).transpose(1, 2)
+    v_all = torch.cat([v_ctx[:, n - r:], vn[:, None]], 1).transpose(1, 2)
+    ref = _ref_decode(q, k_all, v_all)
+    dk, dv = k_ctx.cuda(), v_ctx.cuda()
+    kc = dk[:, n - r:].transpose(1, 2) if r > 0 else None
+    vc = dv[:, n - r:].transpose(1, 2) if r > 0 else None
+    o = ops.decode_attention(q.cuda(), kn.cuda(), vn.cuda(), kc, vc, n_rows=r + 1, new_idx=r, write_back=False)
+    assert_close_bf16(o, ref, "o")
+    assert torch.equal(dk.cpu(), k_ctx) and torch.equal(dv.cpu(), v_ctx), "context must not be written"
+
+
+def test_decode_consecutive_steps_append_in_place():
+    """32 steps on one preallocated ring: every output checked, no host copies in between."""
+    B, H, D, W, t0, steps = 2, 4, 128, 256, 500, 32
+    g = torch.Generator().manual_seed(5)
+    kc = torch.randn(B, H, W, D, generator=g).bfloat16()
+    vc = torch.randn(B, H, W, D, generator=g).bfloat16()
+    dkc, dvc = kc.cuda(), vc.cuda()
+    ws = torch.empty(max(ops.decode_workspace_bytes(B, H, D, W), 1), dtype=torch.uint8, device="cuda:0")
+    for s in range(steps):
+        t = t0 + s
+        q, kn, vn = (torch.randn(B, H, D, generator=g).bfloat16() for _ in range(3))
+        slot = t % W
+        kc[:, :, slot], vc[:, :, slot] = kn, vn
+        ref = _ref_decode(q, kc, vc)
+        o = ops.decode_attention(q.cuda(), kn.cuda(), vn.cuda(), dkc, dvc, n_rows=W, new_idx=slot,
+                                 write_back=True, workspace=ws)
+        assert_close_bf16(o, ref, f"o at step {s}")
+    assert torch.equal(dkc.cpu(), kc) and torch.equal(dvc.cpu(), vc)
+
+
+def test_decode_rejects_bad_arguments():
+    z = torch.zeros(1, 1, 128, dtype=torch.bfloat16, device="cuda:0")
+    rows = torch.zeros(1, 1, 4, 128, dtype=torch.bfloat16, device="cuda:0")
+    with pytest.raises(RuntimeError, match="new_idx"):
+        ops.decode_attention(z, z, z, rows, rows, n_rows=4, new_idx=4, write_back=False)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        y = torch.zeros(1, 1, 32, dtype=torch.bfloat16, device="cuda:0")
+        ops.decode_attention(y, y, y, None, None, n_rows=1, new_idx=0, write_back=False)

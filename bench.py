@@ -1,0 +1,283 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu]
+
+A "step" is one pass of the headline workload: windowed prefill attention with
+fused RoPE on B=8, T=4096, H=8, D=128, window 1024 (bf16), inputs resident in
+HBM.  One JSON line is printed.  `value` is the attention throughput of that
+workload in TFLOP/s (algorithmic flops = 4*D*B*H*visible pairs); the `roofline`
+object prices the dominant kernel against the 2.5 PFLOP/s dense bf16 MFMA peak;
+`cpu_baseline` times the CPU oracle on a bounded sample of the same workload;
+`extra` carries the other workloads (long-context prefill, KV-cache decode
+against the 8 TB/s HBM peak, KDA), each with its own roofline fraction.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBS = 8000.0
+SCALE = 0.12
+
+
+def prefill_flops(B, T, H, D, window):
+    if window is None or window <= 0 or window >= T:
+        pairs = T * (T + 1) // 2
+    else:
+        pairs = window * (window + 1) // 2 + (T - window) * window
+    return 4.0 * D * B * H * pairs
+
+
+def time_gpu(fn, steps, warmup):
+    """Mean milliseconds per call over `steps` calls, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def rope_table(D, T, base=10000.0, device="cuda:0"):
+    freq = (1.0 / base) ** torch.linspace(0, 1, steps=D // 2, dtype=torch.float32)
+    theta = torch.arange(T, dtype=torch.float32)[:, None] * freq[None, :]
+    return theta.cos().to(device), theta.sin().to(device)
+
+
+def rms(x):
+    return torch.nn.functional.rms_norm(x, (x.size(-1),))
+
+
+# ---------------------------------------------------------------------------------
+def bench_prefill_c2(steps, warmup, cpu_baseline=True):
+    """Config 2: B8 T4096 d1024 H8 D128 W1024, merged QKV, q/k/v RMS-normed, RoPE base 10000."""
+    from daisy_amd import ops
+    B, T, H, D, W, dim = 8, 4096, 8, 128, 1024, 1024
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(B, T, dim, generator=g).bfloat16()
+    w = (torch.randn(3 * dim, dim, generator=g) * 0.02).bfloat16()
+    dev = "cuda:0"
+    qkv = torch.nn.functional.linear(x.to(dev), w.to(dev)).view(B, T, 3 * H, D)
+    q, k, v = (rms(t) for t in qkv.chunk(3, dim=-2))
+    cos, sin = rope_table(D, T)
+    o = torch.empty(B, T, H, D, dtype=torch.bfloat16, device=dev)
+    k_rot = torch.empty(B, T, H, D, dtype=torch.bfloat16, device=dev)
+
+    def full():
+        ops.prefill_attention(q, k, v, window=W, scale=SCALE, cos=cos, sin=sin, out=o, k_out=k_rot)
+
+    ms_full = time_gpu(full, steps, warmup)
+
+    # The dominant kernel alone: same launch, keys already rotated (k_rot from above).
+    o2 = torch.empty_like(o)
+
+    def attn_only():
+        ops.prefill_attention(q, k_rot, v, window=W, scale=SCALE, out=o2)
+
+    ms_kernel = time_gpu(attn_only, steps, warmup)
+
+    def fused():
+        ops.prefill_attention(q, k, v, window=W, scale=SCALE, cos=cos, sin=sin, out=o2, k_out=k_rot, rotate_k_in_kernel=True)
+
+    ms_fused = time_gpu(fused, max(steps // 2, 1), max(warmup // 2, 1))
+
+    flops = prefill_flops(B, T, H, D, W)
+    res = {
+        "workload": "prefill_c2_B8_T4096_H8_D128_W1024_rope",
+        "ms_full": ms_full, "ms_kernel": ms_kernel, "ms_rotate_k_in_kernel": ms_fused,
+        "flops": flops,
+        "tflops_full": flops / ms_full / 1e9, "tflops_kernel": flops / ms_kernel / 1e9,
+        "frac_of_peak_kernel": flops / ms_kernel / 1e9 / PEAK_BF16_TFLOPS,
+    }
+    if cpu_baseline:
+        res["cpu_baseline"] = cpu_prefill_baseline(q[:1].cpu(), k[:1].cpu(), v[:1].cpu(), cos.cpu(), sin.cpu(), W,
+                                                   f"1 of {B} batch elements, all {H} heads, T={T}")
+    return res
+
+
+def cpu_prefill_baseline(q, k, v, cos, sin, W, sample):
+    """The reference's CPU path (RoPE + dense additive mask + SDPA) restated by the oracle's pieces."""
+    import oracle
+    torch.set_num_threads(os.cpu_count() or 1)
+    B, T, H, D = q.shape
+    mask = oracle.window_mask(T, W)
+    t0 = time.perf_counter()
+    qr, kr = oracle.apply_rope(q, cos[:T], sin[:T]), oracle.apply_rope(k, cos[:T], sin[:T])
+    torch.nn.functional.scaled_dot_product_attention(qr.transpose(1, 2), kr.transpose(1, 2), v.transpose(1, 2),
+                                                     attn_mask=mask, scale=SCALE)
+    dt = time.perf_counter() - t0
+    return {"value": prefill_flops(B, T, H, D, W) / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": sample, "seconds": dt}
+
+
+def bench_prefill_c3(steps, warmup):
+    """Config 3: B1 T65536 H16 D128, q/k/v ~ N(0,1) already rotated; window 2048 and full causal."""
+    from daisy_amd import ops
+    B, T, H, D = 1, 65536, 16, 128
+    g = torch.Generator(device="cuda:0").manual_seed(0)
+    q, k, v = (torch.randn(B, T, H, D, generator=g, device="cuda:0", dtype=torch.float32).bfloat16() for _ in range(3))
+    o = torch.empty_like(q)
+    out = {}
+    for name, W, n in (("window2048", 2048, steps), ("full_causal", None, max(steps // 4, 2))):
+        ms = time_gpu(lambda: ops.prefill_attention(q, k, v, window=W, scale=SCALE, out=o), n, max(warmup // 2, 1))
+        fl = prefill_flops(B, T, H, D, W)
+        out[name] = {"ms": ms, "flops": fl, "tflops": fl / ms / 1e9, "frac_of_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS}
+    return out
+
+
+def bench_decode_c4(steps=256, warmup=16, cpu_baseline=True):
+    """Config 4: batch 64, H16 D128, ring of 4096 slots holding positions up to 8192, 256 consecutive steps."""
+    from daisy_amd import ops
+    B, H, D, W, t0 = 64, 16, 128, 4096, 8192
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(0)
+    kc = torch.randn(B, H, W, D, generator=g, device=dev, dtype=torch.float32).bfloat16()
+    vc = torch.randn(B, H, W, D, generator=g, device=dev, dtype=torch.float32).bfloat16()
+    n = steps + warmup
+    qs = torch.randn(n, B, H, D, generator=g, device=dev, dtype=torch.float32).bfloat16()
+    ks = torch.randn(n, B, H, D, generator=g, device=dev, dtype=torch.float32).bfloat16()
+    vs = torch.randn(n, B, H, D, generator=g, device=dev, dtype=torch.float32).bfloat16()
+    o = torch.empty(B, H, D, dtype=torch.bfloat16, device=dev)
+    results = {}
+    for nsplit in (1, 2):
+        ws_bytes = ops.decode_workspace_bytes(B, H, D, W, nsplit)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+        step = [0]
+
+        def one():
+            i = step[0] % n
+            t = t0 + step[0]
+            ops.decode_attention(qs[i], ks[i], vs[i], kc, vc, n_rows=W, new_idx=t % W, write_back=True,
+                                 scale=SCALE, out=o, workspace=ws, nsplit=nsplit)
+            step[0] += 1
+
+        ms = time_gpu(one, steps, warmup)
+        nbytes = B * H * W * D * 2 * 2
+        results[f"nsplit{nsplit}"] = {"ms_per_step": ms, "bytes": nbytes, "gbs": nbytes / ms / 1e6,
+                                      "frac_of_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    best = max(results.values(), key=lambda r: r["gbs"])
+    out = {"workload": "decode_c4_B64_H16_D128_W4096_256steps", "variants": results, **best}
+    if cpu_baseline:
+        out["cpu_baseline"] = cpu_decode_baseline(kc[:4].cpu(), vc[:4].cpu(), qs[0, :4].cpu(), ks[0, :4].cpu(), vs[0, :4].cpu(), W,
+                                                  f"4 of {B} batch elements, all {H} heads, 4 steps")
+    return out
+
+
+def cpu_decode_baseline(kc, vc, q, kn, vn, W, sample):
+    """The reference's step path: chronological cat of the last W-1 rows + new row, non-causal SDPA."""
+    torch.set_num_threads(os.cpu_count() or 1)
+    B, H, _, D = kc.shape
+    k_ctx, v_ctx = kc.transpose(1, 2), vc.transpose(1, 2)   # [B, n, H, D] views, n = W
+    reps = 4
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        k_ = torch.cat([k_ctx[:, 1:], kn[:, None]], 1).transpose(1, 2)
+        v_ = torch.cat([v_ctx[:, 1:], vn[:, None]], 1).transpose(1, 2)
+        torch.nn.functional.scaled_dot_product_attention(q[:, :, None], k_, v_, scale=SCALE, is_causal=False)
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": B * H * W * D * 4 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": sample, "seconds_per_step": dt}
+
+
+def bench_kda_c5(steps, warmup, cpu_baseline=True):
+    """Config 5: B4 T8192 H16 Dk=Dv=128, chunk 64."""
+    from daisy_amd import ops
+    B, T, H, Dk, Dv = 4, 8192, 16, 128, 128
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev, dtype=torch.float32)
+    q = torch.nn.functional.normalize(rn(B, T, H, Dk), dim=-1).bfloat16()
+    k = torch.nn.functional.normalize(rn(B, T, H, Dk), dim=-1).bfloat16()
+    v = rn(B, T, H, Dv).bfloat16()
+    gl = torch.nn.functional.logsigmoid(rn(B, T, H, Dk))
+    beta = torch.sigmoid(rn(B, T, H))
+    ws = torch.empty(max(ops.kda_workspace_bytes(B, T, H, Dk, Dv), 1), dtype=torch.uint8, device=dev)
+    ms = time_gpu(lambda: ops.kda_chunk_fwd(q, k, v, gl, beta, output_final_state=True, workspace=ws), steps, warmup)
+    min_bytes = 5 * B * T * H * Dk * 2
+    flops = 7.0 * Dk * Dv * B * T * H
+    out = {"workload": "kda_c5_B4_T8192_H16_D128_chunk64", "ms": ms, "min_bytes": min_bytes,
+           "gbs_min_io": min_bytes / ms / 1e6, "frac_of_hbm_peak": min_bytes / ms / 1e6 / PEAK_HBM_GBS,
+           "naive_flops": flops, "tflops_naive": flops / ms / 1e9}
+    if cpu_baseline:
+        import oracle
+        torch.set_num_threads(os.cpu_count() or 1)
+        Ts = 512
+        t0 = time.perf_counter()
+        oracle.kda_recurrent(q[:1, :Ts, :2].cpu(), k[:1, :Ts, :2].cpu(), v[:1, :Ts, :2].cpu(), gl[:1, :Ts, :2].cpu(), beta[:1, :Ts, :2].cpu())
+        dt = time.perf_counter() - t0
+        tok_heads = Ts * 2
+        out["cpu_baseline"] = {"value": tok_heads / dt, "unit": "token-heads/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"B=1, H=2 of 16, T={Ts} of {T} (naive recurrence)", "seconds": dt,
+                               "gpu_token_heads_per_s": B * T * H / (ms / 1e3)}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--only", default=None, help="prefill | long | decode | kda (default: all)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: every kernel here works on one GPU's share of the (batch, head) "
+                 "range and nothing is exchanged between GPUs; run with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an AMD GPU")
+    from daisy_amd import _lib
+    _lib.load()
+
+    want = lambda name: args.only in (None, name)
+    cpu = not args.no_cpu
+    extra = {}
+    head = bench_prefill_c2(args.steps, args.warmup, cpu) if want("prefill") else None
+    if want("long"):
+        extra["prefill_c3_B1_T65536_H16_D128"] = bench_prefill_c3(max(args.steps // 5, 4), max(args.warmup // 2, 2))
+    if want("decode"):
+        extra["decode_c4"] = bench_decode_c4(256, 16, cpu)
+    if want("kda"):
+        try:
+            extra["kda_c5"] = bench_kda_c5(max(args.steps // 5, 4), max(args.warmup // 2, 2), cpu)
+        except RuntimeError as e:
+            extra["kda_c5"] = {"error": str(e)}
+
+    line = {
+        "metric": "prefill attn TFLOP/s + decode KV GB/s (fraction of MI355X roofline)",
+        "value": None if head is None else head["tflops_full"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": None if head is None else head["ms_full"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "windowed prefill attention, fused RoPE: B=8 T=4096 H=8 D=128 window=1024 (BASELINE configs[1])",
+                   "timed": "K rotation pre-pass + attention kernel, inputs and outputs in HBM"},
+    }
+    if head is not None:
+        line["roofline"] = {"bound": "mfma", "achieved": head["tflops_kernel"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                            "frac": head["frac_of_peak_kernel"], "traffic": None,
+                            "kernel": "prefill_mfma_kernel<128,false>", "ms": head["ms_kernel"]}
+        if "cpu_baseline" in head:
+            line["cpu_baseline"] = head.pop("cpu_baseline")
+        extra["prefill_c2"] = head
+    line["extra"] = extra
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

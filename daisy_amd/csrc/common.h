@@ -58,10 +58,16 @@ __device__ __forceinline__ u32x4 pack8(const float* f) {
 // elementwise tensor library evaluates the expression, so that the bf16 result
 // is bit-identical to it.
 __device__ __forceinline__ float rope_lo(float x1, float x2, float c, float s) {
-  return __fadd_rn(__fmul_rn(x1, c), __fmul_rn(x2, s));
+#pragma clang fp contract(off)
+  const float a = x1 * c;
+  const float b = x2 * s;
+  return a + b;
 }
 __device__ __forceinline__ float rope_hi(float x1, float x2, float c, float s) {
-  return __fadd_rn(__fmul_rn(x1, -s), __fmul_rn(x2, c));
+#pragma clang fp contract(off)
+  const float a = x1 * -s;
+  const float b = x2 * c;
+  return a + b;
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

@@ -72,6 +72,24 @@ __device__ __forceinline__ float rope_hi(float x1, float x2, float c, float s) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// ---- cross-lane sums with DPP (no LDS traffic) -------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+  int y = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false);
+  return x + __int_as_float(y);
+}
+
+// Sum over the LPR consecutive lanes that share a cache row; every lane of the
+// group ends with the total.
+template <int LPR>
+__device__ __forceinline__ float group_sum(float x) {
+  x = dpp_add<0xB1>(x);                     // quad_perm [1,0,3,2]   (xor 1)
+  x = dpp_add<0x4E>(x);                     // quad_perm [2,3,0,1]   (xor 2)
+  if (LPR >= 8) x = dpp_add<0x141>(x);      // row_half_mirror       (joins the two quads of 8 lanes)
+  if (LPR >= 16) x = dpp_add<0x128>(x);     // row_ror 8             (joins the two halves of 16 lanes)
+  return x;
+}
+
 // ---- host-side error plumbing --------------------------------------------
 void set_error(const char* fmt, ...);
 

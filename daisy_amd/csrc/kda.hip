@@ -20,6 +20,458 @@ __global__ __launch_bounds__(256) void kda_gate_kernel(const void* g, const floa
   else ((float*)out)[i] = y;
 }
 
+
+// ===========================================================================
+// Chunked forward.  Per (batch, head), chunk of C = 64 positions, Dk = Dv = 128.
+//
+// With G_i the inclusive running sum of the log-decay g inside the chunk (per
+// channel), S0 the state at the chunk start, and (per channel products written
+// with (.)):
+//   A_ij = beta_i sum_d k_id k_jd exp(G_id - G_jd)     (j <  i)
+//   P_ij =        sum_d q_id k_jd exp(G_id - G_jd)     (j <= i)
+//   (I + A) [W | U0] = diag(beta) [exp(G) (.) K | V]
+//   U  = U0 - W S0
+//   O  = scale ((exp(G) (.) Q) S0 + P U)
+//   S' = diag(exp(G_last)) S0 + (exp(G_last - G) (.) K)^T U
+//
+// kda_prep_kernel (one workgroup per chunk, all chunks in parallel) produces
+// everything that does not depend on S0 into the workspace:
+//   Wn  = -W                        bf16 [64][128]   contraction index (channel) permuted
+//   Qg  = scale exp(G) (.) Q        bf16 [64][128]   channel permuted
+//   Pm  = scale tril(P)             bf16 [64][64]    column (position) permuted
+//   KtH + KtL = (exp(G_last - G) (.) K)^T split into two bf16 terms, [128][64], position permuted
+//   U0T = U0^T                      fp32 [128][64]
+//   dec = exp(G_last)               fp32 [128]
+// kda_state_kernel (one wavefront per (batch, head, 16 value columns)) then
+// walks the chunks in order with the fp32 state in registers; every product in
+// it is a v_mfma_f32_16x16x32_bf16 whose B operand is an accumulator (S0 or U)
+// converted to bf16 in place: in the 16x16 accumulator layout lane l holds
+// column l%16 and rows 4*(l/16)+r of each tile, so two stacked tiles give the
+// lane 8 contraction indices 16*t + 4*(l/16) + r (t = 0,1; r = 0..3).  The A
+// operands are stored with their contraction index permuted inside every
+// aligned group of 32 (perm32) so that those 8 indices are 8 consecutive
+// elements, one 16-byte load.
+//
+// Numerics: off-diagonal 16x16 blocks of A and P run on MFMA with both operands
+// referenced to the row before the block (every exponent <= 0); diagonal blocks
+// are accumulated in fp32 from running products of exp(g) (no exponent is ever
+// positive, so strong decays cannot overflow).  The triangular solve is fp32.
+// The state update uses a two-term bf16 split of both operands (three MFMAs),
+// which keeps the state error near fp32.
+// ===========================================================================
+constexpr int KC = 64;    // chunk length
+constexpr int KD = 128;   // Dk = Dv
+constexpr int KVS = 16;   // value columns per state wavefront
+constexpr size_t kChunkBytes = (size_t)KC * KD * 2 * 2 + KC * KC * 2 + (size_t)KD * KC * 2 * 2 + (size_t)KD * KC * 4 + KD * 4;
+
+struct KdaParams {
+  const uint16_t* q; const uint16_t* k; const uint16_t* v;
+  const void* g; int g_bf16; const float* beta;
+  const float* s0; uint16_t* o; float* s_out;
+  int B, T, H, NC; float scale; int l2norm; float l2eps;
+  uint16_t* Wn; uint16_t* Qg; uint16_t* Pm; uint16_t* KtH; uint16_t* KtL; float* U0T; float* dec;
+};
+
+// Stored position of contraction index x inside its aligned group of 32: bits (4,3,2) -> (3,2,4).
+__host__ __device__ constexpr int perm32(int x) { return (x & ~0x1c) | ((x & 0x0c) << 1) | ((x & 0x10) >> 2); }
+__host__ __device__ constexpr int perm32_inv(int p) { return (p & ~0x1c) | ((p & 0x18) >> 1) | ((p & 0x04) << 2); }
+
+__device__ __forceinline__ f32x4 lds_f4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+
+__global__ __launch_bounds__(256) void kda_prep_kernel(KdaParams p) {
+  __shared__ __attribute__((aligned(16))) float G[KC][KD];           // inclusive running log-decay
+  __shared__ __attribute__((aligned(16))) float EG[KC][KD];          // exp(g) per row; later staging for Wn
+  __shared__ __attribute__((aligned(16))) uint16_t Kr[KC][KD + 8];   // k as given (bf16)
+  __shared__ __attribute__((aligned(16))) uint16_t Qr[KC][KD + 8];   // q as given
+  __shared__ __attribute__((aligned(16))) float AT[KC][KC];          // AT[j][i] = A_ij (j < i)
+  __shared__ float rk[KC], rq[KC], bt[KC];                           // 1/|k|, 1/|q|, beta (0 for padded rows)
+
+  const int n = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int t0 = n * KC;
+  const int64_t ci = ((int64_t)b * p.H + h) * p.NC + n;
+  auto row_off = [&](int r) -> int64_t { return (((int64_t)b * p.T + t0 + r) * p.H + h) * KD; };
+
+  // ---- phase 0a: G = cumsum(g), EG = exp(g) ---------------------------------
+  {
+    const int d = tid & 127, half = tid >> 7;
+    float gv[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      const int r = 32 * half + i;
+      float x = 0.f;
+      if (t0 + r < p.T) {
+        x = p.g_bf16 ? bf16lo_to_f32(((const uint16_t*)p.g)[row_off(r) + d]) : ((const float*)p.g)[row_off(r) + d];
+      }
+      gv[i] = x;
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      acc += gv[i];
+      G[32 * half + i][d] = acc;
+      EG[32 * half + i][d] = __expf(gv[i]);
+    }
+    __syncthreads();
+    if (half == 1) {
+      const float add = G[31][d];
+#pragma unroll
+      for (int i = 0; i < 32; ++i) G[32 + i][d] += add;
+    }
+  }
+
+  // ---- phase 0b: raw q, k to LDS, row norms, beta ---------------------------
+  const int cc = tid & 15, r4 = tid >> 4;
+  u32x4 qraw[4];
+  float rqv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r4 + 16 * i;
+    u32x4 kraw = {0, 0, 0, 0};
+    qraw[i] = kraw;
+    if (t0 + r < p.T) {
+      kraw = *reinterpret_cast<const u32x4*>(p.k + row_off(r) + 8 * cc);
+      qraw[i] = *reinterpret_cast<const u32x4*>(p.q + row_off(r) + 8 * cc);
+    }
+    float kf[8], qf[8];
+    unpack8(kraw, kf);
+    unpack8(qraw[i], qf);
+    float sk = 0.f, sq = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { sk = fmaf(kf[e], kf[e], sk); sq = fmaf(qf[e], qf[e], sq); }
+    sk = group_sum<16>(sk);
+    sq = group_sum<16>(sq);
+    const float nk = p.l2norm ? rsqrtf(sk + p.l2eps) : 1.f;
+    rqv[i] = p.l2norm ? rsqrtf(sq + p.l2eps) : 1.f;
+    if (cc == 0) {
+      rk[r] = nk;
+      rq[r] = rqv[i];
+      bt[r] = (t0 + r < p.T) ? p.beta[((int64_t)b * p.T + t0 + r) * p.H + h] : 0.f;
+    }
+    *reinterpret_cast<u32x4*>(&Kr[r][8 * cc]) = kraw;
+    *reinterpret_cast<u32x4*>(&Qr[r][8 * cc]) = qraw[i];
+  }
+  __syncthreads();
+
+  // ---- phase 1: Qg = scale exp(G) q/|q| (channel permuted), dec = exp(G_last) ----
+  {
+    const int pos0 = ((cc >> 2) << 5) | ((cc & 1) << 4) | (((cc >> 1) & 1) << 2);  // perm32(8*cc)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = r4 + 16 * i;
+      float qf[8], o8[8];
+      unpack8(qraw[i], qf);
+      const f32x4 g0 = lds_f4(&G[r][8 * cc]), g1 = lds_f4(&G[r][8 * cc + 4]);
+      const float sc = p.scale * rqv[i];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        o8[e] = sc * __expf(g0[e]) * qf[e];
+        o8[4 + e] = sc * __expf(g1[e]) * qf[4 + e];
+      }
+      const u32x4 pk = pack8(o8);
+      uint16_t* dst = p.Qg + (ci * KC + r) * KD + pos0;
+      u32x2 lo2 = {pk.x, pk.y}, hi2 = {pk.z, pk.w};
+      *reinterpret_cast<u32x2*>(dst) = lo2;        // channels 8cc+0..3
+      *reinterpret_cast<u32x2*>(dst + 8) = hi2;    // channels 8cc+4..7
+    }
+    if (r4 == 0) {
+      const f32x4 g0 = lds_f4(&G[KC - 1][8 * cc]), g1 = lds_f4(&G[KC - 1][8 * cc + 4]);
+      f32x4 d0, d1;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { d0[e] = __expf(g0[e]); d1[e] = __expf(g1[e]); }
+      float* dd = p.dec + ci * KD + 8 * cc;
+      *reinterpret_cast<f32x4*>(dd) = d0;
+      *reinterpret_cast<f32x4*>(dd + 4) = d1;
+    }
+  }
+
+  // ---- phase 2a: off-diagonal 16x16 blocks of A and P on MFMA ----------------
+  {
+    const int li = lane & 15, q4 = lane >> 4;
+    for (int bi = wave; bi < 6; bi += 4) {
+      // blocks (I, J), I > J, in the order (1,0) (2,0) (2,1) (3,0) (3,1) (3,2)
+      const int I = (bi == 0) ? 1 : (bi < 3 ? 2 : 3);
+      const int J = (bi == 0) ? 0 : (bi < 3 ? bi - 1 : bi - 3);
+      const int ref = 16 * I - 1;
+      const int ri = 16 * I + li, rj = 16 * J + li;
+      f32x4 accA = {0.f, 0.f, 0.f, 0.f}, accP = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int d0 = 32 * m + 8 * q4;
+        float ki[8], qi[8], kj[8], ak[8], aq[8], bk[8];
+        unpack8(*reinterpret_cast<const u32x4*>(&Kr[ri][d0]), ki);
+        unpack8(*reinterpret_cast<const u32x4*>(&Qr[ri][d0]), qi);
+        unpack8(*reinterpret_cast<const u32x4*>(&Kr[rj][d0]), kj);
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          const f32x4 gi = lds_f4(&G[ri][d0 + 4 * hf]), gr = lds_f4(&G[ref][d0 + 4 * hf]), gj = lds_f4(&G[rj][d0 + 4 * hf]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float fi = __expf(gi[e] - gr[e]);   // <= 1: row ri is at or after the reference row
+            const float fj = __expf(gr[e] - gj[e]);   // <= 1: row rj is before the reference row
+            ak[4 * hf + e] = ki[4 * hf + e] * fi;
+            aq[4 * hf + e] = qi[4 * hf + e] * fi;
+            bk[4 * hf + e] = kj[4 * hf + e] * fj;
+          }
+        }
+        const bf16x8 va = __builtin_bit_cast(bf16x8, pack8(ak));
+        const bf16x8 vq = __builtin_bit_cast(bf16x8, pack8(aq));
+        const bf16x8 vb = __builtin_bit_cast(bf16x8, pack8(bk));
+        accA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, vb, accA, 0, 0, 0);
+        accP = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vq, vb, accP, 0, 0, 0);
+      }
+      // accumulator: lane holds column j = 16J + li, rows i = 16I + 4*q4 + r
+      const int j = 16 * J + li;
+      const float rkj = rk[j];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * I + 4 * q4 + r;
+        AT[j][i] = bt[i] * rk[i] * rkj * accA[r];
+        const float pv = p.scale * rq[i] * rkj * accP[r];
+        p.Pm[(ci * KC + i) * KC + perm32(j)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
+      }
+    }
+    // The state kernel reads P in 16x32 pieces; blocks (0,1) and (2,3) lie above the diagonal.
+    if (wave >= 2) {
+      const int I = (wave == 2) ? 0 : 2, J = I + 1;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) p.Pm[(ci * KC + 16 * I + 4 * q4 + r) * KC + perm32(16 * J + li)] = 0;
+    }
+  }
+
+  // ---- phase 2b: diagonal 16x16 blocks, fp32, running products of exp(g) ------
+  {
+    const int I = wave, il = lane >> 2, dq = lane & 3;
+    const int ri = 16 * I + il;
+    float a[16], pp[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) { a[j] = 0.f; pp[j] = 0.f; }
+#pragma unroll 1
+    for (int dc = 0; dc < 4; ++dc) {
+      const int d0 = 32 * dq + 8 * dc;
+      float ki[8], qi[8], E[8];
+      unpack8(*reinterpret_cast<const u32x4*>(&Kr[ri][d0]), ki);
+      unpack8(*reinterpret_cast<const u32x4*>(&Qr[ri][d0]), qi);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) E[e] = 1.f;
+#pragma unroll
+      for (int j = 15; j >= 0; --j) {
+        const int rj = 16 * I + j;
+        float kj[8];
+        unpack8(*reinterpret_cast<const u32x4*>(&Kr[rj][d0]), kj);
+        if (j < 15) {
+          // E = exp(G_i - G_j) for j < i: multiply in exp(g) of row j+1; rows j >= i restart at 1.
+          const f32x4 e0 = lds_f4(&EG[rj + 1][d0]), e1 = lds_f4(&EG[rj + 1][d0 + 4]);
+          const bool live = j < il;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            E[e] = live ? E[e] * e0[e] : 1.f;
+            E[4 + e] = live ? E[4 + e] * e1[e] : 1.f;
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float t = kj[e] * E[e];
+          a[j] = fmaf(ki[e], t, a[j]);
+          pp[j] = fmaf(qi[e], t, pp[j]);
+        }
+      }
+    }
+    const float bi = bt[ri] * rk[ri], qs = p.scale * rq[ri];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      float av = dpp_add<0x4E>(dpp_add<0xB1>(a[j]));    // sum over the 4 channel quarters
+      float pv = dpp_add<0x4E>(dpp_add<0xB1>(pp[j]));
+      if ((j & 3) == dq) {
+        const int rj = 16 * I + j;
+        const float rkj = rk[rj];
+        if (j < il) AT[rj][ri] = bi * rkj * av;
+        pv = (j <= il) ? qs * rkj * pv : 0.f;
+        p.Pm[(ci * KC + ri) * KC + perm32(rj)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 3: forward substitution (I + A) X = diag(beta) [exp(G) K | V] ----
+  // One thread per right-hand-side column; the column lives in registers.
+  {
+    float X[KC];
+    const int c = tid;
+    if (c < KD) {
+#pragma unroll
+      for (int i = 0; i < KC; ++i) X[i] = bt[i] * rk[i] * __expf(G[i][c]) * bf16lo_to_f32(Kr[i][c]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < KC; ++i) {
+        float vv = 0.f;
+        if (t0 + i < p.T) vv = bf16lo_to_f32(p.v[row_off(i) + (c - KD)]);
+        X[i] = bt[i] * vv;
+      }
+    }
+    // Right-looking elimination: once X[j] is final, remove it from every later row.
+#pragma unroll
+    for (int j = 0; j < KC - 1; ++j) {
+      const float xj = X[j];
+#pragma unroll
+      for (int i4 = (j + 1) / 4; i4 < KC / 4; ++i4) {
+        const f32x4 av = lds_f4(&AT[j][4 * i4]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = 4 * i4 + e;
+          if (i > j) X[i] = fmaf(-av[e], xj, X[i]);
+        }
+      }
+    }
+    uint16_t* Wst = reinterpret_cast<uint16_t*>(&EG[0][0]);   // [64][128] bf16 staging (EG is dead)
+    if (c < KD) {
+      const int pc = perm32(c);
+#pragma unroll
+      for (int i = 0; i < KC; ++i) Wst[i * KD + pc] = (uint16_t)(pack_bf16x2(-X[i], 0.f) & 0xffffu);
+    } else {
+      float* dst = p.U0T + (ci * KD + (c - KD)) * KC;
+#pragma unroll
+      for (int i4 = 0; i4 < KC / 4; ++i4) {
+        f32x4 w = {X[4 * i4], X[4 * i4 + 1], X[4 * i4 + 2], X[4 * i4 + 3]};
+        *reinterpret_cast<f32x4*>(dst + 4 * i4) = w;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ch = tid + 256 * i;   // 16-byte chunk of the [64][128] bf16 tile
+      *reinterpret_cast<u32x4*>(p.Wn + ci * KC * KD + 8 * ch) = *reinterpret_cast<const u32x4*>(Wst + 8 * ch);
+    }
+  }
+
+  // ---- phase 4: (exp(G_last - G) k/|k|)^T as two bf16 terms, position permuted ----
+  {
+    const int d = tid & 127, gh = tid >> 7;
+    const float glast = G[KC - 1][d];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int g8 = 4 * gh + i;   // group of 8 stored positions
+      float hi[8], lo[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int pos = perm32_inv(8 * g8 + e);
+        const float val = __expf(glast - G[pos][d]) * bf16lo_to_f32(Kr[pos][d]) * rk[pos];
+        hi[e] = round_bf16(val);
+        lo[e] = val - hi[e];
+      }
+      *reinterpret_cast<u32x4*>(p.KtH + (ci * KD + d) * KC + 8 * g8) = pack8(hi);
+      *reinterpret_cast<u32x4*>(p.KtL + (ci * KD + d) * KC + 8 * g8) = pack8(lo);
+    }
+  }
+}
+
+__device__ __forceinline__ bf16x8 pack_acc2(const f32x4& t0, const f32x4& t1) {
+  u32x4 r;
+  r.x = pack_bf16x2(t0[0], t0[1]); r.y = pack_bf16x2(t0[2], t0[3]);
+  r.z = pack_bf16x2(t1[0], t1[1]); r.w = pack_bf16x2(t1[2], t1[3]);
+  return __builtin_bit_cast(bf16x8, r);
+}
+__device__ __forceinline__ bf16x8 ldg_bf16x8(const uint16_t* p) {
+  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(p));
+}
+
+__global__ __launch_bounds__(64) void kda_state_kernel(KdaParams p) {
+  // Keep the 8 column slices of one (batch, head) on one XCD: they read the same chunk data.
+  int vid = blockIdx.x;
+  if ((gridDim.x & 7) == 0) vid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  constexpr int NSL = KD / KVS;
+  const int slice = vid % NSL, bh = vid / NSL;
+  const int h = bh % p.H, b = bh / p.H;
+  const int lane = threadIdx.x, ln = lane & 15, q4 = lane >> 4;
+  const int vcol = KVS * slice + ln;
+
+  // State tile dt: rows (key channels) 16*dt + 4*q4 + r, column vcol.
+  f32x4 S[8];
+#pragma unroll
+  for (int dt = 0; dt < 8; ++dt) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      S[dt][r] = p.s0 ? p.s0[((int64_t)bh * KD + 16 * dt + 4 * q4 + r) * KD + vcol] : 0.f;
+  }
+
+  for (int n = 0; n < p.NC; ++n) {
+    const int64_t ci = (int64_t)bh * p.NC + n;
+    const uint16_t* Wn = p.Wn + ci * KC * KD;
+    const uint16_t* Qg = p.Qg + ci * KC * KD;
+    const uint16_t* Pm = p.Pm + ci * KC * KC;
+    const uint16_t* KtH = p.KtH + ci * KD * KC;
+    const uint16_t* KtL = p.KtL + ci * KD * KC;
+
+    bf16x8 Sb[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) Sb[m] = pack_acc2(S[2 * m], S[2 * m + 1]);
+
+    // U = U0 + (-W) S0; tile mt: rows (positions) 16*mt + 4*q4 + r, column vcol.
+    f32x4 U[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      U[mt] = *reinterpret_cast<const f32x4*>(p.U0T + (ci * KD + vcol) * KC + 16 * mt + 4 * q4);
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+        U[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ldg_bf16x8(Wn + (16 * mt + ln) * KD + 32 * m + 8 * q4), Sb[m], U[mt], 0, 0, 0);
+    }
+    bf16x8 Uh[2], Ul[2];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      Uh[m] = pack_acc2(U[2 * m], U[2 * m + 1]);
+      f32x4 l0, l1;
+      const u32x4 hb = __builtin_bit_cast(u32x4, Uh[m]);
+      l0[0] = U[2 * m][0] - bf16lo_to_f32(hb.x); l0[1] = U[2 * m][1] - bf16hi_to_f32(hb.x);
+      l0[2] = U[2 * m][2] - bf16lo_to_f32(hb.y); l0[3] = U[2 * m][3] - bf16hi_to_f32(hb.y);
+      l1[0] = U[2 * m + 1][0] - bf16lo_to_f32(hb.z); l1[1] = U[2 * m + 1][1] - bf16hi_to_f32(hb.z);
+      l1[2] = U[2 * m + 1][2] - bf16lo_to_f32(hb.w); l1[3] = U[2 * m + 1][3] - bf16hi_to_f32(hb.w);
+      Ul[m] = pack_acc2(l0, l1);
+    }
+
+    // O = Qg S0 + Pm U  (scale already folded into Qg and Pm)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      f32x4 O = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+        O = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ldg_bf16x8(Qg + (16 * mt + ln) * KD + 32 * m + 8 * q4), Sb[m], O, 0, 0, 0);
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+        if (32 * m <= 16 * mt + 15)   // columns up to the diagonal only
+          O = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ldg_bf16x8(Pm + (16 * mt + ln) * KC + 32 * m + 8 * q4), Uh[m], O, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = n * KC + 16 * mt + 4 * q4 + r;
+        if (t < p.T) p.o[(((int64_t)b * p.T + t) * p.H + h) * KD + vcol] = (uint16_t)(pack_bf16x2(O[r], 0.f) & 0xffffu);
+      }
+    }
+
+    // S = exp(G_last) (.) S + Kt^T U, with both operands split into two bf16 terms.
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) {
+      const f32x4 dc = *reinterpret_cast<const f32x4*>(p.dec + ci * KD + 16 * dt + 4 * q4);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) S[dt][r] *= dc[r];
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+        const bf16x8 ah = ldg_bf16x8(KtH + (16 * dt + ln) * KC + 32 * m + 8 * q4);
+        const bf16x8 al = ldg_bf16x8(KtL + (16 * dt + ln) * KC + 32 * m + 8 * q4);
+        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, Uh[m], S[dt], 0, 0, 0);
+        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, Ul[m], S[dt], 0, 0, 0);
+        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, Uh[m], S[dt], 0, 0, 0);
+      }
+    }
+  }
+
+  if (p.s_out != nullptr) {
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) p.s_out[((int64_t)bh * KD + 16 * dt + 4 * q4 + r) * KD + vcol] = S[dt][r];
+  }
+}
+
 }  // namespace daisy
 
 using namespace daisy;
@@ -43,9 +495,11 @@ extern "C" int daisy_kda_gate_fwd(const void* g, const float* A_log, const float
   return DAISY_OK;
 }
 
+
 extern "C" size_t daisy_kda_workspace_bytes(int B, int T, int H, int Dk, int Dv, int chunk) {
-  (void)B; (void)T; (void)H; (void)Dk; (void)Dv; (void)chunk;
-  return 0;
+  if (B <= 0 || T <= 0 || H <= 0 || Dk != KD || Dv != KD || chunk != KC) return 0;
+  const size_t nc = (size_t)(T + KC - 1) / KC;
+  return (size_t)B * H * nc * kChunkBytes;
 }
 
 extern "C" int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
@@ -54,6 +508,38 @@ extern "C" int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
                                    int B, int T, int H, int Dk, int Dv, int chunk,
                                    float scale, int l2norm_qk, float l2_eps,
                                    void* workspace, size_t workspace_bytes, void* stream) {
-  set_error("kda_chunk_fwd: not built yet");
-  return DAISY_ERR_UNSUPPORTED;
+  DAISY_CHECK_SUPPORTED(Dk == KD && Dv == KD, "kda: Dk=%d, Dv=%d not supported (both must be %d)", Dk, Dv, KD);
+  DAISY_CHECK_SUPPORTED(chunk == KC, "kda: chunk=%d not supported (must be %d)", chunk, KC);
+  DAISY_CHECK_ARG(q && k && v && g && beta && o, "kda: q, k, v, g, beta and o must be non-NULL");
+  DAISY_CHECK_ARG(B > 0 && T > 0 && H > 0, "kda: B=%d, T=%d, H=%d must be positive", B, T, H);
+  DAISY_CHECK_ARG(B <= 65535 && H <= 65535, "kda: B and H must each be <= 65535");
+  auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+  DAISY_CHECK_ARG(al16(q) && al16(k) && al16(v) && al16(g) && al16(o) && al16(workspace),
+                  "kda: tensors and workspace must be 16-byte aligned");
+  const size_t need = daisy_kda_workspace_bytes(B, T, H, Dk, Dv, chunk);
+  if (!workspace || workspace_bytes < need) {
+    set_error("kda: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    return DAISY_ERR_WORKSPACE;
+  }
+  KdaParams p;
+  p.q = (const uint16_t*)q; p.k = (const uint16_t*)k; p.v = (const uint16_t*)v;
+  p.g = g; p.g_bf16 = g_is_bf16; p.beta = beta;
+  p.s0 = initial_state; p.o = (uint16_t*)o; p.s_out = final_state;
+  p.B = B; p.T = T; p.H = H; p.NC = (T + KC - 1) / KC;
+  p.scale = scale; p.l2norm = l2norm_qk; p.l2eps = l2_eps;
+  const size_t chunks = (size_t)B * H * p.NC;
+  char* w = (char*)workspace;
+  p.Wn = (uint16_t*)w;  w += chunks * KC * KD * 2;
+  p.Qg = (uint16_t*)w;  w += chunks * KC * KD * 2;
+  p.KtH = (uint16_t*)w; w += chunks * KD * KC * 2;
+  p.KtL = (uint16_t*)w; w += chunks * KD * KC * 2;
+  p.U0T = (float*)w;    w += chunks * KD * KC * 4;
+  p.Pm = (uint16_t*)w;  w += chunks * KC * KC * 2;
+  p.dec = (float*)w;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(kda_prep_kernel, dim3(p.NC, H, B), dim3(256), 0, s, p);
+  DAISY_CHECK_LAUNCH("kda_prep_kernel");
+  hipLaunchKernelGGL(kda_state_kernel, dim3((unsigned)(B * H * (KD / KVS))), dim3(64), 0, s, p);
+  DAISY_CHECK_LAUNCH("kda_state_kernel");
+  return DAISY_OK;
 }

@@ -1,0 +1,138 @@
+"""Generator plumbing with a one-hot fake model: the scenarios of the
+reference's tests/test_generator.py:128-189,251-277 (prefill fills the cache in
+order, step passes pre-write contexts and appends, greedy generation)."""
+import pytest
+import torch
+import torch.nn as nn
+
+from daisy_amd import Generator
+
+
+class FakeAttn:
+    def __init__(self, num_heads, head_dim):
+        self.num_heads, self.head_dim = num_heads, head_dim
+
+
+class FakeBlock(nn.Module):
+    def __init__(self, attn):
+        super().__init__()
+        self.attn = attn
+
+
+class OneHotModel(nn.Module):
+    """embed = identity, logits = embedding of the current token, K = V = embedding."""
+
+    def __init__(self, vocab, layers=2):
+        super().__init__()
+        self.eos_token_id = 50256
+        self.embed = nn.Embedding(vocab, vocab)
+        with torch.no_grad():
+            self.embed.weight.copy_(torch.eye(vocab))
+        self.blocks = nn.ModuleList([FakeBlock(FakeAttn(1, vocab)) for _ in range(layers)])
+        self.seen_k = self.seen_v = None
+
+    def reset_history(self):
+        self.seen_k = self.seen_v = None
+
+    @torch.no_grad()
+    def prefill(self, ids):
+        B, T = ids.shape
+        e = self.embed(ids)
+        k = e.view(B, T, 1, -1).transpose(1, 2)
+        K = torch.stack([k for _ in self.blocks])
+        return e[:, -1], torch.stack([K, K.clone()])
+
+    @torch.no_grad()
+    def step(self, token_id, k_ctxs, v_ctxs, pos):
+        self.seen_k = [k.clone() for k in k_ctxs]
+        self.seen_v = [v.clone() for v in v_ctxs]
+        e = self.embed(token_id)
+        kv = e.view(1, 1, 1, -1)
+        return e.view(1, -1), [kv for _ in self.blocks], [kv.clone() for _ in self.blocks]
+
+
+V = 16
+
+
+@pytest.fixture()
+def env():
+    torch.manual_seed(0)
+    model = OneHotModel(V).eval()
+    gen = Generator(model, window=8, seed=1337, device=torch.device("cpu"), dtype=torch.bfloat16, temperature=0.0)
+    return model, gen
+
+
+def onehot(i):
+    v = torch.zeros(V)
+    v[i] = 1.0
+    return v
+
+
+def test_prefill_updates_cache_and_returns_logits(env):
+    model, gen = env
+    prompt = torch.tensor([3, 5, 7, 9])
+    logits = gen._prefill(prompt)
+    assert logits.shape == (1, V) and torch.equal(logits[0].float(), onehot(9))
+    assert gen.cache.t == 4
+    for layer in range(2):
+        k, v = gen.cache.view(layer)
+        assert k.shape == (1, 4, 1, V)
+        for t, tok in enumerate(prompt.tolist()):
+            assert torch.equal(k[0, t, 0].float(), onehot(tok)) and torch.equal(v[0, t, 0].float(), onehot(tok))
+    assert torch.equal(gen.history, prompt)
+    assert gen.use_ring_context is False   # a foreign model gets chronological tensors
+
+
+def test_step_writes_kv_and_advances_cache(env):
+    model, gen = env
+    gen._prefill(torch.tensor([2, 4, 6]))
+    t0 = gen.cache.t
+    logits = gen._step(torch.tensor(11))
+    assert torch.equal(logits[0].float(), onehot(11))
+    assert gen.cache.t == t0 + 1
+    for layer in range(2):
+        k, v = gen.cache.view(layer)
+        assert torch.equal(k[0, -1, 0].float(), onehot(11)) and torch.equal(v[0, -1, 0].float(), onehot(11))
+        # the model saw the cache as it was BEFORE this token's row was written
+        assert torch.equal(model.seen_k[layer].float(), k[:, :-1].float())
+        assert torch.equal(model.seen_v[layer].float(), v[:, :-1].float())
+    assert gen.history[-1].item() == 11
+
+
+def test_window_limits_what_prefill_stores(env):
+    model, gen = env
+    prompt = torch.arange(12) % V
+    gen._prefill(prompt)
+    k, _ = gen.cache.view(0)          # W = 8: a view shows 8 rows, bulk write stored the last W - 1 = 7
+    assert k.shape[1] == 8
+    for j, tok in enumerate(prompt[-7:].tolist()):
+        assert torch.equal(k[0, 1 + j, 0].float(), onehot(tok))
+
+
+def test_generate_end_to_end(env):
+    model, gen = env
+    prompt = torch.tensor([4, 1, 4])
+    assert [int(t) for t in gen.generate(prompt, max_new_tokens=3)] == [4, 4, 4]
+    g = gen.generate(prompt, max_new_tokens=2)
+    toks = []
+    try:
+        while True:
+            toks.append(int(next(g)))
+    except StopIteration as e:
+        out, pre, step = e.value
+    assert toks == [4, 4] and out.tolist() == [4, 1, 4, 4, 4]
+    assert isinstance(pre, float) and isinstance(step, float)
+
+
+def test_sampling_helpers():
+    model = OneHotModel(8, layers=1)
+    gen = Generator(model, window=4, seed=1, device=torch.device("cpu"), dtype=torch.bfloat16)
+    gen.history = torch.tensor([1, 2, 3, 2, 1])
+    logits = torch.tensor([0.1, 0.9, 0.5, -1.0, 0.0, 0.0, 0.0, 0.0])
+    assert int(gen.sample(logits, 0.0, None, None)) == 1
+    assert int(gen.sample(logits, 1.0, 1, None)) == 1                 # top-1 == argmax
+    assert 0 <= int(gen.sample(logits, 1.0, None, 0.6)) <= 2           # nucleus keeps {1, 2, 0}
+    gen.set_repetition_penalty(1.2)
+    l2 = torch.tensor([0.95, 0.94, 0.93, 0.0, 0.0, 0.0, 0.0, 0.0])
+    pen = gen.apply_repetition_penalty(l2, gen.history[-128:], gen.rep_p_t.float(), gen._one)
+    assert int(torch.argmax(pen)) == 0                                   # tokens 1 and 2 were seen, 0 was not

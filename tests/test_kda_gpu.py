@@ -1,0 +1,115 @@
+"""Kernel 3 parity: chunked KDA (HIP) vs the naive fp32 recurrence (through the C ABI).
+
+Tolerances: outputs max-abs <= 2e-2 and mean-abs <= 2e-3 (bf16 I/O), final state
+relative Frobenius error <= 1e-3.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from daisy_amd import chunk_kda, fused_kda_gate, ops
+from helpers import assert_close_bf16, say
+
+pytestmark = pytest.mark.gpu
+
+STATE_REL = 1e-3
+
+
+def _inputs(B, T, H, seed, g_scale=1.0, D=128):
+    g = torch.Generator().manual_seed(seed)
+    q = F.normalize(torch.randn(B, T, H, D, generator=g), dim=-1).bfloat16()
+    k = F.normalize(torch.randn(B, T, H, D, generator=g), dim=-1).bfloat16()
+    v = torch.randn(B, T, H, D, generator=g).bfloat16()
+    gl = F.logsigmoid(torch.randn(B, T, H, D, generator=g)) * g_scale
+    beta = torch.sigmoid(torch.randn(B, T, H, generator=g))
+    return q, k, v, gl, beta
+
+
+def _check(o, S, o_ref, S_ref, what):
+    assert_close_bf16(o, o_ref, f"{what}: o")
+    rel = ((S.float().cpu() - S_ref).norm() / S_ref.norm()).item()
+    say(f"{what}: state rel err {rel:.3e}")
+    assert rel <= STATE_REL, f"{what}: state relative error {rel:.3e} > {STATE_REL}"
+
+
+@pytest.mark.parametrize("B,T,H,g_scale", [
+    (1, 64, 1, 1.0),      # exactly one chunk
+    (1, 128, 2, 1.0),     # two chunks: state hand-over
+    (2, 200, 2, 1.0),     # ragged last chunk
+    (1, 17, 1, 1.0),      # shorter than a chunk
+    (1, 512, 2, 0.05),    # slow decay: long memory, the S0 terms matter
+    (1, 256, 2, 8.0),     # very fast decay (|g| up to ~50 per step): nothing may overflow
+    (2, 1024, 4, 1.0),
+])
+def test_kda_matches_recurrence(B, T, H, g_scale):
+    say(f"kda case B{B} T{T} H{H} g_scale{g_scale}")
+    q, k, v, gl, beta = _inputs(B, T, H, seed=T + H, g_scale=g_scale)
+    o_ref, S_ref = oracle.kda_recurrent(q, k, v, gl, beta)
+    o, S = chunk_kda(q.cuda(), k.cuda(), v.cuda(), gl.cuda(), beta.cuda(), output_final_state=True,
+                     use_qk_l2norm_in_kernel=True)
+    torch.cuda.synchronize()
+    _check(o, S, o_ref, S_ref, "kda")
+
+
+def test_kda_initial_state_and_split_equivalence():
+    """Running [0, T1) then [T1, T) with the carried state equals one run (reference tests/test_attention_kimi.py:195-219)."""
+    B, T, H, T1 = 1, 320, 2, 128
+    q, k, v, gl, beta = (t.cuda() for t in _inputs(B, T, H, seed=5))
+    o_full, S_full = chunk_kda(q, k, v, gl, beta, output_final_state=True, use_qk_l2norm_in_kernel=True)
+    o1, S1 = chunk_kda(q[:, :T1], k[:, :T1], v[:, :T1], gl[:, :T1], beta[:, :T1], output_final_state=True,
+                       use_qk_l2norm_in_kernel=True)
+    o2, S2 = chunk_kda(q[:, T1:], k[:, T1:], v[:, T1:], gl[:, T1:], beta[:, T1:], initial_state=S1,
+                       output_final_state=True, use_qk_l2norm_in_kernel=True)
+    assert_close_bf16(torch.cat([o1, o2], 1), o_full.float(), "split o", max_abs=1e-3, mean_abs=1e-4)
+    assert ((S2 - S_full).norm() / S_full.norm()).item() < 1e-5
+    # against the oracle with a random initial state
+    S0 = torch.randn(B, H, 128, 128, generator=torch.Generator().manual_seed(1)) * 0.1
+    o_ref, S_ref = oracle.kda_recurrent(q.cpu(), k.cpu(), v.cpu(), gl.cpu(), beta.cpu(), initial_state=S0)
+    o, S = chunk_kda(q, k, v, gl, beta, initial_state=S0.cuda(), output_final_state=True, use_qk_l2norm_in_kernel=True)
+    _check(o, S, o_ref, S_ref, "kda with S0")
+
+
+def test_kda_without_l2norm_and_explicit_scale_bf16_gate():
+    B, T, H = 1, 192, 2
+    q, k, v, gl, beta = _inputs(B, T, H, seed=9)
+    glb = gl.bfloat16()
+    o_ref, S_ref = oracle.kda_recurrent(q, k, v, glb.float(), beta, scale=0.25, use_qk_l2norm=False)
+    o, S = chunk_kda(q.cuda(), k.cuda(), v.cuda(), glb.cuda(), beta.cuda(), scale=0.25, output_final_state=True,
+                     use_qk_l2norm_in_kernel=False)
+    _check(o, S, o_ref, S_ref, "kda no-l2norm")
+
+
+def test_kda_closed_forms():
+    """beta = 0: the state only decays and o reads the decayed S0; g = 0, beta = 1, q = k: o = scale * v."""
+    B, T, H = 1, 64, 1
+    q, k, v, gl, beta = (t.cuda() for t in _inputs(B, T, H, seed=2))
+    S0 = torch.randn(B, H, 128, 128, generator=torch.Generator().manual_seed(3)).cuda()
+    o, S = chunk_kda(q, k, v, gl, torch.zeros_like(beta), initial_state=S0, output_final_state=True, use_qk_l2norm_in_kernel=True)
+    want = S0 * torch.exp(gl.sum(1))[..., None]
+    assert ((S - want).norm() / want.norm()).item() < 1e-5
+    o2, _ = chunk_kda(k, k, v, torch.zeros_like(gl), torch.ones_like(beta), scale=1.0, output_final_state=False,
+                      use_qk_l2norm_in_kernel=True)
+    assert_close_bf16(o2, v.float(), "delta rule returns v")
+
+
+def test_kda_gate_matches_oracle():
+    g = torch.Generator().manual_seed(4)
+    H, Dk = 4, 128
+    x = torch.randn(2, 50, H * Dk, generator=g) * 8
+    A_log = torch.log(torch.empty(H).uniform_(1, 16, generator=g))
+    bias = torch.randn(H * Dk, generator=g)
+    for dt in (torch.float32, torch.bfloat16):
+        want = oracle.kda_gate(x.to(dt), A_log.view(1, 1, H, 1), Dk, bias)
+        got = fused_kda_gate(x.to(dt).cuda(), A_log.view(1, 1, H, 1).cuda(), Dk, bias.cuda())
+        assert got.shape == (2, 50, H, Dk) and got.dtype == dt
+        tol = 1e-5 if dt == torch.float32 else 2 ** -7
+        assert torch.allclose(got.float().cpu(), want.float(), rtol=tol, atol=1e-6)
+    y, b = fused_kda_gate(x.cuda(), A_log.cuda(), Dk, None, b=torch.zeros(2, 50, H).cuda())
+    assert torch.allclose(b, torch.full_like(b, 0.5))
+
+
+def test_kda_rejects_unsupported_shapes():
+    z = torch.zeros(1, 64, 1, 64, dtype=torch.bfloat16, device="cuda:0")
+    with pytest.raises(RuntimeError, match="Dk"):
+        ops.kda_chunk_fwd(z, z, z, z.float(), torch.zeros(1, 64, 1, device="cuda:0"))

@@ -1,0 +1,186 @@
+"""Drop-in module parity on the GPU: CausalSelfAttention.forward/prefill/step,
+KVCache ring decode and the Generator, against the CPU oracle."""
+import os
+
+import pytest
+import torch
+import torch.nn as nn
+
+os.environ["DISABLE_O_ZERO_INIT"] = "1"
+
+import oracle
+from daisy_amd import CausalSelfAttention, Generator, KVCache, WindowMask, build_window_mask
+from daisy_amd.functional import norm
+from helpers import assert_close_bf16, say
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _make(dim, H, D, receives_ve=False, seed=0, max_seq_len=4096):
+    torch.manual_seed(seed)
+    attn = CausalSelfAttention(dim=dim, num_heads=H, head_dim=D, receives_ve=receives_ve, max_seq_len=max_seq_len)
+    with torch.no_grad():
+        attn.qkvo_w.copy_((torch.randn(4, dim, dim) * 0.02).bfloat16())
+    return attn.eval()
+
+
+def test_library_rms_norm_on_gpu_matches_oracle():
+    """The projection outputs are normalised by the library routine on the GPU; pin its epsilon there too."""
+    x = (torch.randn(4, 7, 3, 128, generator=torch.Generator().manual_seed(0)) * 1e-3).bfloat16()
+    assert torch.equal(norm(x.to(DEV)).cpu(), oracle.rms_norm(x))
+    x = torch.randn(4, 7, 3, 64, generator=torch.Generator().manual_seed(1)).bfloat16()
+    assert (norm(x.to(DEV)).cpu().float() - oracle.rms_norm(x).float()).abs().max().item() <= 2 ** -7
+
+
+def test_config1_plumbing_layer():
+    """BASELINE config 1: B1 T256 d256 H4 D64 W128, fp32 x, weights N(0, 0.02), seed 0:
+    the oracle's fp32 CPU path vs the HIP path (bf16 compute)."""
+    torch.manual_seed(0)
+    dim, H, D, T, W = 256, 4, 64, 256, 128
+    w = torch.randn(4, dim, dim) * 0.02
+    x = torch.randn(1, T, dim)
+    for base, trunc in ((10000.0, False), (1024.0, True)):
+        cos, sin = oracle.rope_tables(D, T, base=base, half_truncate=trunc)
+        y_ref, k_ref, v_ref = oracle.attn_prefill(x, w, H, D, cos, sin, W)   # fp32 weights: the CPU reference
+        attn = _make(dim, H, D)
+        with torch.no_grad():
+            attn.qkvo_w.copy_(w.bfloat16())
+            attn.rotary.cos[:T].copy_(cos)
+            attn.rotary.sin[:T].copy_(sin)
+        attn = attn.to(DEV)
+        y, k, v = attn.prefill(x.to(DEV), None, attn_mask=WindowMask(W))
+        assert y.shape == (1, T, dim) and k.shape == (1, H, T, D) and v.shape == (1, H, T, D)
+        assert y.dtype == torch.bfloat16
+        assert_close_bf16(y, y_ref, f"y (base {base})")
+        assert_close_bf16(k, k_ref, "k", max_abs=4e-2, mean_abs=4e-3)   # unit-RMS values rounded to bf16
+        assert_close_bf16(v, v_ref, "v", max_abs=4e-2, mean_abs=4e-3)
+
+
+@pytest.mark.parametrize("receives_ve", [False, True])
+def test_prefill_matches_oracle_with_documents_and_ve(receives_ve):
+    dim, H, D, T, W = 512, 4, 128, 333, 100
+    attn = _make(dim, H, D, receives_ve=receives_ve, seed=1).to(DEV)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(2, T, dim, generator=g).bfloat16()
+    ve = torch.randn(2, T, dim, generator=g).bfloat16() if receives_ve else None
+    ids = torch.randint(0, 6, (1, T), generator=g)
+    w = attn.qkvo_w.detach().cpu()
+    cos, sin = attn.rotary.cos.cpu(), attn.rotary.sin.cpu()
+    y_ref, k_ref, v_ref = oracle.attn_prefill(x, w, H, D, cos, sin, W, doc_start=oracle.doc_start_from_ids(ids, 3),
+                                              ve=ve, g_ve=0.0 if receives_ve else None)
+    mask = build_window_mask(ids.to(DEV), W, 3)
+    y, k, v = attn.prefill(x.to(DEV), None if ve is None else ve.to(DEV), attn_mask=mask)
+    assert_close_bf16(y, y_ref, "y")
+    assert_close_bf16(k, k_ref, "k")
+    assert_close_bf16(v, v_ref, "v")
+    # the reference's dense additive mask is accepted too and means the same thing
+    dense = oracle.build_attn_mask(ids, W, 3).to(DEV)
+    y2 = attn(x.to(DEV), None if ve is None else ve.to(DEV), attn_mask=dense)
+    assert torch.equal(y2, y)
+
+
+@pytest.mark.parametrize("T,W", [(128, 128), (131, 128), (70, 16)])
+def test_forward_equals_steps(T, W):
+    """Reference tests/test_causal_self_attention_equivalence.py: full forward == T streaming steps (bf16, 2e-2)."""
+    dim, H, D = 128, 2, 64
+    attn = _make(dim, H, D, receives_ve=True, seed=3).to(DEV)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(1, T, dim, generator=g).bfloat16().to(DEV)
+    ve = torch.randn(1, T, H, D, generator=g).bfloat16().to(DEV)
+    y_full = attn(x, ve, attn_mask=WindowMask(W))
+    K = torch.empty(1, 0, H, D, device=DEV, dtype=torch.bfloat16)
+    V = torch.empty(1, 0, H, D, device=DEV, dtype=torch.bfloat16)
+    ys = []
+    for pos in range(T):
+        y, k_new, v_new = attn.step(x[:, pos:pos + 1], k_ctx=K, v_ctx=V, pos=pos, ve=ve[:, pos:pos + 1], window=W)
+        assert y.shape == (1, 1, dim) and k_new.shape == (1, 1, H, D)
+        K, V = torch.cat([K, k_new], 1), torch.cat([V, v_new], 1)
+        ys.append(y)
+    y_step = torch.cat(ys, 1)
+    assert torch.allclose(y_full.float(), y_step.float(), atol=2e-2, rtol=2e-2), \
+        f"max err {(y_full.float() - y_step.float()).abs().max().item()}"
+
+
+def test_step_ring_context_equals_chronological_context():
+    """The in-place ring path and the reference's tensor path give the same step, and the ring gets the new row."""
+    dim, H, D, W, B = 256, 2, 128, 32, 3
+    attn = _make(dim, H, D, seed=5).to(DEV)
+    g = torch.Generator().manual_seed(6)
+    cache_a = KVCache(L=1, B=B, H=H, W=W, D=D, device=DEV, dtype=torch.bfloat16)
+    cache_b = KVCache(L=1, B=B, H=H, W=W, D=D, device=DEV, dtype=torch.bfloat16)
+    for t in range(W + 9):     # wraps the ring
+        x = torch.randn(B, 1, dim, generator=g).bfloat16().to(DEV)
+        ring = cache_a.ring(0)
+        ya, ka, va = attn.step(x, ring, ring, t, None, window=W)
+        assert cache_a._staged[0] is True          # the kernel appended the row itself
+        cache_a.advance()
+        kc, vc = cache_b.view(0)
+        yb, kb, vb = attn.step(x, kc, vc, t, None, window=W)
+        cache_b.write(0, kb, vb)
+        cache_b.advance()
+        assert_close_bf16(ya, yb.float(), f"y at t={t}", max_abs=1e-2, mean_abs=1e-3)
+        assert torch.equal(ka, kb) and torch.equal(va, vb)
+    assert torch.equal(cache_a.k, cache_b.k) and torch.equal(cache_a.v, cache_b.v)
+
+
+class TinyModel(nn.Module):
+    """Two attention layers + embeddings, with the model-level prefill/step contract the Generator needs."""
+
+    def __init__(self, vocab=64, dim=128, H=2, D=64, window=16):
+        super().__init__()
+        self.eos_token_id = vocab - 1
+        self.window = window
+        self.embed = nn.Embedding(vocab, dim)
+        self.blocks = nn.ModuleList([nn.Module() for _ in range(2)])
+        for i, b in enumerate(self.blocks):
+            b.attn = _make(dim, H, D, seed=10 + i, max_seq_len=512)
+        self.head = nn.Linear(dim, vocab, bias=False)
+
+    def reset_history(self):
+        for b in self.blocks:
+            b.attn.reset_history()
+
+    def prefill(self, ids):
+        x = norm(self.embed(ids)).bfloat16()
+        mask = build_window_mask(ids, self.window, self.eos_token_id)
+        ks, vs = [], []
+        for b in self.blocks:
+            y, k, v = b.attn.prefill(x, None, attn_mask=mask)
+            x = x + y
+            ks.append(k); vs.append(v)
+        logits = self.head(norm(x)[:, -1].float())
+        return logits, torch.stack([torch.stack(ks), torch.stack(vs)])
+
+    def step(self, token, k_ctxs, v_ctxs, pos):
+        x = norm(self.embed(token.view(1, 1))).bfloat16()
+        ks, vs = [], []
+        for i, b in enumerate(self.blocks):
+            y, k, v = b.attn.step(x, k_ctxs[i], v_ctxs[i], pos, None, window=self.window)
+            x = x + y
+            ks.append(k); vs.append(v)
+        return self.head(norm(x).float()).view(1, -1), ks, vs
+
+
+def test_generator_ring_path_matches_full_prefill():
+    """Greedy generation with the in-place ring path: every step's logits equal a fresh prefill of the whole
+    sequence (same window semantics), so prefill -> cache -> step is consistent end to end."""
+    torch.manual_seed(0)
+    model = TinyModel().to(DEV).eval()
+    gen = Generator(model, window=model.window, seed=1, device=torch.device(DEV), dtype=torch.bfloat16, temperature=0.0)
+    assert gen.use_ring_context
+    prompt = torch.randint(0, 60, (23,), generator=torch.Generator().manual_seed(3)).to(DEV)
+    with torch.inference_mode():
+        gen.reset_history()
+        logits = gen._prefill(prompt)
+        seq = prompt
+        for _ in range(12):
+            tok = torch.argmax(logits[-1])
+            logits = gen._step(tok)
+            seq = torch.cat([seq, tok.view(1)])
+            want, _ = model.prefill(seq[None])
+            assert torch.allclose(logits.float(), want.float(), atol=3e-2, rtol=3e-2), \
+                f"step logits differ from prefill logits by {(logits.float() - want.float()).abs().max().item()}"
+        assert gen.cache.t == seq.numel()
+        out = [int(t) for t in gen.generate(prompt, max_new_tokens=5)]
+        assert len(out) == 5

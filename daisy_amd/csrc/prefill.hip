@@ -18,13 +18,16 @@
 //   A and B operands agree, so V^T is stored in LDS with key rows permuted to
 //   match (swap bits 2 and 3 of the key index inside each group of 16).
 //
-// LDS (double buffered): K tile [64][D+8] bf16 row major, V^T tile [D][64+8]
-// bf16.  The +8 element pad makes the 16-byte operand reads of 8 consecutive
-// lanes fall into distinct banks.  V is transposed in registers as 4x4 blocks
-// on its way from global memory to LDS.
+// LDS (double buffered): K and V tiles [64][D] bf16, row major, filled by direct
+// global->LDS copies (global_load_lds_dwordx4: no staging registers, no LDS
+// store instructions); the 16-byte chunks of each row are XOR-swizzled so that
+// operand reads are bank-conflict free.  V^T operands come out of the row-major
+// V tile through LDS transpose reads (ds_read_b64_tr_b16).
 //
 // Algorithmic work: 4*D flops per visible (query, key) pair.
 #include "common.h"
+
+#include <type_traits>
 
 namespace daisy {
 
@@ -60,24 +63,53 @@ __device__ __forceinline__ float pair_sum(float x) {
   return __int_as_float(r[0]) + __int_as_float(r[1]);
 }
 
-// Position inside a V^T row of key row `kv` (0..63): bits 2 and 3 swapped.
-__device__ __forceinline__ int vt_pos(int kv) { return (kv & ~12) | ((kv & 4) << 1) | ((kv & 8) >> 1); }
+// LDS transpose read (ds_read_b64_tr_b16).  Inside every block of 16 lanes, lane L receives
+// element (L % 4) of the four 8-byte chunks addressed by lanes L/4, L/4 + 4, L/4 + 8 and
+// L/4 + 12 of the block.  With lanes 4a..4a+3 of a block pointing at four key rows of V
+// (row = a) and lanes of equal L % 4... see the address set-up at the call site.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* p) {
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p);
+  return __builtin_bit_cast(u32x2, v);
+}
+
+// Asynchronous 16-byte global -> LDS copy that bypasses the vector registers
+// (global_load_lds_dwordx4): lane i of the wavefront deposits the 16 bytes at
+// gbase + byte_off at LDS address lds_addr + 16*i.  gbase and lds_addr are wavefront-uniform.
+// Issued as inline assembly so that the compiler does not serialise later LDS reads of the
+// OTHER buffer behind it; the caller waits with s_waitcnt vmcnt(0) before publishing the tile.
+__device__ __forceinline__ void copy16_to_lds_async(const uint16_t* gbase, int byte_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(byte_off), "s"(gbase), "s"(lds_addr) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(size_t)(__attribute__((address_space(3))) const void*)p;
+}
 
 template <int D, bool ROPE_K>
 __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(PrefillParams p) {
-  constexpr int KS = D + 8;        // K tile row stride (elements)
-  constexpr int VS = kBN + 8;      // V^T tile row stride (elements)
+  // LDS tiles are [64 rows][D] bf16 without padding; the 16-byte chunks of a row are stored
+  // XOR-swizzled (chunk c of row r sits at position c ^ f(r)) so that operand reads are free
+  // of bank conflicts.  The LDS has 64 banks of 4 bytes, i.e. 256 bytes per clock:
+  //   K: a 16-byte read serves 16 lanes per clock = 16 consecutive rows, same chunk
+  //      -> those rows must land in 16 different 16-byte slots of the 256-byte bank window;
+  //   V: an 8-byte transpose read serves 32 lanes per clock = 4 consecutive rows x 64 bytes
+  //      -> those rows must land in 4 different 64-byte slots.
   constexpr int NS = D / 16;       // MFMA steps over the head dim for S^T
   constexpr int NDT = D / 32;      // 32-row tiles of O^T
   constexpr int HALF = D / 2;
-  constexpr int CPR = D / 8;       // 16-byte chunks per K row
-  constexpr int NKC = ROPE_K ? (kBN * CPR / 2) / kPrefillThreads : (kBN * CPR) / kPrefillThreads;
-  constexpr int NVB = (kBN / 4) * (D / 4) / kPrefillThreads;  // 4x4 V blocks per thread
+  constexpr int CPR = D / 8;       // 16-byte chunks per row
+  constexpr int RPL = 64 / CPR;    // rows covered by one wavefront copy (1 KiB)
+  constexpr int NLD = kBN / RPL / 4;   // wavefront copies per tensor, tile and wavefront
+  constexpr int TILE = kBN * D;    // elements per LDS tile
+  auto swz_k = [](int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); };
+  auto swz_v = [](int r) { return D == 128 ? 4 * (r & 3) : 4 * ((r >> 1) & 1); };
 
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][kBN * KS];
-  __shared__ __attribute__((aligned(16))) uint16_t Vt[2][D * VS];
+  __shared__ __attribute__((aligned(1024))) uint16_t Ks[2][TILE];
+  __shared__ __attribute__((aligned(1024))) uint16_t Vs[2][TILE];
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lq = lane & 31, lh = lane >> 5;
 
   // ---- workgroup -> (batch, head, query block); XCD-aware ------------------
@@ -137,36 +169,57 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
   const uint16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
   const uint16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
 
-  // ---- staging registers ----------------------------------------------------
-  u32x4 kst[ROPE_K ? 2 * NKC : NKC];
-  u32x4 cst[ROPE_K ? 2 * NKC : 1], sst[ROPE_K ? 2 * NKC : 1];
-  u32x2 vst[NVB][4];
-
-  // V 4x4 block coordinates of this thread (see the bank analysis above VS).
-  int v_db[NVB], v_kb[NVB];
-  {
-    const int l16 = tid & 15, grp = tid >> 4;
-    constexpr int DBH = (D / 4) / 8;  // number of groups of 8 channel blocks
+  // ---- global -> LDS staging --------------------------------------------------
+  // Wavefront copy j (0 .. 64/RPL-1) of a tile moves rows RPL*j .. RPL*j+RPL-1; lane i lands
+  // at chunk position i % CPR of row i / CPR, so it fetches the chunk that belongs there.
+  const int ld_row = lane / CPR, ld_pos = lane % CPR;
+  int k_lane_off[NLD], v_lane_off[NLD];   // element offsets inside a tile's rows, per copy
 #pragma unroll
-    for (int i = 0; i < NVB; ++i) {
-      const int idx = grp + 16 * i;             // 0 .. DBH*8-1
-      const int db_hi = idx % DBH;
-      const int rest = idx / DBH;               // 3 bits: kb bit0, bit2, bit3
-      v_db[i] = db_hi * 8 + (l16 & 7);
-      v_kb[i] = (rest & 1) | ((l16 >> 3) << 1) | (((rest >> 1) & 1) << 2) | (((rest >> 2) & 1) << 3);
-    }
+  for (int i = 0; i < NLD; ++i) {
+    const int r = RPL * (4 * i + wave) + ld_row;
+    k_lane_off[i] = 8 * (ld_pos ^ swz_k(r));
+    v_lane_off[i] = 8 * (ld_pos ^ swz_v(r));
   }
 
-  auto load_tile = [&](int tile) {
-    const int kv0 = tile * kBN;
-    if constexpr (!ROPE_K) {
+  u32x4 kst[ROPE_K ? 2 * ((kBN * CPR / 2) / kPrefillThreads) : 1];
+  u32x4 cst[ROPE_K ? 2 * ((kBN * CPR / 2) / kPrefillThreads) : 1], sst[ROPE_K ? 2 * ((kBN * CPR / 2) / kPrefillThreads) : 1];
+  constexpr int NKC = (kBN * CPR / 2) / kPrefillThreads;   // (row, channel-pair chunk) items per thread when rotating K
+
+  // Per-lane source offsets of the wavefront copies relative to the first row of a tile
+  // (32-bit; the tile base is uniform, so the copy can use scalar-base addressing).
+  int k_src_off[NLD], v_src_off[NLD];
 #pragma unroll
-      for (int i = 0; i < NKC; ++i) {
-        const int c = tid + kPrefillThreads * i;
-        const int row = min(kv0 + c / CPR, p.T - 1);
-        kst[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)row * p.k_st + 8 * (c % CPR));
+  for (int i = 0; i < NLD; ++i) {
+    const int row = RPL * (4 * i + wave) + ld_row;
+    k_src_off[i] = row * (int)p.k_st + k_lane_off[i];
+    v_src_off[i] = row * (int)p.v_st + v_lane_off[i];
+  }
+
+  const uint32_t ks_lds = lds_address(&Ks[0][0]), vs_lds = lds_address(&Vs[0][0]);
+
+  auto issue_copies = [&](int tile, auto buf_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
+    const int kv0 = tile * kBN;
+    const uint16_t* kt = kbase + (int64_t)kv0 * p.k_st;
+    const uint16_t* vt = vbase + (int64_t)kv0 * p.v_st;
+    if (kv0 + kBN <= p.T) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const uint32_t dst = 2 * (buf * TILE + (4 * i + wave) * 512);
+        if constexpr (!ROPE_K) copy16_to_lds_async(kt, 2 * k_src_off[i], ks_lds + dst);
+        copy16_to_lds_async(vt, 2 * v_src_off[i], vs_lds + dst);
       }
     } else {
+      // The tile reaches past the last row: clamp (the surplus rows are masked by causality).
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const uint32_t dst = 2 * (buf * TILE + (4 * i + wave) * 512);
+        const int row = min(RPL * (4 * i + wave) + ld_row, p.T - 1 - kv0);
+        if constexpr (!ROPE_K) copy16_to_lds_async(kt, 2 * (row * (int)p.k_st + k_lane_off[i]), ks_lds + dst);
+        copy16_to_lds_async(vt, 2 * (row * (int)p.v_st + v_lane_off[i]), vs_lds + dst);
+      }
+    }
+    if constexpr (ROPE_K) {
 #pragma unroll
       for (int i = 0; i < NKC; ++i) {
         const int c = tid + kPrefillThreads * i;
@@ -183,30 +236,18 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
         sst[2 * i + 1] = *reinterpret_cast<const u32x4*>(sp + 4);
       }
     }
-#pragma unroll
-    for (int i = 0; i < NVB; ++i) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int row = min(kv0 + 4 * v_kb[i] + j, p.T - 1);
-        vst[i][j] = *reinterpret_cast<const u32x2*>(vbase + (int64_t)row * p.v_st + 4 * v_db[i]);
-      }
-    }
   };
 
-  auto store_tile = [&](int tile, int buf) {
-    if constexpr (!ROPE_K) {
-#pragma unroll
-      for (int i = 0; i < NKC; ++i) {
-        const int c = tid + kPrefillThreads * i;
-        *reinterpret_cast<u32x4*>(&Ks[buf][(c / CPR) * KS + 8 * (c % CPR)]) = kst[i];
-      }
-    } else {
-      // This workgroup also publishes the rotated keys of its own query rows.
+  // Completes the staging of a tile: waits for the asynchronous copies and, when K is rotated
+  // here, rotates the register-staged K rows into LDS (and publishes this workgroup's own rows).
+  auto finish_copies = [&](int tile, auto buf_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
+    if constexpr (ROPE_K) {
       const bool publish = p.k_out != nullptr && (tile * kBN) / kBM == qb;
 #pragma unroll
       for (int i = 0; i < NKC; ++i) {
         const int c = tid + kPrefillThreads * i;
-        const int r = c / (CPR / 2), dc = 8 * (c % (CPR / 2));
+        const int r = c / (CPR / 2), cc = c % (CPR / 2), dc = 8 * cc;
         float x1[8], x2[8], y1[8], y2[8];
         unpack8(kst[2 * i], x1);
         unpack8(kst[2 * i + 1], x2);
@@ -222,8 +263,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
           y2[e] = rope_hi(x1[e], x2[e], cs[e], sn[e]);
         }
         const u32x4 a = pack8(y1), bb = pack8(y2);
-        *reinterpret_cast<u32x4*>(&Ks[buf][r * KS + dc]) = a;
-        *reinterpret_cast<u32x4*>(&Ks[buf][r * KS + dc + HALF]) = bb;
+        *reinterpret_cast<u32x4*>(&Ks[buf][r * D + 8 * (cc ^ swz_k(r))]) = a;
+        *reinterpret_cast<u32x4*>(&Ks[buf][r * D + 8 * ((cc + CPR / 2) ^ swz_k(r))]) = bb;
         const int grow = tile * kBN + r;
         if (publish && grow < p.T) {
           uint16_t* op = p.k_out + b * p.ko_sb + (int64_t)grow * p.ko_st + h * p.ko_sh + dc;
@@ -232,20 +273,12 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
         }
       }
     }
-#pragma unroll
-    for (int i = 0; i < NVB; ++i) {
-      const u32x2 r0 = vst[i][0], r1 = vst[i][1], r2 = vst[i][2], r3 = vst[i][3];
-      u32x2 c0, c1, c2, c3;
-      c0.x = (r0.x & 0xffffu) | (r1.x << 16);         c0.y = (r2.x & 0xffffu) | (r3.x << 16);
-      c1.x = (r0.x >> 16) | (r1.x & 0xffff0000u);     c1.y = (r2.x >> 16) | (r3.x & 0xffff0000u);
-      c2.x = (r0.y & 0xffffu) | (r1.y << 16);         c2.y = (r2.y & 0xffffu) | (r3.y << 16);
-      c3.x = (r0.y >> 16) | (r1.y & 0xffff0000u);     c3.y = (r2.y >> 16) | (r3.y & 0xffff0000u);
-      uint16_t* dst = &Vt[buf][(4 * v_db[i]) * VS + vt_pos(4 * v_kb[i])];
-      *reinterpret_cast<u32x2*>(dst) = c0;
-      *reinterpret_cast<u32x2*>(dst + VS) = c1;
-      *reinterpret_cast<u32x2*>(dst + 2 * VS) = c2;
-      *reinterpret_cast<u32x2*>(dst + 3 * VS) = c3;
-    }
+    // vmcnt(0) as a compiler-visible wait (encoding: vmcnt = 0, expcnt = 7, lgkmcnt = 15): the
+    // asynchronous copies have landed, and the compiler also learns that no earlier vector
+    // load is pending, so it places no conservative vmcnt waits inside the tile loop (those
+    // would wait for the copies of the NEXT tile, which it cannot see).
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" ::: "memory");
   };
 
   // ---- accumulators -----------------------------------------------------------
@@ -254,111 +287,152 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
   for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
-  float m_run = -INFINITY;  // running max of scale*log2e*s for this lane's query
+  float m_run = -INFINITY;  // reference maximum (scaled, log2 domain) of this lane's query
   float l_run = 0.f;        // this lane's share of the running sum
 
-  load_tile(t_lo);
-  store_tile(t_lo, 0);
-  __syncthreads();
-
-  for (int tile = t_lo; tile <= t_hi; ++tile) {
-    const int buf = (tile - t_lo) & 1;
-    if (tile < t_hi) load_tile(tile + 1);
-
-    const int kv0 = tile * kBN;
-    // Sub-blocks of 32 keys this wavefront needs (wave-uniform).
-    bool need[2];
+  // Per-lane LDS element offsets of the operand reads (inside one tile).
+  //   K (A operand of S^T): row = key lq of the 32-key sub-block, step s wants chunk 2s + lh.
+  //   V (A operand of O^T, LDS transpose read): the lane's block of 16 covers output channels
+  //   32dt + 16*(block & 1) + 0..15 and keys 4*lh + 0..3 (+8, +16, ... as immediates); lane i of
+  //   the block addresses key i/4, channels 4*(i%4)..+3 and receives channel i, four keys.
+  const uint16_t* k_rd[NS];
+  const uint16_t* v_rd[NDT];
 #pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-      const int kmin = kv0 + 32 * sb, kmax = kmin + 31;
-      need[sb] = wave_live && kmin <= q_w_max && kmax >= lo_w_min;
+  for (int s = 0; s < NS; ++s) k_rd[s] = &Ks[0][0] + lq * D + 8 * ((2 * s + lh) ^ swz_k(lq));
+  {
+    const int i16 = lane & 15, vrow = 4 * lh + (i16 >> 2);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      const int chunk = 4 * dt + 2 * ((lane >> 4) & 1) + ((i16 & 3) >> 1);
+      v_rd[dt] = &Vs[0][0] + vrow * D + 8 * (chunk ^ swz_v(vrow)) + 4 * (i16 & 1);
     }
+  }
 
-    if (need[0] || need[1]) {
-      f32x16 sacc[2];
+  // One tile of 64 keys.  MASKED = false: both 32-key sub-blocks are needed by this
+  // wavefront and fully visible to all of its queries (no mask, no skipping).
+  auto process_tile = [&](auto buf_tag, int kv0, auto masked_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    bool need[2] = {true, true};
+    if constexpr (MASKED) {
 #pragma unroll
       for (int sb = 0; sb < 2; ++sb) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[sb][r] = 0.f;
-        if (need[sb]) {
-          const uint16_t* kp = &Ks[buf][(32 * sb + lq) * KS + 8 * lh];
-#pragma unroll
-          for (int s = 0; s < NS; ++s) {
-            const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(kp + 16 * s));
-            sacc[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[s], sacc[sb], 0, 0, 0);
-          }
-          const int kmin = kv0 + 32 * sb, kmax = kmin + 31;
-          const bool full = kmax <= q_w_min && kmin >= lo_w_max;
-          if (!full) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int kv = kmin + 8 * (r >> 2) + 4 * lh + (r & 3);
-              if (kv > qrow || kv < lo_q) sacc[sb][r] = -INFINITY;
-            }
-          }
-        } else {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) sacc[sb][r] = -INFINITY;
-        }
+        const int kmin = kv0 + 32 * sb, kmax = kmin + 31;
+        need[sb] = kmin <= q_w_max && kmax >= lo_w_min;
       }
+    }
+    f32x16 sacc[2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[sb][r] = 0.f;
+      if (!MASKED || need[sb]) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+          const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(k_rd[s] + (buf * TILE + 32 * sb * D)));
+          sacc[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[s], sacc[sb], 0, 0, 0);
+        }
+        if constexpr (MASKED) {
+          const int kmin = kv0 + 32 * sb;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int kv = kmin + 8 * (r >> 2) + 4 * lh + (r & 3);
+            if (kv > qrow || kv < lo_q) sacc[sb][r] = -INFINITY;
+          }
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[sb][r] = -INFINITY;
+      }
+    }
 
-      // ---- online softmax (log2 domain) --------------------------------------
-      float mt = -INFINITY;
+    // ---- online softmax (log2 domain, lazy rescale) ------------------------------
+    // The reference maximum m_run only moves when some query of the wavefront sees a
+    // score more than 8 (log2 units) above it; until then probabilities are at most 2^8,
+    // which bf16 and the fp32 sums hold without loss, and O is not touched.
+    float mt = -INFINITY;
 #pragma unroll
-      for (int sb = 0; sb < 2; ++sb)
+    for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sacc[sb][r]);
-      mt = pair_max(mt) * p.scale_log2e;
+      for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sacc[sb][r]);
+    mt = pair_max(mt) * p.scale_log2e;
+    if (__builtin_amdgcn_ballot_w64(mt > m_run + 8.f) != 0) {
       const float m_new = fmaxf(m_run, mt);
       const float mu = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = fast_exp2(m_run - mu);
       m_run = m_new;
-      float lsum = 0.f;
-      bf16x8 pfrag[2][2];
-#pragma unroll
-      for (int sb = 0; sb < 2; ++sb) {
-        float pv[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          pv[r] = fast_exp2(fmaf(sacc[sb][r], p.scale_log2e, -mu));
-          lsum += pv[r];
-        }
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-          u32x4 pk;
-          pk.x = pack_bf16x2(pv[8 * m + 0], pv[8 * m + 1]);
-          pk.y = pack_bf16x2(pv[8 * m + 2], pv[8 * m + 3]);
-          pk.z = pack_bf16x2(pv[8 * m + 4], pv[8 * m + 5]);
-          pk.w = pack_bf16x2(pv[8 * m + 6], pv[8 * m + 7]);
-          pfrag[sb][m] = __builtin_bit_cast(bf16x8, pk);
-        }
-      }
-      l_run = l_run * alpha + lsum;
+      l_run *= alpha;
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+    }
+    const float mu = (m_run == -INFINITY) ? 0.f : m_run;
+    float lsum = 0.f;
+    bf16x8 pfrag[2][2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      float pv[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        pv[r] = fast_exp2(fmaf(sacc[sb][r], p.scale_log2e, -mu));
+        lsum += pv[r];
+      }
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+        u32x4 pk;
+        pk.x = pack_bf16x2(pv[8 * m + 0], pv[8 * m + 1]);
+        pk.y = pack_bf16x2(pv[8 * m + 2], pv[8 * m + 3]);
+        pk.z = pack_bf16x2(pv[8 * m + 4], pv[8 * m + 5]);
+        pk.w = pack_bf16x2(pv[8 * m + 6], pv[8 * m + 7]);
+        pfrag[sb][m] = __builtin_bit_cast(bf16x8, pk);
+      }
+    }
+    l_run += lsum;
 
-      // ---- O^T += V^T P^T ---------------------------------------------------------
+    // ---- O^T += V^T P^T ---------------------------------------------------------
 #pragma unroll
-      for (int sb = 0; sb < 2; ++sb) {
-        if (need[sb]) {
+    for (int sb = 0; sb < 2; ++sb) {
+      if (!MASKED || need[sb]) {
 #pragma unroll
-          for (int m = 0; m < 2; ++m) {
-            const int m16 = 2 * sb + m;
+        for (int m = 0; m < 2; ++m) {
+          const int voff = buf * TILE + (32 * sb + 16 * m) * D;
 #pragma unroll
-            for (int dt = 0; dt < NDT; ++dt) {
-              const uint16_t* vp = &Vt[buf][(32 * dt + lq) * VS + 16 * m16 + 8 * lh];
-              const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(vp));
-              oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pfrag[sb][m], oacc[dt], 0, 0, 0);
-            }
+          for (int dt = 0; dt < NDT; ++dt) {
+            const u32x2 a0 = lds_read_tr16(v_rd[dt] + voff);            // keys 16m + 4lh + 0..3
+            const u32x2 a1 = lds_read_tr16(v_rd[dt] + voff + 8 * D);    // keys 16m + 8 + 4lh + 0..3
+            const u32x4 av = {a0.x, a0.y, a1.x, a1.y};
+            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), pfrag[sb][m], oacc[dt], 0, 0, 0);
           }
         }
       }
     }
+  };
 
-    if (tile < t_hi) store_tile(tile + 1, buf ^ 1);
+  using Buf0 = std::integral_constant<int, 0>;
+  using Buf1 = std::integral_constant<int, 1>;
+  issue_copies(t_lo, Buf0{});
+  finish_copies(t_lo, Buf0{});
+  __syncthreads();
+
+  // One iteration: start the copies of the next tile into the other buffer, compute on this
+  // buffer, then wait for the copies and meet the other wavefronts.
+  auto iteration = [&](int tile, auto buf_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
+    using Other = std::integral_constant<int, buf ^ 1>;
+    if (tile < t_hi) issue_copies(tile + 1, Other{});
+    const int kv0 = tile * kBN;
+    if (wave_live && kv0 <= q_w_max && kv0 + kBN - 1 >= lo_w_min) {
+      const bool clean = kv0 + kBN - 1 <= q_w_min && kv0 >= lo_w_max;
+      if (clean) process_tile(buf_tag, kv0, std::false_type{});
+      else process_tile(buf_tag, kv0, std::true_type{});
+    }
+    if (tile < t_hi) finish_copies(tile + 1, Other{});
     __syncthreads();
+  };
+  for (int tile = t_lo; tile <= t_hi; tile += 2) {
+    iteration(tile, Buf0{});
+    if (tile + 1 <= t_hi) iteration(tile + 1, Buf1{});
   }
 
   // ---- epilogue ---------------------------------------------------------------

@@ -15,14 +15,21 @@
 //   rescale of O^T is a per-lane scalar, and the accumulator registers of S^T,
 //   converted to bf16, already ARE the B operand of the second product: the
 //   contraction index of an MFMA may be enumerated in any order as long as the
-//   A and B operands agree, so V^T is stored in LDS with key rows permuted to
-//   match (swap bits 2 and 3 of the key index inside each group of 16).
+//   A and B operands agree, so the V^T operand simply fetches, per lane, the key
+//   rows 16m + 8g + 4*(l/32) + 0..3 that the lane's P registers hold.
 //
 // LDS (double buffered): K and V tiles [64][D] bf16, row major, filled by direct
 // global->LDS copies (global_load_lds_dwordx4: no staging registers, no LDS
 // store instructions); the 16-byte chunks of each row are XOR-swizzled so that
 // operand reads are bank-conflict free.  V^T operands come out of the row-major
-// V tile through LDS transpose reads (ds_read_b64_tr_b16).
+// V tile through LDS transpose reads (ds_read_b64_tr_b16): inside a block of 16
+// lanes, lane L receives element L%4 of the four 8-byte chunks addressed by
+// lanes L/4, L/4+4, L/4+8, L/4+12; with lane i of a block addressing key i/4,
+// channels 4*(i%4)..+3, lane i receives channel i of four consecutive keys.
+//
+// Two kernels share this structure: prefill_pipe_kernel (keys need no rotation
+// here; software pipelined) and prefill_mfma_kernel<D, true> (keys are rotated
+// while they are staged into LDS).
 //
 // Algorithmic work: 4*D flops per visible (query, key) pair.
 #include "common.h"
@@ -63,10 +70,7 @@ __device__ __forceinline__ float pair_sum(float x) {
   return __int_as_float(r[0]) + __int_as_float(r[1]);
 }
 
-// LDS transpose read (ds_read_b64_tr_b16).  Inside every block of 16 lanes, lane L receives
-// element (L % 4) of the four 8-byte chunks addressed by lanes L/4, L/4 + 4, L/4 + 8 and
-// L/4 + 12 of the block.  With lanes 4a..4a+3 of a block pointing at four key rows of V
-// (row = a) and lanes of equal L % 4... see the address set-up at the call site.
+// LDS transpose read (ds_read_b64_tr_b16); semantics in the header comment.
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* p) {
   s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p);
@@ -81,6 +85,11 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* p) {
 __device__ __forceinline__ void copy16_to_lds_async(const uint16_t* gbase, int byte_off, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :: "v"(byte_off), "s"(gbase), "s"(lds_addr) : "memory");
+}
+typedef __attribute__((address_space(3))) const uint16_t* lds_u16_ptr;
+__device__ __forceinline__ u32x2 lds_read_tr16_as3(lds_u16_ptr p) {
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p);
+  return __builtin_bit_cast(u32x2, v);
 }
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(size_t)(__attribute__((address_space(3))) const void*)p;
@@ -453,6 +462,325 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
   }
 }
 
+// Software-pipelined variant (keys already rotated or no RoPE on keys): the O^T += V^T P^T
+// product of tile i-1 is issued in the same basic block as the softmax of tile i, so the matrix
+// pipe works while the vector ALU does max / exp2 / sum / convert, inside one wavefront and
+// not only across the two wavefronts that share a SIMD.  V therefore runs one tile behind K:
+//   iteration i:  copies  K(i+1) -> Kbuf[(i+1)&1],  V(i) -> Vbuf[i&1]
+//                 S(i) = K(i) Q^T;   then   O += V(i-1)^T P(i-1)  ||  P(i) = softmax(S(i))
+// A rescale of O that the softmax of tile i asks for is applied at the start of the next fused
+// block (before P(i) is accumulated), which keeps that block free of branches.
+// A wavefront works on the contiguous tile range [tw_lo, tw_hi] that its 32 queries can see
+// (inside the workgroup's range); both 32-key halves of a tile in that range are computed and
+// masked per element where needed.
+template <int D>
+__global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(PrefillParams p) {
+  constexpr int NS = D / 16, NDT = D / 32, HALF = D / 2, CPR = D / 8;
+  constexpr int RPL = 64 / CPR, NLD = kBN / RPL / 4, TILE = kBN * D;
+  auto swz_k = [](int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); };
+  auto swz_v = [](int r) { return D == 128 ? 4 * (r & 3) : 4 * ((r >> 1) & 1); };
+
+  __shared__ __attribute__((aligned(1024))) uint16_t Ks[2][TILE];
+  __shared__ __attribute__((aligned(1024))) uint16_t Vs[2][TILE];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lq = lane & 31, lh = lane >> 5;
+
+  int vid = blockIdx.x;
+  {
+    const int nwg = gridDim.x;
+    if ((nwg & 7) == 0) vid = (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3);
+  }
+  const int qb = p.nqb - 1 - (vid % p.nqb);
+  const int bh = vid / p.nqb;
+  const int h = bh % p.H, b = bh / p.H;
+
+  const int q0 = qb * kBM;
+  const int qw0 = q0 + wave * 32;
+  const int qrow = min(qw0 + lq, p.T - 1);
+  const int lo_q = row_lo(p, qrow);
+  const int lo_w_min = __builtin_amdgcn_readlane(lo_q, 0);
+  const int lo_w_max = __builtin_amdgcn_readlane(lo_q, 31);
+  const int q_w_min = min(qw0, p.T - 1), q_w_max = min(qw0 + 31, p.T - 1);
+
+  const int t_lo = row_lo(p, q0) / kBN;
+  const int t_hi = min(q0 + kBM - 1, p.T - 1) / kBN;
+  // This wavefront's own tile range (empty when all of its rows are past the end).
+  const int tw_lo = lo_w_min / kBN;
+  const int tw_hi = (qw0 < p.T) ? q_w_max / kBN : -1;
+
+  const uint16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
+  const uint16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
+
+  // ---- global -> LDS copies (layout as in prefill_mfma_kernel) ---------------------------
+  const int ld_row = lane / CPR, ld_pos = lane % CPR;
+  int k_src_off[NLD], v_src_off[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; ++i) {
+    const int r = RPL * (4 * i + wave) + ld_row;
+    k_src_off[i] = r * (int)p.k_st + 8 * (ld_pos ^ swz_k(r));
+    v_src_off[i] = r * (int)p.v_st + 8 * (ld_pos ^ swz_v(r));
+  }
+  const uint32_t ks_lds = lds_address(&Ks[0][0]), vs_lds = lds_address(&Vs[0][0]);
+
+  auto copy_tile = [&](const uint16_t* base, int stride, const int* src_off, bool is_k, uint32_t lds, int tile, int buf) {
+    const int kv0 = tile * kBN;
+    const uint16_t* tb = base + (int64_t)kv0 * stride;
+    const uint32_t dst = lds + 2 * (buf * TILE + wave * 512);
+    if (kv0 + kBN <= p.T) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) copy16_to_lds_async(tb, 2 * src_off[i], dst + 2 * (4 * i * 512));
+    } else {
+      // The tile reaches past the last row: clamp (the surplus rows are masked by causality).
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int r = RPL * (4 * i + wave) + ld_row;
+        const int row = min(r, p.T - 1 - kv0);
+        const int chunk = ld_pos ^ (is_k ? swz_k(r) : swz_v(r));
+        copy16_to_lds_async(tb, 2 * (row * stride + 8 * chunk), dst + 2 * (4 * i * 512));
+      }
+    }
+  };
+  auto copy_k = [&](int tile, int buf) { copy_tile(kbase, (int)p.k_st, k_src_off, true, ks_lds, tile, buf); };
+  auto copy_v = [&](int tile, int buf) { copy_tile(vbase, (int)p.v_st, v_src_off, false, vs_lds, tile, buf); };
+  auto copies_landed = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), visible to the compiler's wait-count model
+    asm volatile("" ::: "memory");
+  };
+
+  // The first copy goes out before anything else so that its latency overlaps the Q loads.
+  copy_k(t_lo, 0);
+  // V buffer 1 is read (times a zero P) before anything was copied into it: clear it.
+  {
+    u32x4 z = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < TILE / 8 / kPrefillThreads; ++i)
+      *reinterpret_cast<u32x4*>(&Vs[1][8 * (tid + kPrefillThreads * i)]) = z;
+  }
+
+  // ---- Q fragment (B operand), RoPE fused ----------------------------------
+  bf16x8 qreg[NS];
+  {
+    const uint16_t* qptr = p.q + b * p.q_sb + (int64_t)qrow * p.q_st + h * p.q_sh + 8 * lh;
+    u32x4 raw[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) raw[s] = *reinterpret_cast<const u32x4*>(qptr + 16 * s);
+    if (p.cos != nullptr) {
+      const float* cr = p.cos + (int64_t)qrow * HALF + 8 * lh;
+      const float* sr = p.sin + (int64_t)qrow * HALF + 8 * lh;
+#pragma unroll
+      for (int s = 0; s < NS / 2; ++s) {
+        float x1[8], x2[8], y1[8], y2[8];
+        unpack8(raw[s], x1);
+        unpack8(raw[s + NS / 2], x2);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float c = cr[16 * s + e], sn = sr[16 * s + e];
+          y1[e] = rope_lo(x1[e], x2[e], c, sn);
+          y2[e] = rope_hi(x1[e], x2[e], c, sn);
+        }
+        raw[s] = pack8(y1);
+        raw[s + NS / 2] = pack8(y2);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < NS; ++s) qreg[s] = __builtin_bit_cast(bf16x8, raw[s]);
+  }
+
+  // Per-lane LDS read pointers into buffer 0 (32-bit LDS addresses).
+  lds_u16_ptr k_rd[NS];
+  lds_u16_ptr v_rd[NDT];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) k_rd[s] = (lds_u16_ptr)&Ks[0][0] + lq * D + 8 * ((2 * s + lh) ^ swz_k(lq));
+  {
+    const int i16 = lane & 15, vrow = 4 * lh + (i16 >> 2);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      const int chunk = 4 * dt + 2 * ((lane >> 4) & 1) + ((i16 & 3) >> 1);
+      v_rd[dt] = (lds_u16_ptr)&Vs[0][0] + vrow * D + 8 * (chunk ^ swz_v(vrow)) + 4 * (i16 & 1);
+    }
+  }
+
+  f32x16 oacc[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  float alpha_pend = 1.f;          // rescale of O asked for by the last softmax, not applied yet
+  bool rescale_pend = false;       // wave-uniform
+  bf16x8 pfrag[2][2];              // P of the previous tile (B operands of the delayed product)
+  {
+    const u32x4 z = {0, 0, 0, 0};
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int m = 0; m < 2; ++m) pfrag[sb][m] = __builtin_bit_cast(bf16x8, z);
+  }
+
+  auto apply_pending_rescale = [&]() {
+    if (rescale_pend) {
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha_pend;
+      rescale_pend = false;
+    }
+  };
+
+  // O^T += V^T P^T with the P left by the previous tile, V from buffer offset vofs (elements).
+  auto pv_product = [&](int vofs) {
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+          lds_u16_ptr vp = v_rd[dt] + vofs;
+          const u32x2 a0 = lds_read_tr16_as3(vp + (32 * sb + 16 * m) * D);
+          const u32x2 a1 = lds_read_tr16_as3(vp + (32 * sb + 16 * m + 8) * D);
+          const u32x4 av = {a0.x, a0.y, a1.x, a1.y};
+          oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), pfrag[sb][m], oacc[dt], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  // One tile of this wavefront: S = K Q^T, then (one basic block) the delayed product of the
+  // previous tile together with the softmax of this one.
+  auto wave_tile = [&](int tile, int par, auto masked_tag) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    const int kv0 = tile * kBN;
+    const int kofs = par * TILE, vofs = (par ^ 1) * TILE;
+    f32x16 sc[2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[sb][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      lds_u16_ptr kp = k_rd[s] + kofs;
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(kp + 32 * sb * D));
+        sc[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[s], sc[sb], 0, 0, 0);
+      }
+    }
+    apply_pending_rescale();
+    pv_product(vofs);
+    if constexpr (MASKED) {
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb) {
+        // element r of this lane is key kv0 + 32sb + 4lh + c_r with c_r = 8*(r/4) + r%4
+        const int hi = qrow - (kv0 + 32 * sb + 4 * lh);    // visible iff lo <= c_r <= hi
+        const int lo = lo_q - (kv0 + 32 * sb + 4 * lh);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int c = 8 * (r >> 2) + (r & 3);
+          if (c > hi || c < lo) sc[sb][r] = -INFINITY;
+        }
+      }
+    }
+    float mt = -INFINITY;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sc[sb][r]);
+    mt = pair_max(mt) * p.scale_log2e;
+    // Lazy rescale: the reference maximum only moves when some query of the wavefront sees a
+    // score more than 8 (log2 units) above it; until then probabilities stay below 2^8, which
+    // bf16 and the fp32 sums hold without loss, and O is not touched.
+    const bool move = __builtin_amdgcn_ballot_w64(mt > m_run + 8.f) != 0;
+    const float m_new = move ? fmaxf(m_run, mt) : m_run;
+    const float mu = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = fast_exp2(m_run - mu);      // 1 when the maximum did not move, 0 on the first tile
+    m_run = m_new;
+    alpha_pend = alpha;
+    rescale_pend = move;
+    float lsum = 0.f;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      float pv[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        pv[r] = fast_exp2(fmaf(sc[sb][r], p.scale_log2e, -mu));
+        lsum += pv[r];
+      }
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+        u32x4 pk;
+        pk.x = pack_bf16x2(pv[8 * m + 0], pv[8 * m + 1]);
+        pk.y = pack_bf16x2(pv[8 * m + 2], pv[8 * m + 3]);
+        pk.z = pack_bf16x2(pv[8 * m + 4], pv[8 * m + 5]);
+        pk.w = pack_bf16x2(pv[8 * m + 6], pv[8 * m + 7]);
+        pfrag[sb][m] = __builtin_bit_cast(bf16x8, pk);
+      }
+    }
+    l_run = l_run * alpha + lsum;
+  };
+
+  copies_landed();
+  __syncthreads();
+
+  // Iteration `tile`, parity par = (tile - t_lo) & 1: K(tile) is in K buffer par and V(tile-1)
+  // in V buffer par^1.  The tiles of a wavefront come in three runs -- masked ones at the window
+  // / document edge, fully visible ones, masked ones at the diagonal -- and each run has its own
+  // loop, so that the hot loop over fully visible tiles contains one code path only.
+  auto generic_tiles = [&](int from, int to) {
+    for (int tile = from; tile <= to; ++tile) {
+      const int par = (tile - t_lo) & 1;
+      if (tile + 1 <= t_hi) copy_k(tile + 1, par ^ 1);
+      copy_v(tile, par);
+      if (tile >= tw_lo && tile <= tw_hi) {
+        wave_tile(tile, par, std::true_type{});
+      } else if (tile == tw_hi + 1 && tw_hi >= tw_lo) {
+        // drain: the product of this wavefront's last tile
+        apply_pending_rescale();
+        pv_product((par ^ 1) * TILE);
+      }
+      copies_landed();
+      __syncthreads();
+    }
+  };
+  // Fully visible tiles of this wavefront: first key >= every row's lower bound, last key <=
+  // the first row.
+  int c_lo = max((lo_w_max + kBN - 1) / kBN, max(tw_lo, t_lo));
+  int c_hi = min((q_w_min + 1) / kBN - 1, min(tw_hi, t_hi));
+  if (c_hi < c_lo) { c_lo = t_hi + 1; c_hi = t_hi; }   // none: everything runs in the first generic loop
+  generic_tiles(t_lo, c_lo - 1);
+  for (int tile = c_lo; tile <= c_hi; ++tile) {
+    const int par = (tile - t_lo) & 1;
+    if (tile + 1 <= t_hi) copy_k(tile + 1, par ^ 1);
+    copy_v(tile, par);
+    wave_tile(tile, par, std::false_type{});
+    copies_landed();
+    __syncthreads();
+  }
+  generic_tiles(c_hi + 1, t_hi);
+  // Wavefronts whose range ends with the workgroup's last tile drain after the loop.
+  if (tw_hi == t_hi && tw_hi >= tw_lo) {
+    apply_pending_rescale();
+    pv_product(((t_hi - t_lo) & 1) * TILE);
+  }
+
+  const float l_tot = pair_sum(l_run);
+  const float inv = 1.f / l_tot;
+  if (qw0 + lq < p.T) {
+    uint16_t* op = p.o + b * p.o_sb + (int64_t)(qw0 + lq) * p.o_st + h * p.o_sh + 4 * lh;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w.x = pack_bf16x2(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
+        w.y = pack_bf16x2(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
+        *reinterpret_cast<u32x2*>(op + 32 * dt + 8 * g) = w;
+      }
+    }
+  }
+}
+
 // Rotates keys once and stores them with the caller's output strides.
 template <int D>
 __global__ __launch_bounds__(256) void rope_k_kernel(PrefillParams p) {
@@ -559,11 +887,11 @@ static int launch_mfma(PrefillParams p, bool rope_in_kernel, hipStream_t s) {
     hipLaunchKernelGGL(rope_k_kernel<D>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, p);
     DAISY_CHECK_LAUNCH("rope_k_kernel");
     p.k = p.k_out; p.k_sb = p.ko_sb; p.k_st = p.ko_st; p.k_sh = p.ko_sh;
-    hipLaunchKernelGGL((prefill_mfma_kernel<D, false>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
+    hipLaunchKernelGGL((prefill_pipe_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
   } else if (p.cos != nullptr) {
     hipLaunchKernelGGL((prefill_mfma_kernel<D, true>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
   } else {
-    hipLaunchKernelGGL((prefill_mfma_kernel<D, false>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
+    hipLaunchKernelGGL((prefill_pipe_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
   }
   DAISY_CHECK_LAUNCH("prefill_mfma_kernel");
   return DAISY_OK;

@@ -90,6 +90,20 @@ __device__ __forceinline__ float group_sum(float x) {
   return x;
 }
 
+// ---- asynchronous global -> LDS copies ------------------------------------------
+// Asynchronous 16-byte global -> LDS copy that bypasses the vector registers
+// (global_load_lds_dwordx4): lane i of the wavefront deposits the 16 bytes at
+// gbase + byte_off at LDS address lds_addr + 16*i.  gbase and lds_addr are wavefront-uniform.
+// Issued as inline assembly so that the compiler does not serialise later LDS reads of the
+// OTHER buffer behind it; the caller waits with s_waitcnt vmcnt(0) before publishing the tile.
+__device__ __forceinline__ void copy16_to_lds_async(const uint16_t* gbase, int byte_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(byte_off), "s"(gbase), "s"(lds_addr) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(size_t)(__attribute__((address_space(3))) const void*)p;
+}
+
 // ---- host-side error plumbing --------------------------------------------
 void set_error(const char* fmt, ...);
 

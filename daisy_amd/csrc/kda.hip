@@ -42,7 +42,8 @@ __global__ __launch_bounds__(256) void kda_gate_kernel(const void* g, const floa
 //   KtH + KtL = (exp(G_last - G) (.) K)^T split into two bf16 terms, [128][64], position permuted
 //   U0T = U0^T                      fp32 [128][64]
 //   dec = exp(G_last)               fp32 [128]
-// kda_state_kernel (one wavefront per (batch, head, 16 value columns)) then
+// kda_state_kernel (one wavefront per (batch, head, 16 value columns), two wavefronts per
+// workgroup sharing the chunk data through double-buffered LDS stages) then
 // walks the chunks in order with the fp32 state in registers; every product in
 // it is a v_mfma_f32_16x16x32_bf16 whose B operand is an accumulator (S0 or U)
 // converted to bf16 in place: in the 16x16 accumulator layout lane l holds
@@ -78,13 +79,15 @@ __host__ __device__ constexpr int perm32_inv(int p) { return (p & ~0x1c) | ((p &
 
 __device__ __forceinline__ f32x4 lds_f4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 
-__global__ __launch_bounds__(256) void kda_prep_kernel(KdaParams p) {
+__global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
   __shared__ __attribute__((aligned(16))) float G[KC][KD];           // inclusive running log-decay
   __shared__ __attribute__((aligned(16))) float EG[KC][KD];          // exp(g) per row; later staging for Wn
   __shared__ __attribute__((aligned(16))) uint16_t Kr[KC][KD + 8];   // k as given (bf16)
   __shared__ __attribute__((aligned(16))) uint16_t Qr[KC][KD + 8];   // q as given
+  __shared__ __attribute__((aligned(16))) uint16_t Vr[KC][KD + 8];   // v as given (right-hand side of the solve)
   __shared__ __attribute__((aligned(16))) float AT[KC][KC];          // AT[j][i] = A_ij (j < i)
-  __shared__ float rk[KC], rq[KC], bt[KC];                           // 1/|k|, 1/|q|, beta (0 for padded rows)
+  __shared__ float rk[KC], rq[KC], bt[KC];
+  __shared__ int steep[4];                                           // per 16-row block: total decay beyond exp(-80)                           // 1/|k|, 1/|q|, beta (0 for padded rows)
 
   const int n = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -93,17 +96,19 @@ __global__ __launch_bounds__(256) void kda_prep_kernel(KdaParams p) {
   auto row_off = [&](int r) -> int64_t { return (((int64_t)b * p.T + t0 + r) * p.H + h) * KD; };
 
   // ---- phase 0a: G = cumsum(g), EG = exp(g) ---------------------------------
+  if (tid < 4) steep[tid] = 0;
+  __syncthreads();
   {
     const int d = tid & 127, half = tid >> 7;
     float gv[32];
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       const int r = 32 * half + i;
-      float x = 0.f;
-      if (t0 + r < p.T) {
-        x = p.g_bf16 ? bf16lo_to_f32(((const uint16_t*)p.g)[row_off(r) + d]) : ((const float*)p.g)[row_off(r) + d];
-      }
-      gv[i] = x;
+      // Rows past the end re-read the last row (always valid) and are zeroed afterwards, so
+      // that the loads carry no branches and all go out together.
+      const int64_t off = row_off(min(r, p.T - 1 - t0)) + d;
+      const float x = p.g_bf16 ? bf16lo_to_f32(((const uint16_t*)p.g)[off]) : ((const float*)p.g)[off];
+      gv[i] = (t0 + r < p.T) ? x : 0.f;
     }
     float acc = 0.f;
 #pragma unroll
@@ -111,6 +116,13 @@ __global__ __launch_bounds__(256) void kda_prep_kernel(KdaParams p) {
       acc += gv[i];
       G[32 * half + i][d] = acc;
       EG[32 * half + i][d] = __expf(gv[i]);
+    }
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      float tot = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) tot += gv[16 * blk + i];
+      if (tot < -80.f) steep[2 * half + blk] = 1;   // same value from every writer
     }
     __syncthreads();
     if (half == 1) {
@@ -127,12 +139,13 @@ __global__ __launch_bounds__(256) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = r4 + 16 * i;
-    u32x4 kraw = {0, 0, 0, 0};
-    qraw[i] = kraw;
-    if (t0 + r < p.T) {
-      kraw = *reinterpret_cast<const u32x4*>(p.k + row_off(r) + 8 * cc);
-      qraw[i] = *reinterpret_cast<const u32x4*>(p.q + row_off(r) + 8 * cc);
-    }
+    const bool live = t0 + r < p.T;
+    const int64_t off = row_off(min(r, p.T - 1 - t0)) + 8 * cc;
+    const u32x4 zero4 = {0, 0, 0, 0};
+    u32x4 kraw = *reinterpret_cast<const u32x4*>(p.k + off);
+    u32x4 vraw = *reinterpret_cast<const u32x4*>(p.v + off);
+    qraw[i] = *reinterpret_cast<const u32x4*>(p.q + off);
+    if (!live) { kraw = zero4; vraw = zero4; qraw[i] = zero4; }
     float kf[8], qf[8];
     unpack8(kraw, kf);
     unpack8(qraw[i], qf);
@@ -146,9 +159,10 @@ __global__ __launch_bounds__(256) void kda_prep_kernel(KdaParams p) {
     if (cc == 0) {
       rk[r] = nk;
       rq[r] = rqv[i];
-      bt[r] = (t0 + r < p.T) ? p.beta[((int64_t)b * p.T + t0 + r) * p.H + h] : 0.f;
+      bt[r] = live ? p.beta[((int64_t)b * p.T + t0 + r) * p.H + h] : 0.f;
     }
     *reinterpret_cast<u32x4*>(&Kr[r][8 * cc]) = kraw;
+    *reinterpret_cast<u32x4*>(&Vr[r][8 * cc]) = vraw;
     *reinterpret_cast<u32x4*>(&Qr[r][8 * cc]) = qraw[i];
   }
   __syncthreads();
@@ -185,62 +199,78 @@ __global__ __launch_bounds__(256) void kda_prep_kernel(KdaParams p) {
     }
   }
 
-  // ---- phase 2a: off-diagonal 16x16 blocks of A and P on MFMA ----------------
-  {
+  // ---- phase 2a: 16x16 blocks of A and P on MFMA --------------------------------
+  // Block (I, J), J <= I: both operands are referenced to the row before block I, so the row
+  // factor exp(G_i - G_ref) is <= 1 and, for J < I, so is the column factor exp(G_ref - G_j).
+  // For a diagonal block (J == I) the column factor grows to exp(total decay of the block); the
+  // block takes this path only when that total stays below 80 (flag `steep` otherwise).
+  auto mfma_block = [&](int I, int J) {
     const int li = lane & 15, q4 = lane >> 4;
+    const int ref = 16 * I - 1;   // -1 for the first block: G_ref = 0
+    const int ri = 16 * I + li, rj = 16 * J + li;
+    f32x4 accA = {0.f, 0.f, 0.f, 0.f}, accP = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int d0 = 32 * m + 8 * q4;
+      float ki[8], qi[8], kj[8], ak[8], aq[8], bk[8];
+      unpack8(*reinterpret_cast<const u32x4*>(&Kr[ri][d0]), ki);
+      unpack8(*reinterpret_cast<const u32x4*>(&Qr[ri][d0]), qi);
+      unpack8(*reinterpret_cast<const u32x4*>(&Kr[rj][d0]), kj);
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+        const f32x4 gi = lds_f4(&G[ri][d0 + 4 * hf]), gj = lds_f4(&G[rj][d0 + 4 * hf]);
+        const f32x4 gr = (ref >= 0) ? lds_f4(&G[max(ref, 0)][d0 + 4 * hf]) : zero;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float fi = __expf(gi[e] - gr[e]);
+          const float fj = __expf(gr[e] - gj[e]);
+          ak[4 * hf + e] = ki[4 * hf + e] * fi;
+          aq[4 * hf + e] = qi[4 * hf + e] * fi;
+          bk[4 * hf + e] = kj[4 * hf + e] * fj;
+        }
+      }
+      const bf16x8 va = __builtin_bit_cast(bf16x8, pack8(ak));
+      const bf16x8 vq = __builtin_bit_cast(bf16x8, pack8(aq));
+      const bf16x8 vb = __builtin_bit_cast(bf16x8, pack8(bk));
+      accA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, vb, accA, 0, 0, 0);
+      accP = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vq, vb, accP, 0, 0, 0);
+    }
+    // accumulator: lane holds column j = 16J + li, rows i = 16I + 4*q4 + r
+    const int j = 16 * J + li;
+    const float rkj = rk[j];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = 16 * I + 4 * q4 + r;
+      if (j < i) AT[j][i] = bt[i] * rk[i] * rkj * accA[r];
+      const float pv = (j <= i) ? p.scale * rq[i] * rkj * accP[r] : 0.f;
+      p.Pm[(ci * KC + i) * KC + perm32(j)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
+    }
+  };
+  {
     for (int bi = wave; bi < 6; bi += 4) {
-      // blocks (I, J), I > J, in the order (1,0) (2,0) (2,1) (3,0) (3,1) (3,2)
+      // off-diagonal blocks in the order (1,0) (2,0) (2,1) (3,0) (3,1) (3,2)
       const int I = (bi == 0) ? 1 : (bi < 3 ? 2 : 3);
       const int J = (bi == 0) ? 0 : (bi < 3 ? bi - 1 : bi - 3);
-      const int ref = 16 * I - 1;
-      const int ri = 16 * I + li, rj = 16 * J + li;
-      f32x4 accA = {0.f, 0.f, 0.f, 0.f}, accP = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const int d0 = 32 * m + 8 * q4;
-        float ki[8], qi[8], kj[8], ak[8], aq[8], bk[8];
-        unpack8(*reinterpret_cast<const u32x4*>(&Kr[ri][d0]), ki);
-        unpack8(*reinterpret_cast<const u32x4*>(&Qr[ri][d0]), qi);
-        unpack8(*reinterpret_cast<const u32x4*>(&Kr[rj][d0]), kj);
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-          const f32x4 gi = lds_f4(&G[ri][d0 + 4 * hf]), gr = lds_f4(&G[ref][d0 + 4 * hf]), gj = lds_f4(&G[rj][d0 + 4 * hf]);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float fi = __expf(gi[e] - gr[e]);   // <= 1: row ri is at or after the reference row
-            const float fj = __expf(gr[e] - gj[e]);   // <= 1: row rj is before the reference row
-            ak[4 * hf + e] = ki[4 * hf + e] * fi;
-            aq[4 * hf + e] = qi[4 * hf + e] * fi;
-            bk[4 * hf + e] = kj[4 * hf + e] * fj;
-          }
-        }
-        const bf16x8 va = __builtin_bit_cast(bf16x8, pack8(ak));
-        const bf16x8 vq = __builtin_bit_cast(bf16x8, pack8(aq));
-        const bf16x8 vb = __builtin_bit_cast(bf16x8, pack8(bk));
-        accA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, vb, accA, 0, 0, 0);
-        accP = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vq, vb, accP, 0, 0, 0);
-      }
-      // accumulator: lane holds column j = 16J + li, rows i = 16I + 4*q4 + r
-      const int j = 16 * J + li;
-      const float rkj = rk[j];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = 16 * I + 4 * q4 + r;
-        AT[j][i] = bt[i] * rk[i] * rkj * accA[r];
-        const float pv = p.scale * rq[i] * rkj * accP[r];
-        p.Pm[(ci * KC + i) * KC + perm32(j)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
-      }
+      mfma_block(I, J);
     }
     // The state kernel reads P in 16x32 pieces; blocks (0,1) and (2,3) lie above the diagonal.
     if (wave >= 2) {
+      const int li = lane & 15, q4 = lane >> 4;
       const int I = (wave == 2) ? 0 : 2, J = I + 1;
 #pragma unroll
       for (int r = 0; r < 4; ++r) p.Pm[(ci * KC + 16 * I + 4 * q4 + r) * KC + perm32(16 * J + li)] = 0;
     }
   }
 
-  // ---- phase 2b: diagonal 16x16 blocks, fp32, running products of exp(g) ------
-  {
+  // ---- phase 2b: diagonal 16x16 blocks ----------------------------------------
+  // Wavefront w owns diagonal block w.  Usual case: the MFMA path above.  If some channel
+  // decays by more than exp(-80) across the block, the column factors of that path could
+  // overflow; the block is then accumulated in fp32 from running products of exp(g), where no
+  // exponent is ever positive.
+  if (!steep[wave]) {
+    mfma_block(wave, wave);
+  } else {
     const int I = wave, il = lane >> 2, dq = lane & 3;
     const int ri = 16 * I + il;
     float a[16], pp[16];
@@ -303,23 +333,29 @@ __global__ __launch_bounds__(256) void kda_prep_kernel(KdaParams p) {
       for (int i = 0; i < KC; ++i) X[i] = bt[i] * rk[i] * __expf(G[i][c]) * bf16lo_to_f32(Kr[i][c]);
     } else {
 #pragma unroll
-      for (int i = 0; i < KC; ++i) {
-        float vv = 0.f;
-        if (t0 + i < p.T) vv = bf16lo_to_f32(p.v[row_off(i) + (c - KD)]);
-        X[i] = bt[i] * vv;
-      }
+      for (int i = 0; i < KC; ++i) X[i] = bt[i] * bf16lo_to_f32(Vr[i][c - KD]);
     }
-    // Right-looking elimination: once X[j] is final, remove it from every later row.
+    // Right-looking elimination: once X[j] is final, remove it from every later row.  Row j of
+    // A^T is the same for all threads (an LDS broadcast); rows are fetched two steps ahead of
+    // their use so that the LDS latency is hidden behind the multiply-adds of the current step.
+    f32x4 arow[3][KC / 4];
+    auto fetch_row = [&](int j, f32x4* dst) {
+#pragma unroll
+      for (int i4 = 0; i4 < KC / 4; ++i4)
+        if (4 * i4 + 3 > j) dst[i4] = lds_f4(&AT[j][4 * i4]);
+    };
+    fetch_row(0, arow[0]);
+    fetch_row(1, arow[1]);
 #pragma unroll
     for (int j = 0; j < KC - 1; ++j) {
+      if (j + 2 < KC - 1) fetch_row(j + 2, arow[(j + 2) % 3]);
       const float xj = X[j];
 #pragma unroll
       for (int i4 = (j + 1) / 4; i4 < KC / 4; ++i4) {
-        const f32x4 av = lds_f4(&AT[j][4 * i4]);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int i = 4 * i4 + e;
-          if (i > j) X[i] = fmaf(-av[e], xj, X[i]);
+          if (i > j) X[i] = fmaf(-arow[j % 3][i4][e], xj, X[i]);
         }
       }
     }
@@ -371,19 +407,87 @@ __device__ __forceinline__ bf16x8 pack_acc2(const f32x4& t0, const f32x4& t1) {
   r.z = pack_bf16x2(t1[0], t1[1]); r.w = pack_bf16x2(t1[2], t1[3]);
   return __builtin_bit_cast(bf16x8, r);
 }
-__device__ __forceinline__ bf16x8 ldg_bf16x8(const uint16_t* p) {
-  return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(p));
+
+// LDS stage of the state kernel: everything of one chunk that does not depend on the value
+// column, copied with asynchronous global->LDS copies while the previous chunk is computed.
+// Rows are stored with their 16-byte chunks XOR-swizzled (chunk c of row r at position
+// c ^ f(r)) so that the 16-byte operand reads of 16 consecutive rows fall into 16 different
+// slots of the 256-byte bank window: f(r) = r & 15 for 256-byte rows, (r >> 1) & 7 for 128-byte
+// rows (two rows per window).
+constexpr int KSW = 2;                        // wavefronts per workgroup (16 value columns each)
+constexpr int kStageWn = 0;                   // [64][128] bf16
+constexpr int kStageQg = 16384;               // [64][128] bf16
+constexpr int kStageKtH = 32768;              // [128][64] bf16
+constexpr int kStageKtL = 49152;              // [128][64] bf16
+constexpr int kStagePm = 65536;               // [64][64]  bf16
+constexpr int kStageDec = 73728;              // [128] fp32
+constexpr int kStageBytes = 74240;
+
+typedef __attribute__((address_space(3))) const char* lds_cptr;
+__device__ __forceinline__ bf16x8 lds_bf16x8(lds_cptr p) {
+  return __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)p);
 }
 
-__global__ __launch_bounds__(64) void kda_state_kernel(KdaParams p) {
-  // Keep the 8 column slices of one (batch, head) on one XCD: they read the same chunk data.
+__global__ __launch_bounds__(64 * KSW, 1) void kda_state_kernel(KdaParams p) {
+  __shared__ __attribute__((aligned(1024))) char stage[2][kStageBytes];
+
+  // Keep the column groups of one (batch, head) on one XCD: they read the same chunk data.
   int vid = blockIdx.x;
   if ((gridDim.x & 7) == 0) vid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  constexpr int NSL = KD / KVS;
-  const int slice = vid % NSL, bh = vid / NSL;
+  constexpr int NGRP = KD / (KVS * KSW);
+  const int grp = vid % NGRP, bh = vid / NGRP;
   const int h = bh % p.H, b = bh / p.H;
-  const int lane = threadIdx.x, ln = lane & 15, q4 = lane >> 4;
-  const int vcol = KVS * slice + ln;
+  const int lane = threadIdx.x & 63, ln = lane & 15, q4 = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int vcol = KVS * (KSW * grp + wave) + ln;
+
+  // ---- copies of one chunk into a stage (this wavefront's share) --------------------------
+  const uint32_t stage_lds = lds_address(&stage[0][0]);
+  // 256-byte rows: a wavefront copy moves 4 rows; lane i lands at row i/16, position i%16.
+  // 128-byte rows: 8 rows per copy; lane i lands at row i/8, position i%8.
+  int src256[4], src128[2];   // source byte offsets inside a group of 16 rows, by (copy index & 3) / (& 1)
+#pragma unroll
+  for (int v = 0; v < 4; ++v) src256[v] = (4 * v + (lane >> 4)) * 256 + 16 * ((lane & 15) ^ ((4 * v + (lane >> 4)) & 15));
+#pragma unroll
+  for (int v = 0; v < 2; ++v) src128[v] = (8 * v + (lane >> 3)) * 128 + 16 * ((lane & 7) ^ ((4 * v + (lane >> 4)) & 7));
+
+  auto issue_copies = [&](int n, int st) {
+    const int64_t ci = (int64_t)bh * p.NC + n;
+    const uint32_t dst = stage_lds + st * kStageBytes;
+    const uint16_t* wn = p.Wn + ci * KC * KD;
+    const uint16_t* qg = p.Qg + ci * KC * KD;
+    const uint16_t* kh = p.KtH + ci * KD * KC;
+    const uint16_t* kl = p.KtL + ci * KD * KC;
+    const uint16_t* pm = p.Pm + ci * KC * KC;
+#pragma unroll
+    for (int j = wave; j < 16; j += KSW) {   // 16 copies of 4 rows x 256 B each
+      copy16_to_lds_async(wn + (j >> 2) * 2048, src256[j & 3], dst + kStageWn + j * 1024);
+      copy16_to_lds_async(qg + (j >> 2) * 2048, src256[j & 3], dst + kStageQg + j * 1024);
+    }
+#pragma unroll
+    for (int j = wave; j < 16; j += KSW) {   // 16 copies of 8 rows x 128 B each
+      copy16_to_lds_async(kh + (j >> 1) * 1024, src128[j & 1], dst + kStageKtH + j * 1024);
+      copy16_to_lds_async(kl + (j >> 1) * 1024, src128[j & 1], dst + kStageKtL + j * 1024);
+    }
+#pragma unroll
+    for (int j = wave; j < 8; j += KSW)
+      copy16_to_lds_async(pm + (j >> 1) * 1024, src128[j & 1], dst + kStagePm + j * 1024);
+    if (wave == 0 && lane < 32)
+      copy16_to_lds_async(reinterpret_cast<const uint16_t*>(p.dec + ci * KD), 16 * lane, dst + kStageDec);
+  };
+  auto copies_landed = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), visible to the compiler's wait-count model
+    asm volatile("" ::: "memory");
+  };
+
+  // ---- per-lane LDS read offsets (bytes, inside a stage) ------------------------------------
+  // A operand of a 16x16x32 MFMA: lane (row ln, k-group q4) reads chunk 4m + q4 of its row.
+  int rd256[4], rd128[2];
+#pragma unroll
+  for (int m = 0; m < 4; ++m) rd256[m] = ln * 256 + 16 * ((4 * m + q4) ^ ln);
+#pragma unroll
+  for (int m = 0; m < 2; ++m) rd128[m] = ln * 128 + 16 * ((4 * m + q4) ^ ((ln >> 1) & 7));
+  lds_cptr stage0 = (lds_cptr)&stage[0][0];
 
   // State tile dt: rows (key channels) 16*dt + 4*q4 + r, column vcol.
   f32x4 S[8];
@@ -394,13 +498,25 @@ __global__ __launch_bounds__(64) void kda_state_kernel(KdaParams p) {
       S[dt][r] = p.s0 ? p.s0[((int64_t)bh * KD + 16 * dt + 4 * q4 + r) * KD + vcol] : 0.f;
   }
 
+  // U0 (accumulator initial value of U) comes straight from global memory, one chunk ahead.
+  auto load_u0 = [&](int n, f32x4* dst) {
+    const float* src = p.U0T + (((int64_t)bh * p.NC + n) * KD + vcol) * KC + 4 * q4;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) dst[mt] = *reinterpret_cast<const f32x4*>(src + 16 * mt);
+  };
+  f32x4 u0c[4], u0n[4];
+  issue_copies(0, 0);
+  load_u0(0, u0c);
+  copies_landed();
+  __syncthreads();
+
   for (int n = 0; n < p.NC; ++n) {
-    const int64_t ci = (int64_t)bh * p.NC + n;
-    const uint16_t* Wn = p.Wn + ci * KC * KD;
-    const uint16_t* Qg = p.Qg + ci * KC * KD;
-    const uint16_t* Pm = p.Pm + ci * KC * KC;
-    const uint16_t* KtH = p.KtH + ci * KD * KC;
-    const uint16_t* KtL = p.KtL + ci * KD * KC;
+    const int st = n & 1;
+    if (n + 1 < p.NC) {
+      issue_copies(n + 1, st ^ 1);
+      load_u0(n + 1, u0n);
+    }
+    lds_cptr sb = stage0 + st * kStageBytes;
 
     bf16x8 Sb[4];
 #pragma unroll
@@ -410,10 +526,10 @@ __global__ __launch_bounds__(64) void kda_state_kernel(KdaParams p) {
     f32x4 U[4];
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
-      U[mt] = *reinterpret_cast<const f32x4*>(p.U0T + (ci * KD + vcol) * KC + 16 * mt + 4 * q4);
+      U[mt] = u0c[mt];
 #pragma unroll
       for (int m = 0; m < 4; ++m)
-        U[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ldg_bf16x8(Wn + (16 * mt + ln) * KD + 32 * m + 8 * q4), Sb[m], U[mt], 0, 0, 0);
+        U[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lds_bf16x8(sb + kStageWn + 4096 * mt + rd256[m]), Sb[m], U[mt], 0, 0, 0);
     }
     bf16x8 Uh[2], Ul[2];
 #pragma unroll
@@ -434,11 +550,11 @@ __global__ __launch_bounds__(64) void kda_state_kernel(KdaParams p) {
       f32x4 O = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int m = 0; m < 4; ++m)
-        O = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ldg_bf16x8(Qg + (16 * mt + ln) * KD + 32 * m + 8 * q4), Sb[m], O, 0, 0, 0);
+        O = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lds_bf16x8(sb + kStageQg + 4096 * mt + rd256[m]), Sb[m], O, 0, 0, 0);
 #pragma unroll
       for (int m = 0; m < 2; ++m) {
         if (32 * m <= 16 * mt + 15)   // columns up to the diagonal only
-          O = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ldg_bf16x8(Pm + (16 * mt + ln) * KC + 32 * m + 8 * q4), Uh[m], O, 0, 0, 0);
+          O = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lds_bf16x8(sb + kStagePm + 2048 * mt + rd128[m]), Uh[m], O, 0, 0, 0);
       }
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -450,18 +566,23 @@ __global__ __launch_bounds__(64) void kda_state_kernel(KdaParams p) {
     // S = exp(G_last) (.) S + Kt^T U, with both operands split into two bf16 terms.
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
-      const f32x4 dc = *reinterpret_cast<const f32x4*>(p.dec + ci * KD + 16 * dt + 4 * q4);
+      const f32x4 dc = *(const f32x4 __attribute__((address_space(3)))*)(sb + kStageDec + 4 * (16 * dt + 4 * q4));
 #pragma unroll
       for (int r = 0; r < 4; ++r) S[dt][r] *= dc[r];
 #pragma unroll
       for (int m = 0; m < 2; ++m) {
-        const bf16x8 ah = ldg_bf16x8(KtH + (16 * dt + ln) * KC + 32 * m + 8 * q4);
-        const bf16x8 al = ldg_bf16x8(KtL + (16 * dt + ln) * KC + 32 * m + 8 * q4);
+        const bf16x8 ah = lds_bf16x8(sb + kStageKtH + 2048 * dt + rd128[m]);
+        const bf16x8 al = lds_bf16x8(sb + kStageKtL + 2048 * dt + rd128[m]);
         S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, Uh[m], S[dt], 0, 0, 0);
         S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, Ul[m], S[dt], 0, 0, 0);
         S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, Uh[m], S[dt], 0, 0, 0);
       }
     }
+
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) u0c[mt] = u0n[mt];
+    copies_landed();
+    __syncthreads();
   }
 
   if (p.s_out != nullptr) {
@@ -539,7 +660,7 @@ extern "C" int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(kda_prep_kernel, dim3(p.NC, H, B), dim3(256), 0, s, p);
   DAISY_CHECK_LAUNCH("kda_prep_kernel");
-  hipLaunchKernelGGL(kda_state_kernel, dim3((unsigned)(B * H * (KD / KVS))), dim3(64), 0, s, p);
+  hipLaunchKernelGGL(kda_state_kernel, dim3((unsigned)(B * H * (KD / (KVS * KSW)))), dim3(64 * KSW), 0, s, p);
   DAISY_CHECK_LAUNCH("kda_state_kernel");
   return DAISY_OK;
 }

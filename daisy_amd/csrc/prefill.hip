@@ -77,22 +77,10 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* p) {
   return __builtin_bit_cast(u32x2, v);
 }
 
-// Asynchronous 16-byte global -> LDS copy that bypasses the vector registers
-// (global_load_lds_dwordx4): lane i of the wavefront deposits the 16 bytes at
-// gbase + byte_off at LDS address lds_addr + 16*i.  gbase and lds_addr are wavefront-uniform.
-// Issued as inline assembly so that the compiler does not serialise later LDS reads of the
-// OTHER buffer behind it; the caller waits with s_waitcnt vmcnt(0) before publishing the tile.
-__device__ __forceinline__ void copy16_to_lds_async(const uint16_t* gbase, int byte_off, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :: "v"(byte_off), "s"(gbase), "s"(lds_addr) : "memory");
-}
 typedef __attribute__((address_space(3))) const uint16_t* lds_u16_ptr;
 __device__ __forceinline__ u32x2 lds_read_tr16_as3(lds_u16_ptr p) {
   s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p);
   return __builtin_bit_cast(u32x2, v);
-}
-__device__ __forceinline__ uint32_t lds_address(const void* p) {
-  return (uint32_t)(size_t)(__attribute__((address_space(3))) const void*)p;
 }
 
 template <int D, bool ROPE_K>

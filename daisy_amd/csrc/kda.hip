@@ -79,15 +79,26 @@ __host__ __device__ constexpr int perm32_inv(int p) { return (p & ~0x1c) | ((p &
 
 __device__ __forceinline__ f32x4 lds_f4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 
-__global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
-  __shared__ __attribute__((aligned(16))) float G[KC][KD];           // inclusive running log-decay
-  __shared__ __attribute__((aligned(16))) float EG[KC][KD];          // exp(g) per row; later staging for Wn
+// Packed storage of A^T (AT[j][i] = A_ij, j < i): row j keeps the entries i >= at_first(j), the
+// multiple of 4 at or below j + 1, so that every row starts 16-byte aligned; rows follow each other.
+__host__ __device__ constexpr int at_first(int j) { return 4 * ((j + 1) >> 2); }
+__host__ __device__ constexpr int at_off(int j) {
+  const int m = (j + 1) >> 2;
+  const int before = (m >= 1) ? 192 + 256 * (m - 1) - 8 * m * (m - 1) : 0;
+  const int idx = (m == 0) ? j : ((j + 1) & 3);
+  return before + idx * (KC - 4 * m);
+}
+constexpr int kAtPacked = at_off(KC - 2) + 4;   // row 62 is the last one with entries
+
+__global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
+  __shared__ __attribute__((aligned(16))) float G[KC][KD];           // inclusive running log-decay; later staging for Wn
   __shared__ __attribute__((aligned(16))) uint16_t Kr[KC][KD + 8];   // k as given (bf16)
-  __shared__ __attribute__((aligned(16))) uint16_t Qr[KC][KD + 8];   // q as given
-  __shared__ __attribute__((aligned(16))) uint16_t Vr[KC][KD + 8];   // v as given (right-hand side of the solve)
-  __shared__ __attribute__((aligned(16))) float AT[KC][KC];          // AT[j][i] = A_ij (j < i)
-  __shared__ float rk[KC], rq[KC], bt[KC];
-  __shared__ int steep[4];                                           // per 16-row block: total decay beyond exp(-80)                           // 1/|k|, 1/|q|, beta (0 for padded rows)
+  __shared__ __attribute__((aligned(16))) uint16_t QV[KC][KD + 8];   // q as given; v as given once A and P are done
+  __shared__ __attribute__((aligned(16))) float ATp[kAtPacked];      // A^T, strictly lower part, rows packed (at_off)
+  __shared__ float rk[KC], rq[KC], bt[KC];                           // 1/|k|, 1/|q|, beta (0 for padded rows)
+  __shared__ int steep[4];                                           // per 16-row block: total decay beyond exp(-80)
+  auto& Qr = QV;
+  auto& Vr = QV;
 
   const int n = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -95,7 +106,7 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
   const int64_t ci = ((int64_t)b * p.H + h) * p.NC + n;
   auto row_off = [&](int r) -> int64_t { return (((int64_t)b * p.T + t0 + r) * p.H + h) * KD; };
 
-  // ---- phase 0a: G = cumsum(g), EG = exp(g) ---------------------------------
+  // ---- phase 0a: G = cumsum(g) -----------------------------------------------
   if (tid < 4) steep[tid] = 0;
   __syncthreads();
   {
@@ -115,7 +126,6 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
     for (int i = 0; i < 32; ++i) {
       acc += gv[i];
       G[32 * half + i][d] = acc;
-      EG[32 * half + i][d] = __expf(gv[i]);
     }
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
@@ -134,7 +144,7 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
 
   // ---- phase 0b: raw q, k to LDS, row norms, beta ---------------------------
   const int cc = tid & 15, r4 = tid >> 4;
-  u32x4 qraw[4];
+  u32x4 qraw[4], vraw[4];
   float rqv[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -143,9 +153,9 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
     const int64_t off = row_off(min(r, p.T - 1 - t0)) + 8 * cc;
     const u32x4 zero4 = {0, 0, 0, 0};
     u32x4 kraw = *reinterpret_cast<const u32x4*>(p.k + off);
-    u32x4 vraw = *reinterpret_cast<const u32x4*>(p.v + off);
+    vraw[i] = *reinterpret_cast<const u32x4*>(p.v + off);
     qraw[i] = *reinterpret_cast<const u32x4*>(p.q + off);
-    if (!live) { kraw = zero4; vraw = zero4; qraw[i] = zero4; }
+    if (!live) { kraw = zero4; vraw[i] = zero4; qraw[i] = zero4; }
     float kf[8], qf[8];
     unpack8(kraw, kf);
     unpack8(qraw[i], qf);
@@ -162,7 +172,6 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
       bt[r] = live ? p.beta[((int64_t)b * p.T + t0 + r) * p.H + h] : 0.f;
     }
     *reinterpret_cast<u32x4*>(&Kr[r][8 * cc]) = kraw;
-    *reinterpret_cast<u32x4*>(&Vr[r][8 * cc]) = vraw;
     *reinterpret_cast<u32x4*>(&Qr[r][8 * cc]) = qraw[i];
   }
   __syncthreads();
@@ -242,7 +251,7 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int i = 16 * I + 4 * q4 + r;
-      if (j < i) AT[j][i] = bt[i] * rk[i] * rkj * accA[r];
+      if (j < i) ATp[at_off(j) + i - at_first(j)] = bt[i] * rk[i] * rkj * accA[r];
       const float pv = (j <= i) ? p.scale * rq[i] * rkj * accP[r] : 0.f;
       p.Pm[(ci * KC + i) * KC + perm32(j)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
     }
@@ -291,7 +300,11 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
         unpack8(*reinterpret_cast<const u32x4*>(&Kr[rj][d0]), kj);
         if (j < 15) {
           // E = exp(G_i - G_j) for j < i: multiply in exp(g) of row j+1; rows j >= i restart at 1.
-          const f32x4 e0 = lds_f4(&EG[rj + 1][d0]), e1 = lds_f4(&EG[rj + 1][d0 + 4]);
+          const f32x4 ga0 = lds_f4(&G[rj + 1][d0]), ga1 = lds_f4(&G[rj + 1][d0 + 4]);
+          const f32x4 gb0 = lds_f4(&G[rj][d0]), gb1 = lds_f4(&G[rj][d0 + 4]);
+          f32x4 e0, e1;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { e0[e] = __expf(ga0[e] - gb0[e]); e1[e] = __expf(ga1[e] - gb1[e]); }
           const bool live = j < il;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -315,7 +328,7 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
       if ((j & 3) == dq) {
         const int rj = 16 * I + j;
         const float rkj = rk[rj];
-        if (j < il) AT[rj][ri] = bi * rkj * av;
+        if (j < il) ATp[at_off(rj) + ri - at_first(rj)] = bi * rkj * av;
         pv = (j <= il) ? qs * rkj * pv : 0.f;
         p.Pm[(ci * KC + ri) * KC + perm32(rj)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
       }
@@ -323,7 +336,32 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
   }
   __syncthreads();
 
-  // ---- phase 3: forward substitution (I + A) X = diag(beta) [exp(G) K | V] ----
+  // Q is no longer needed: V takes its place in LDS (right-hand side of the solve).
+#pragma unroll
+  for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&Vr[r4 + 16 * i][8 * cc]) = vraw[i];
+
+  // ---- phase 3: (exp(G_last - G) k/|k|)^T as two bf16 terms, position permuted ----
+  {
+    const int d = tid & 127, gh = tid >> 7;
+    const float glast = G[KC - 1][d];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int g8 = 4 * gh + i;   // group of 8 stored positions
+      float hi[8], lo[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int pos = perm32_inv(8 * g8 + e);
+        const float val = __expf(glast - G[pos][d]) * bf16lo_to_f32(Kr[pos][d]) * rk[pos];
+        hi[e] = round_bf16(val);
+        lo[e] = val - hi[e];
+      }
+      *reinterpret_cast<u32x4*>(p.KtH + (ci * KD + d) * KC + 8 * g8) = pack8(hi);
+      *reinterpret_cast<u32x4*>(p.KtL + (ci * KD + d) * KC + 8 * g8) = pack8(lo);
+    }
+  }
+  __syncthreads();   // V is in place
+
+  // ---- phase 4: forward substitution (I + A) X = diag(beta) [exp(G) K | V] ----
   // One thread per right-hand-side column; the column lives in registers.
   {
     float X[KC];
@@ -335,31 +373,31 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
       for (int i = 0; i < KC; ++i) X[i] = bt[i] * bf16lo_to_f32(Vr[i][c - KD]);
     }
+    __syncthreads();   // every thread has read G: its space becomes the staging tile for Wn
     // Right-looking elimination: once X[j] is final, remove it from every later row.  Row j of
-    // A^T is the same for all threads (an LDS broadcast); rows are fetched two steps ahead of
+    // A^T is the same for all threads (an LDS broadcast); rows are fetched one step ahead of
     // their use so that the LDS latency is hidden behind the multiply-adds of the current step.
-    f32x4 arow[3][KC / 4];
-    auto fetch_row = [&](int j, f32x4* dst) {
+    f32x4 arow[2][KC / 4];
 #pragma unroll
-      for (int i4 = 0; i4 < KC / 4; ++i4)
-        if (4 * i4 + 3 > j) dst[i4] = lds_f4(&AT[j][4 * i4]);
-    };
-    fetch_row(0, arow[0]);
-    fetch_row(1, arow[1]);
+    for (int i4 = 0; i4 < KC / 4; ++i4) arow[0][i4] = lds_f4(&ATp[at_off(0) + 4 * i4 - at_first(0)]);
 #pragma unroll
     for (int j = 0; j < KC - 1; ++j) {
-      if (j + 2 < KC - 1) fetch_row(j + 2, arow[(j + 2) % 3]);
+      if (j + 1 < KC - 1) {
+#pragma unroll
+        for (int i4 = (j + 2) / 4; i4 < KC / 4; ++i4)
+          arow[(j + 1) & 1][i4] = lds_f4(&ATp[at_off(j + 1) + 4 * i4 - at_first(j + 1)]);
+      }
       const float xj = X[j];
 #pragma unroll
       for (int i4 = (j + 1) / 4; i4 < KC / 4; ++i4) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int i = 4 * i4 + e;
-          if (i > j) X[i] = fmaf(-arow[j % 3][i4][e], xj, X[i]);
+          if (i > j) X[i] = fmaf(-arow[j & 1][i4][e], xj, X[i]);
         }
       }
     }
-    uint16_t* Wst = reinterpret_cast<uint16_t*>(&EG[0][0]);   // [64][128] bf16 staging (EG is dead)
+    uint16_t* Wst = reinterpret_cast<uint16_t*>(&G[0][0]);   // [64][128] bf16 staging
     if (c < KD) {
       const int pc = perm32(c);
 #pragma unroll
@@ -380,25 +418,6 @@ __global__ __launch_bounds__(256, 1) void kda_prep_kernel(KdaParams p) {
     }
   }
 
-  // ---- phase 4: (exp(G_last - G) k/|k|)^T as two bf16 terms, position permuted ----
-  {
-    const int d = tid & 127, gh = tid >> 7;
-    const float glast = G[KC - 1][d];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int g8 = 4 * gh + i;   // group of 8 stored positions
-      float hi[8], lo[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int pos = perm32_inv(8 * g8 + e);
-        const float val = __expf(glast - G[pos][d]) * bf16lo_to_f32(Kr[pos][d]) * rk[pos];
-        hi[e] = round_bf16(val);
-        lo[e] = val - hi[e];
-      }
-      *reinterpret_cast<u32x4*>(p.KtH + (ci * KD + d) * KC + 8 * g8) = pack8(hi);
-      *reinterpret_cast<u32x4*>(p.KtL + (ci * KD + d) * KC + 8 * g8) = pack8(lo);
-    }
-  }
 }
 
 __device__ __forceinline__ bf16x8 pack_acc2(const f32x4& t0, const f32x4& t1) {

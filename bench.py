@@ -3,6 +3,10 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu]
 
+NAME is one of prefill | long | decode | kda | copy; "copy" runs a plain 1 GiB
+device copy and nothing else (the known-size kernel against which the HBM
+counters FETCH_SIZE / WRITE_SIZE are calibrated under rocprofv3 --pmc).
+
 A "step" is one pass of the headline workload: windowed prefill attention with
 fused RoPE on B=8, T=4096, H=8, D=128, window 1024 (bf16), inputs resident in
 HBM.  One JSON line is printed.  `value` is the attention throughput of that
@@ -125,6 +129,21 @@ def cpu_prefill_baseline(q, k, v, cos, sin, W, sample):
             "kind": "port", "sample": sample, "seconds": dt}
 
 
+# HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# (profiles/prefill_pipe_kernel_c2_hbm_traffic.txt), each scaled by the factor the same counter
+# shows for the 1 GiB copy of `--only copy`.  None until measured.
+PREFILL_C2_TRAFFIC_BYTES = None
+
+
+def bench_copy(steps, warmup):
+    """A plain device-to-device copy of 1 GiB (reads 2^30 bytes, writes 2^30 bytes per launch)."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda:0").fill_(1)
+    dst = torch.empty_like(src)
+    ms = time_gpu(lambda: dst.copy_(src), steps, warmup)
+    return {"workload": "copy_1GiB", "bytes_read": n, "bytes_written": n, "ms": ms, "gbs": 2 * n / ms / 1e6}
+
+
 def bench_prefill_c3(steps, warmup):
     """Config 3: B1 T65536 H16 D128, q/k/v ~ N(0,1) already rotated; window 2048 and full causal."""
     from daisy_amd import ops
@@ -232,7 +251,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", default=None, help="prefill | long | decode | kda (default: all)")
+    ap.add_argument("--only", default=None, help="prefill | long | decode | kda | copy (default: all but copy)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -243,6 +262,9 @@ def main():
     from daisy_amd import _lib
     _lib.load()
 
+    if args.only == "copy":
+        print(json.dumps(bench_copy(args.steps, args.warmup)))
+        return
     want = lambda name: args.only in (None, name)
     cpu = not args.no_cpu
     extra = {}
@@ -270,8 +292,8 @@ def main():
     }
     if head is not None:
         line["roofline"] = {"bound": "mfma", "achieved": head["tflops_kernel"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                            "frac": head["frac_of_peak_kernel"], "traffic": None,
-                            "kernel": "prefill_mfma_kernel<128,false>", "ms": head["ms_kernel"]}
+                            "frac": head["frac_of_peak_kernel"], "traffic": PREFILL_C2_TRAFFIC_BYTES,
+                            "kernel": "prefill_pipe_kernel<128>", "ms": head["ms_kernel"]}
         if "cpu_baseline" in head:
             line["cpu_baseline"] = head.pop("cpu_baseline")
         extra["prefill_c2"] = head

@@ -47,6 +47,7 @@ struct PrefillParams {
   uint16_t* o; int64_t o_sb, o_st, o_sh;
   uint16_t* k_out; int64_t ko_sb, ko_st, ko_sh;
   int B, T, H, D, window, nqb;
+  int n_light;   // leading query blocks that see fewer keys than a full window (0 = order by block only)
   float scale_log2e;
 };
 
@@ -58,6 +59,28 @@ __device__ __forceinline__ int row_lo(const PrefillParams& p, int q) {
   int lo = (p.window > 0) ? max(q - p.window + 1, 0) : 0;
   if (p.doc_start != nullptr) lo = max(lo, p.doc_start[q]);
   return lo;
+}
+
+// Workgroup -> (batch*head, query block).  Workgroups are dealt round-robin to the 8 XCDs, each
+// with its own L2: an XCD is given a contiguous group of (batch, head) pairs so that the query
+// blocks sharing K/V rows share an L2.  Inside a group the blocks with a full window of keys
+// come first, pair by pair from the last block down; the n_light shorter blocks at the start of
+// every sequence come last, longest first across the whole group, and fill the tail of the grid.
+__device__ __forceinline__ void workgroup_to_block(const PrefillParams& p, int& bh, int& qb) {
+  const int nbh = p.B * p.H;
+  int group = 0, gsize = nbh, idx = blockIdx.x;
+  if ((nbh & 7) == 0) { group = blockIdx.x & 7; gsize = nbh >> 3; idx = blockIdx.x >> 3; }
+  const int n_full = p.nqb - p.n_light;
+  int local;
+  if (idx < gsize * n_full) {
+    local = idx / n_full;
+    qb = p.nqb - 1 - idx % n_full;
+  } else {
+    const int j = idx - gsize * n_full;
+    qb = p.n_light - 1 - j / gsize;
+    local = j % gsize;
+  }
+  bh = group * gsize + local;
 }
 
 // Exchange with the lane that holds the other half of this query's keys.
@@ -109,17 +132,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lq = lane & 31, lh = lane >> 5;
 
-  // ---- workgroup -> (batch, head, query block); XCD-aware ------------------
-  // Workgroups are dealt round-robin to the 8 XCDs.  Give each XCD a contiguous
-  // run of (batch, head, query block) ids so that the query blocks sharing K/V
-  // rows also share an L2, and start with the heaviest query blocks.
-  int vid = blockIdx.x;
-  {
-    const int nwg = gridDim.x;
-    if ((nwg & 7) == 0) vid = (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3);
-  }
-  const int qb = p.nqb - 1 - (vid % p.nqb);
-  const int bh = vid / p.nqb;
+  int bh, qb;
+  workgroup_to_block(p, bh, qb);
   const int h = bh % p.H, b = bh / p.H;
 
   const int q0 = qb * kBM;
@@ -475,13 +489,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lq = lane & 31, lh = lane >> 5;
 
-  int vid = blockIdx.x;
-  {
-    const int nwg = gridDim.x;
-    if ((nwg & 7) == 0) vid = (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3);
-  }
-  const int qb = p.nqb - 1 - (vid % p.nqb);
-  const int bh = vid / p.nqb;
+  int bh, qb;
+  workgroup_to_block(p, bh, qb);
   const int h = bh % p.H, b = bh / p.H;
 
   const int q0 = qb * kBM;
@@ -646,14 +655,25 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) sc[sb][r] = 0.f;
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
+    // K fragments are read KPF contraction slices ahead of the MFMAs that use them.
+    constexpr int KPF = 3;
+    bf16x8 ka[KPF][2];
+    auto read_k = [&](int s) {
       lds_u16_ptr kp = k_rd[s] + kofs;
 #pragma unroll
-      for (int sb = 0; sb < 2; ++sb) {
-        const bf16x8 a = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(kp + 32 * sb * D));
-        sc[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[s], sc[sb], 0, 0, 0);
-      }
+      for (int sb = 0; sb < 2; ++sb)
+        ka[s % KPF][sb] = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(kp + 32 * sb * D));
+    };
+#pragma unroll
+    for (int s = 0; s < KPF; ++s) read_k(s);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb)
+        sc[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[s % KPF][sb], qreg[s], sc[sb], 0, 0, 0);
+      if (s + KPF < NS) read_k(s + KPF);
+      __builtin_amdgcn_sched_barrier(0);
     }
     apply_pending_rescale();
     pv_product(vofs);
@@ -915,6 +935,7 @@ extern "C" int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
   p.ko_sb = k_out ? k_out_strides[0] : 0; p.ko_st = k_out ? k_out_strides[1] : 0; p.ko_sh = k_out ? k_out_strides[2] : 0;
   p.B = B; p.T = T; p.H = H; p.D = D; p.window = window;
   p.nqb = (T + kBM - 1) / kBM;
+  p.n_light = (window > 0 && window < T) ? min((window - 1 + kBM - 1) / kBM, p.nqb) : 0;
   p.scale_log2e = scale * kLog2e;
   hipStream_t s = (hipStream_t)stream;
 

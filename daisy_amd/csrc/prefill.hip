@@ -47,6 +47,7 @@ struct PrefillParams {
   uint16_t* o; int64_t o_sb, o_st, o_sh;
   uint16_t* k_out; int64_t ko_sb, ko_st, ko_sh;
   int B, T, H, D, window, nqb;
+  int period;    // tiles in a full window's range (0 = no window): the rotation period of the tile order
   int n_light;   // leading query blocks that see fewer keys than a full window (0 = order by block only)
   float scale_log2e;
 };
@@ -507,6 +508,18 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
   const int tw_lo = lo_w_min / kBN;
   const int tw_hi = (qw0 < p.T) ? q_w_max / kBN : -1;
 
+  // Tiles are visited in rotated order: start at the tile whose index is a multiple of the
+  // window's tile count (one exists in every full range), run up to t_hi, wrap to t_lo.  The
+  // online softmax does not care about the order, and the query blocks of one (batch, head)
+  // that run side by side then read the same K/V tile at the same step, so one fetch into the
+  // L2 serves all of them.  With no window every range starts at tile 0 and nothing is rotated.
+  const int n_tiles = t_hi - t_lo + 1;
+  int t_first = t_lo;
+  if (p.period > 0) {
+    const int c = (t_lo + p.period - 1) / p.period * p.period;
+    if (c <= t_hi) t_first = c;
+  }
+
   const uint16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
   const uint16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
 
@@ -547,7 +560,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
   };
 
   // The first copy goes out before anything else so that its latency overlaps the Q loads.
-  copy_k(t_lo, 0);
+  copy_k(t_first, 0);
   // V buffer 1 is read (times a zero P) before anything was copied into it: clear it.
   {
     u32x4 z = {0, 0, 0, 0};
@@ -608,13 +621,14 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
   float alpha_pend = 1.f;          // rescale of O asked for by the last softmax, not applied yet
   bool rescale_pend = false;       // wave-uniform
   bf16x8 pfrag[2][2];              // P of the previous tile (B operands of the delayed product)
-  {
+  auto clear_pfrag = [&]() {
     const u32x4 z = {0, 0, 0, 0};
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int m = 0; m < 2; ++m) pfrag[sb][m] = __builtin_bit_cast(bf16x8, z);
-  }
+  };
+  clear_pfrag();
 
   auto apply_pending_rescale = [&]() {
     if (rescale_pend) {
@@ -731,21 +745,28 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
   copies_landed();
   __syncthreads();
 
-  // Iteration `tile`, parity par = (tile - t_lo) & 1: K(tile) is in K buffer par and V(tile-1)
-  // in V buffer par^1.  The tiles of a wavefront come in three runs -- masked ones at the window
-  // / document edge, fully visible ones, masked ones at the diagonal -- and each run has its own
-  // loop, so that the hot loop over fully visible tiles contains one code path only.
-  auto generic_tiles = [&](int from, int to) {
-    for (int tile = from; tile <= to; ++tile) {
-      const int par = (tile - t_lo) & 1;
-      if (tile + 1 <= t_hi) copy_k(tile + 1, par ^ 1);
-      copy_v(tile, par);
+  // Step n (parity par = n & 1) works on tile(n): K(tile(n)) is in K buffer par and V of the
+  // previous step's tile in V buffer par^1.  Within each of the two runs of the rotated order
+  // the tiles of a wavefront come as masked ones at the window / document edge, fully visible
+  // ones, masked ones at the diagonal; the fully visible ones get a loop with one code path.
+  bool pending = false;   // wave-uniform: P of the last tile has not been multiplied into O yet
+  auto start_copies = [&](int tile, int n) {
+    if (n + 1 < n_tiles) copy_k(tile == t_hi ? t_lo : tile + 1, (n & 1) ^ 1);
+    copy_v(tile, n & 1);
+  };
+  auto generic_tiles = [&](int from, int to, int n) {
+    for (int tile = from; tile <= to; ++tile, ++n) {
+      const int par = n & 1;
+      start_copies(tile, n);
       if (tile >= tw_lo && tile <= tw_hi) {
         wave_tile(tile, par, std::true_type{});
-      } else if (tile == tw_hi + 1 && tw_hi >= tw_lo) {
-        // drain: the product of this wavefront's last tile
+        pending = true;
+      } else if (pending) {
+        // the product of this wavefront's last tile, before its V buffer is reused
         apply_pending_rescale();
         pv_product((par ^ 1) * TILE);
+        clear_pfrag();   // the wavefront may become active again after the wrap
+        pending = false;
       }
       copies_landed();
       __syncthreads();
@@ -755,21 +776,28 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
   // the first row.
   int c_lo = max((lo_w_max + kBN - 1) / kBN, max(tw_lo, t_lo));
   int c_hi = min((q_w_min + 1) / kBN - 1, min(tw_hi, t_hi));
-  if (c_hi < c_lo) { c_lo = t_hi + 1; c_hi = t_hi; }   // none: everything runs in the first generic loop
-  generic_tiles(t_lo, c_lo - 1);
-  for (int tile = c_lo; tile <= c_hi; ++tile) {
-    const int par = (tile - t_lo) & 1;
-    if (tile + 1 <= t_hi) copy_k(tile + 1, par ^ 1);
-    copy_v(tile, par);
-    wave_tile(tile, par, std::false_type{});
-    copies_landed();
-    __syncthreads();
+  if (c_hi < c_lo) { c_lo = t_hi + 1; c_hi = t_hi; }   // none: everything runs in the generic loops
+#pragma nounroll
+  for (int run = 0; run < 2; ++run) {
+    const int a = run == 0 ? t_first : t_lo;
+    const int b = run == 0 ? t_hi : t_first - 1;
+    const int n0 = run == 0 ? 0 : t_hi - t_first + 1;
+    generic_tiles(a, min(b, c_lo - 1), n0);
+    const int ca = max(a, c_lo), cb = min(b, c_hi);
+    for (int tile = ca, n = n0 + ca - a; tile <= cb; ++tile, ++n) {
+      const int par = n & 1;
+      start_copies(tile, n);
+      wave_tile(tile, par, std::false_type{});
+      pending = true;
+      copies_landed();
+      __syncthreads();
+    }
+    const int g = max(a, c_hi + 1);
+    generic_tiles(g, b, n0 + g - a);
   }
-  generic_tiles(c_hi + 1, t_hi);
-  // Wavefronts whose range ends with the workgroup's last tile drain after the loop.
-  if (tw_hi == t_hi && tw_hi >= tw_lo) {
+  if (pending) {
     apply_pending_rescale();
-    pv_product(((t_hi - t_lo) & 1) * TILE);
+    pv_product(((n_tiles - 1) & 1) * TILE);
   }
 
   const float l_tot = pair_sum(l_run);
@@ -935,6 +963,7 @@ extern "C" int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
   p.ko_sb = k_out ? k_out_strides[0] : 0; p.ko_st = k_out ? k_out_strides[1] : 0; p.ko_sh = k_out ? k_out_strides[2] : 0;
   p.B = B; p.T = T; p.H = H; p.D = D; p.window = window;
   p.nqb = (T + kBM - 1) / kBM;
+  p.period = (window > 0 && window < T) ? (kBM - 1) / kBN + 1 + (window - 1 + kBN - 1) / kBN : 0;
   p.n_light = (window > 0 && window < T) ? min((window - 1 + kBM - 1) / kBM, p.nqb) : 0;
   p.scale_log2e = scale * kLog2e;
   hipStream_t s = (hipStream_t)stream;

@@ -76,8 +76,11 @@ def test_prefill_matches_oracle_with_documents_and_ve(receives_ve):
     assert_close_bf16(v, v_ref, "v")
     # the reference's dense additive mask is accepted too and means the same thing
     dense = oracle.build_attn_mask(ids, W, 3).to(DEV)
+    # (per-row lower bounds instead of a window: the kernel visits the key tiles in another order,
+    # so the two results agree to rounding, not bit for bit)
     y2 = attn(x.to(DEV), None if ve is None else ve.to(DEV), attn_mask=dense)
-    assert torch.equal(y2, y)
+    assert_close_bf16(y2, y, "dense mask vs descriptor", max_abs=8e-3, mean_abs=2e-4)
+    assert_close_bf16(y2, y_ref, "y (dense mask)")
 
 
 @pytest.mark.parametrize("T,W", [(128, 128), (131, 128), (70, 16)])

@@ -24,7 +24,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from . import ops
-from .functional import init_linear, norm
+from .functional import NORM_EPS_BF16, init_linear, norm
 from .kv_cache import RingContext
 
 
@@ -160,8 +160,12 @@ class CausalSelfAttention(nn.Module):
         else:
             self.g_ve = None
         self.debug_logging = False
-        # Set to True to rotate keys while they are staged into LDS instead of in a pre-pass.
+        # Set to True to rotate keys while they are staged into LDS instead of in a pre-pass
+        # (only used when fused_prep is off).
         self.rotate_k_in_kernel = False
+        # Norm + RoPE + ve mix in one streaming kernel ahead of attention (bf16 weights only);
+        # False keeps norm / mix in PyTorch and rotates inside the attention call.
+        self.fused_prep = True
 
     def reset_history(self):
         self.last_q = None
@@ -188,9 +192,34 @@ class CausalSelfAttention(nn.Module):
         # use) are rounded here and the result is widened again by the caller.
         return t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16)
 
+    def _fused_prep_ok(self) -> bool:
+        # The one-pass norm + RoPE + ve-mix kernel works on bf16 rows of 64 or 128 channels.
+        return self.fused_prep and self.qkvo_w.dtype == torch.bfloat16 and self.head_dim in (64, 128)
+
+    def _project_qkv_fused(self, x: Tensor, ve: Optional[Tensor], pos0: int):
+        """QKV projection, then norm + RoPE (rows ``pos0 + t``) + ve mix in one kernel; ``[B, T, H, D]``."""
+        B, T = x.size(0), x.size(1)
+        x = x.to(self.qkvo_w.dtype)
+        qkv = F.linear(x, self.qkvo_w[:3].flatten(end_dim=1)).view(B, T, 3 * self.num_heads, self.head_dim)
+        q, k, v = qkv.chunk(3, dim=-2)
+        gate = None
+        if self.receives_ve:
+            torch._assert(ve is not None, "ve must be provided when receives_ve=True")
+            ve = ve.to(torch.bfloat16).view(B, T, self.num_heads, self.head_dim)
+            gate = torch.sigmoid(self.g_ve.detach()).to(torch.bfloat16).float().reshape(1)
+        else:
+            ve = None
+        cos, sin = self.rotary._get_cos_sin(pos0 + T)
+        return ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, pos0=pos0, ve=ve, gate=gate)
+
     def _attend(self, x: Tensor, ve: Optional[Tensor], attn_mask: MaskLike):
         B, T = x.size(0), x.size(1)
         mask = _as_window_mask(attn_mask)
+        if self._fused_prep_ok():
+            q, k_rot, v = self._project_qkv_fused(x, ve, 0)
+            o, _ = ops.prefill_attention(q, k_rot, v, window=mask.window, scale=self.attn_scale, doc_start=mask.doc_start)
+            y = F.linear(o.view(B, T, self.m_dim), self.qkvo_w[3])
+            return y, k_rot, v
         q, k, v = self._project_qkv(x)
         dtype = q.dtype
         v = self._mix_ve(v, ve)
@@ -232,11 +261,18 @@ class CausalSelfAttention(nn.Module):
         """
         B = x.size(0)
         torch._assert(x.size(1) == 1, "step() requires single position only")
-        q, k, v = self._project_qkv(x)
-        dtype = q.dtype
-        v = self._mix_ve(v, ve)
-        cos, sin = self.rotary._get_cos_sin(pos + 1)
-        cos_row, sin_row = cos[pos], sin[pos]
+        fused = self._fused_prep_ok()
+        if fused:
+            # q and k come back rotated: the decode kernel is told not to rotate again.
+            q, k, v = self._project_qkv_fused(x, ve, pos)
+            dtype = q.dtype
+            cos_row = sin_row = None
+        else:
+            q, k, v = self._project_qkv(x)
+            dtype = q.dtype
+            v = self._mix_ve(v, ve)
+            cos, sin = self.rotary._get_cos_sin(pos + 1)
+            cos_row, sin_row = cos[pos], sin[pos]
         qk, kk, vk = (self._kernel_dtype(t)[:, 0] for t in (q, k, v))  # [B, H, D]
 
         ring = k_ctx if isinstance(k_ctx, RingContext) else None
@@ -255,9 +291,12 @@ class CausalSelfAttention(nn.Module):
         else:
             n = k_ctx.size(1)
             r = n if window is None else min(n, max(window - 1, 0))
-            k_new = _apply_rope(self._kernel_dtype(k), cos_row[None, None, None, :], sin_row[None, None, None, :])
-            v_new = self._kernel_dtype(v)
-            q_rot = _apply_rope(self._kernel_dtype(q), cos_row[None, None, None, :], sin_row[None, None, None, :])
+            if fused:
+                k_new, v_new, q_rot = k, v, q
+            else:
+                k_new = _apply_rope(self._kernel_dtype(k), cos_row[None, None, None, :], sin_row[None, None, None, :])
+                v_new = self._kernel_dtype(v)
+                q_rot = _apply_rope(self._kernel_dtype(q), cos_row[None, None, None, :], sin_row[None, None, None, :])
             if r > 0:
                 kc = self._kernel_dtype(k_ctx)[:, n - r:n].transpose(1, 2)  # [B, H, r, D] view
                 vc = self._kernel_dtype(v_ctx)[:, n - r:n].transpose(1, 2)

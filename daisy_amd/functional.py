@@ -14,6 +14,12 @@ def norm(x: Tensor) -> Tensor:
     return F.rms_norm(x, (x.size(-1),))
 
 
+# What ``F.rms_norm(x, (D,))`` adds to mean(x^2) when no eps is passed: the machine epsilon of
+# the accumulation type, which is fp32 for bf16 inputs (torch 2.10).  The fused pre-attention
+# kernel takes the same value so that it rounds like ``norm``.
+NORM_EPS_BF16 = torch.finfo(torch.float32).eps
+
+
 @torch.no_grad()
 def init_linear(w: Tensor) -> Tensor:
     """Uniform init with std 0.5 / sqrt(fan_in) (models/daisy/functional.py:10-14)."""

@@ -210,3 +210,59 @@ def kda_gate_fwd(g: torch.Tensor, A_log: torch.Tensor, head_k_dim: int,
                                     float(beta), float(threshold), _lib.current_stream(dev))
     _lib.check(rc, "daisy_kda_gate_fwd")
     return out
+
+
+def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
+             cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, pos0: int = 0,
+             ve: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+             q_out: Optional[torch.Tensor] = None, k_out: Optional[torch.Tensor] = None,
+             v_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """RMS norm of q, k, v + RoPE of q, k at rows ``pos0 + t`` + ``gate*v + (1-gate)*ve`` in one pass.
+
+    ``q``, ``k``, ``v`` (and ``ve``) are bf16 ``[B, T, H, D]`` tensors or views with a
+    contiguous last dim; ``gate`` is a one-element fp32 tensor holding the (bf16-rounded)
+    sigmoid of the gate logit.  Outputs default to new contiguous ``[B, T, H, D]`` tensors;
+    any strided bf16 ``[B, T, H, D]`` view may be passed instead.
+    """
+    dev = _lib.require_gpu(q, k, v, ve, gate, cos, sin, q_out, k_out, v_out)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_bf16(name, t, 4)
+    B, T, H, D = q.shape
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError(f"q, k, v shapes differ: {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    if (cos is None) != (sin is None):
+        raise ValueError("cos and sin must be given together")
+    if cos is not None:
+        for name, t in (("cos", cos), ("sin", sin)):
+            if t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != D // 2 or not t.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous fp32 [rows, {D // 2}] table, got {tuple(t.shape)} {t.dtype}")
+            torch._assert(pos0 + T <= t.shape[0], f"Rotary buffers too small {t.shape[0]} < {pos0 + T}")
+    if (ve is None) != (gate is None):
+        raise ValueError("ve and gate must be given together")
+    if ve is not None:
+        _check_bf16("ve", ve, 4)
+        if ve.shape != q.shape:
+            raise ValueError(f"ve must have shape {tuple(q.shape)}, got {tuple(ve.shape)}")
+        if gate.dtype != torch.float32 or gate.numel() != 1:
+            raise ValueError("gate must be a one-element fp32 tensor")
+    outs = []
+    for name, t in (("q_out", q_out), ("k_out", k_out), ("v_out", v_out)):
+        if t is None:
+            t = torch.empty((B, T, H, D), dtype=torch.bfloat16, device=dev)
+        else:
+            _check_bf16(name, t, 4)
+            if t.shape != q.shape:
+                raise ValueError(f"{name} must have shape {tuple(q.shape)}, got {tuple(t.shape)}")
+        outs.append(t)
+    qo, ko, vo = outs
+    d3 = (0, 1, 2)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.daisy_qkv_prep_fwd(
+            q.data_ptr(), _lib.strides(q, d3), k.data_ptr(), _lib.strides(k, d3), v.data_ptr(), _lib.strides(v, d3),
+            _lib.ptr(ve), None if ve is None else _lib.strides(ve, d3), _lib.ptr(gate),
+            _lib.ptr(cos), _lib.ptr(sin), int(pos0),
+            qo.data_ptr(), _lib.strides(qo, d3), ko.data_ptr(), _lib.strides(ko, d3), vo.data_ptr(), _lib.strides(vo, d3),
+            B, T, H, D, float(eps), _lib.current_stream(dev))
+    _lib.check(rc, "daisy_qkv_prep_fwd")
+    return qo, ko, vo

@@ -163,6 +163,35 @@ int daisy_kda_gate_fwd(const void* g, const float* A_log, const float* bias, voi
                        int64_t rows, int H, int Dk, int io_is_bf16,
                        float softplus_beta, float threshold, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Fused pre-attention pass over the QKV projection output.  Replaces, in one
+ * streaming kernel, the elementwise chain of CausalSelfAttention._calc_qkv and
+ * _qkv_common (models/daisy/attention.py:116-135): weightless RMS norm of q, k
+ * and v (models/daisy/functional.py:6-7), RoPE of q and k (attention.py:16-20)
+ * at table rows pos0 + t, and the value-embedding mix
+ * v = gate * v + (1 - gate) * ve (attention.py:132-135).  Intermediates are
+ * rounded to bf16 where the reference materialises bf16 tensors.
+ *
+ * q, k, v : bf16, logical [B, T, H, D], strides {b, t, h} in elements, D
+ *           contiguous (typically three views of the [B, T, 3H, D] GEMM output).
+ * ve, gate: ve bf16 [B, T, H, D] with strides, gate = device pointer to one fp32
+ *           holding sigmoid(g_ve) already rounded to bf16; both NULL = no mix.
+ * cos, sin: fp32 [>= pos0 + T, D/2] or both NULL = no RoPE.
+ * q_out, k_out, v_out : bf16 with their own {b, t, h} strides (e.g. k_out and
+ *           v_out may be laid out [B, H, T, D] or be rows of a KV cache).
+ * eps     : added to mean(x^2) before the reciprocal square root.
+ * D is 64 or 128.
+ */
+int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
+                       const void* k, const int64_t* k_strides,
+                       const void* v, const int64_t* v_strides,
+                       const void* ve, const int64_t* ve_strides, const float* gate,
+                       const float* cos, const float* sin, int pos0,
+                       void* q_out, const int64_t* q_out_strides,
+                       void* k_out, const int64_t* k_out_strides,
+                       void* v_out, const int64_t* v_out_strides,
+                       int B, int T, int H, int D, float eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

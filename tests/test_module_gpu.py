@@ -57,10 +57,12 @@ def test_config1_plumbing_layer():
         assert_close_bf16(v, v_ref, "v", max_abs=4e-2, mean_abs=4e-3)
 
 
+@pytest.mark.parametrize("fused_prep", [True, False])
 @pytest.mark.parametrize("receives_ve", [False, True])
-def test_prefill_matches_oracle_with_documents_and_ve(receives_ve):
+def test_prefill_matches_oracle_with_documents_and_ve(receives_ve, fused_prep):
     dim, H, D, T, W = 512, 4, 128, 333, 100
     attn = _make(dim, H, D, receives_ve=receives_ve, seed=1).to(DEV)
+    attn.fused_prep = fused_prep    # one-pass norm + RoPE + mix kernel, or the library ops + RoPE inside attention
     g = torch.Generator().manual_seed(2)
     x = torch.randn(2, T, dim, generator=g).bfloat16()
     ve = torch.randn(2, T, dim, generator=g).bfloat16() if receives_ve else None
@@ -83,11 +85,12 @@ def test_prefill_matches_oracle_with_documents_and_ve(receives_ve):
     assert_close_bf16(y2, y_ref, "y (dense mask)")
 
 
-@pytest.mark.parametrize("T,W", [(128, 128), (131, 128), (70, 16)])
-def test_forward_equals_steps(T, W):
+@pytest.mark.parametrize("T,W,fused_prep", [(128, 128, True), (131, 128, True), (70, 16, True), (70, 16, False)])
+def test_forward_equals_steps(T, W, fused_prep):
     """Reference tests/test_causal_self_attention_equivalence.py: full forward == T streaming steps (bf16, 2e-2)."""
     dim, H, D = 128, 2, 64
     attn = _make(dim, H, D, receives_ve=True, seed=3).to(DEV)
+    attn.fused_prep = fused_prep
     g = torch.Generator().manual_seed(4)
     x = torch.randn(1, T, dim, generator=g).bfloat16().to(DEV)
     ve = torch.randn(1, T, H, D, generator=g).bfloat16().to(DEV)

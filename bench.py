@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu]
 
-NAME is one of prefill | long | decode | kda | copy; "copy" runs a plain 1 GiB
+NAME is one of prefill | module | long | decode | kda | copy; "copy" runs a plain 1 GiB
 device copy and nothing else (the known-size kernel against which the HBM
 counters FETCH_SIZE / WRITE_SIZE are calibrated under rocprofv3 --pmc).
 
@@ -131,8 +131,8 @@ def cpu_prefill_baseline(q, k, v, cos, sin, W, sample):
 
 # HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # (profiles/prefill_pipe_kernel_c2_hbm_traffic.txt), each scaled by the factor the same counter
-# shows for the 1 GiB copy of `--only copy`.  None until measured.
-PREFILL_C2_TRAFFIC_BYTES = None
+# shows for the 1 GiB copy of `--only copy` (2.000 for reads, 1.000 for writes).
+PREFILL_C2_TRAFFIC_BYTES = (126413 * 2 + 65558) * 1024
 
 
 def bench_copy(steps, warmup):
@@ -142,6 +142,36 @@ def bench_copy(steps, warmup):
     dst = torch.empty_like(src)
     ms = time_gpu(lambda: dst.copy_(src), steps, warmup)
     return {"workload": "copy_1GiB", "bytes_read": n, "bytes_written": n, "ms": ms, "gbs": 2 * n / ms / 1e6}
+
+
+def bench_module_c2(steps, warmup):
+    """CausalSelfAttention.prefill on config 2 (QKV GEMM, norm, RoPE, attention, output GEMM), with the
+    one-pass norm + RoPE kernel and with the library's elementwise ops; plus that kernel alone."""
+    from daisy_amd import CausalSelfAttention, WindowMask, ops
+    from daisy_amd.functional import NORM_EPS_BF16
+    B, T, H, D, W, dim = 8, 4096, 8, 128, 1024, 1024
+    dev = "cuda:0"
+    torch.manual_seed(0)
+    attn = CausalSelfAttention(dim=dim, num_heads=H, head_dim=D, max_seq_len=T)
+    with torch.no_grad():
+        attn.qkvo_w.copy_((torch.randn(4, dim, dim) * 0.02).bfloat16())
+    attn = attn.to(dev).eval()
+    x = torch.randn(B, T, dim, generator=torch.Generator().manual_seed(0)).bfloat16().to(dev)
+    mask = WindowMask(W)
+    out = {"workload": "module_prefill_c2_B8_T4096_d1024_H8_D128_W1024"}
+    with torch.no_grad():
+        for name, fused in (("ms_fused_prep", True), ("ms_library_elementwise", False)):
+            attn.fused_prep = fused
+            out[name] = time_gpu(lambda: attn.prefill(x, None, attn_mask=mask), steps, warmup)
+        qkv = torch.nn.functional.linear(x, attn.qkvo_w[:3].flatten(end_dim=1)).view(B, T, 3 * H, D)
+        q, k, v = qkv.chunk(3, dim=-2)
+        cos, sin = attn.rotary._get_cos_sin(T)
+        qo, ko, vo = (torch.empty(B, T, H, D, dtype=torch.bfloat16, device=dev) for _ in range(3))
+        ms = time_gpu(lambda: ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, q_out=qo, k_out=ko, v_out=vo),
+                      steps, warmup)
+    nbytes = 6 * B * T * H * D * 2
+    out["qkv_prep_kernel"] = {"ms": ms, "bytes": nbytes, "gbs": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    return out
 
 
 def bench_prefill_c3(steps, warmup):
@@ -251,7 +281,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", default=None, help="prefill | long | decode | kda | copy (default: all but copy)")
+    ap.add_argument("--only", default=None, help="prefill | module | long | decode | kda | copy (default: all but copy)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -269,6 +299,8 @@ def main():
     cpu = not args.no_cpu
     extra = {}
     head = bench_prefill_c2(args.steps, args.warmup, cpu) if want("prefill") else None
+    if want("module"):
+        extra["module_c2"] = bench_module_c2(max(args.steps // 2, 4), max(args.warmup // 2, 2))
     if want("long"):
         extra["prefill_c3_B1_T65536_H16_D128"] = bench_prefill_c3(max(args.steps // 5, 4), max(args.warmup // 2, 2))
     if want("decode"):

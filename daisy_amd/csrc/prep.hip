@@ -45,8 +45,9 @@ __global__ __launch_bounds__(256) void qkv_prep_kernel(PrepParams p) {
 
   auto load_row = [&](const uint16_t* base, int64_t sb, int64_t st, int64_t sh, float* lo, float* hi) {
     const uint16_t* src = base + b * sb + t * st + h * sh + 8 * c;
-    const u32x4 a = *reinterpret_cast<const u32x4*>(src);
-    const u32x4 d = *reinterpret_cast<const u32x4*>(src + HALF);
+    // streamed once: keep the rows out of the way of the tables in the caches
+    const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src));
+    const u32x4 d = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + HALF));
     unpack8(a, lo);
     unpack8(d, hi);
   };

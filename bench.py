@@ -262,6 +262,15 @@ def bench_kda_c5(steps, warmup, cpu_baseline=True):
     out = {"workload": "kda_c5_B4_T8192_H16_D128_chunk64", "ms": ms, "min_bytes": min_bytes,
            "gbs_min_io": min_bytes / ms / 1e6, "frac_of_hbm_peak": min_bytes / ms / 1e6 / PEAK_HBM_GBS,
            "naive_flops": flops, "tflops_naive": flops / ms / 1e9}
+    # One decode step of the same layer at batch 64: the token-by-token kernel reads and writes the fp32 state once.
+    Bd = 64
+    S = torch.zeros(Bd, H, Dk, Dv, dtype=torch.float32, device=dev)
+    qd, kd, vd = (rn(Bd, 1, H, Dk).bfloat16() for _ in range(3))
+    gd, bd = torch.nn.functional.logsigmoid(rn(Bd, 1, H, Dk)), torch.sigmoid(rn(Bd, 1, H))
+    ms_step = time_gpu(lambda: ops.kda_recurrent_fwd(qd, kd, vd, gd, bd, initial_state=S, inplace_state=True), 64, 8)
+    state_bytes = 2 * Bd * H * Dk * Dv * 4
+    out["decode_step_B64"] = {"ms": ms_step, "state_bytes_rw": state_bytes, "gbs": state_bytes / ms_step / 1e6,
+                              "frac_of_hbm_peak": state_bytes / ms_step / 1e6 / PEAK_HBM_GBS}
     if cpu_baseline:
         import oracle
         torch.set_num_threads(os.cpu_count() or 1)

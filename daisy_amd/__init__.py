@@ -9,10 +9,10 @@ from .attention import (CausalSelfAttention, Rotary, WindowMask, build_window_ma
                         dense_mask_to_window, doc_start_from_ids)
 from .functional import norm  # noqa: F401
 from .generate import Generator  # noqa: F401
-from .kda import chunk_kda, fused_kda_gate  # noqa: F401
+from .kda import chunk_kda, fused_kda_gate, fused_recurrent_kda  # noqa: F401
 from .kv_cache import KVCache, RingContext  # noqa: F401
 
 __all__ = [
     "CausalSelfAttention", "Rotary", "WindowMask", "build_window_mask", "dense_mask_to_window",
-    "doc_start_from_ids", "norm", "Generator", "chunk_kda", "fused_kda_gate", "KVCache", "RingContext",
+    "doc_start_from_ids", "norm", "Generator", "chunk_kda", "fused_kda_gate", "fused_recurrent_kda", "KVCache", "RingContext",
 ]

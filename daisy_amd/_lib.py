@@ -49,6 +49,11 @@ SIGNATURES = {
         c_int, c_int, c_int, c_int, c_int, c_int,               # B, T, H, Dk, Dv, chunk
         c_float, c_int, c_float,                                # scale, l2norm_qk, l2_eps
         c_void_p, c_size_t, c_void_p]),                         # workspace, bytes, stream
+    "daisy_kda_recurrent_fwd": (c_int, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,  # q, k, v, g, g_is_bf16, beta
+        c_void_p, c_void_p, c_void_p,                           # initial_state, o, final_state
+        c_int, c_int, c_int, c_int, c_int,                      # B, T, H, Dk, Dv
+        c_float, c_int, c_float, c_void_p]),                    # scale, l2norm_qk, l2_eps, stream
     "daisy_kda_gate_fwd": (c_int, [
         c_void_p, c_void_p, c_void_p, c_void_p,                 # g, A_log, bias, out
         c_int64, c_int, c_int, c_int,                           # rows, H, Dk, io_is_bf16

@@ -178,6 +178,55 @@ def kda_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
     return o, final
 
 
+def kda_recurrent_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, *,
+                      scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
+                      output_final_state: bool = True, use_qk_l2norm_in_kernel: bool = True,
+                      l2_eps: float = 1e-6, inplace_state: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Token-by-token KDA with the state in registers; see ``daisy_kda_recurrent_fwd``.
+
+    With ``inplace_state`` the final state overwrites ``initial_state`` (which must then be a
+    contiguous fp32 ``[B, H, Dk, Dv]`` tensor) and is returned as such -- the decode loop's mode.
+    """
+    dev = _lib.require_gpu(q, k, v, g, beta, initial_state)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_bf16(name, t, 4)
+    B, T, H, Dk = q.shape
+    Dv = v.shape[-1]
+    if k.shape != q.shape or g.shape != q.shape or v.shape[:3] != q.shape[:3] or beta.shape != (B, T, H):
+        raise ValueError("kda: expected q,k,g [B,T,H,Dk], v [B,T,H,Dv], beta [B,T,H]")
+    if g.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"g must be fp32 or bf16, got {g.dtype}")
+    q, k, v, g = q.contiguous(), k.contiguous(), v.contiguous(), g.contiguous()
+    beta = beta.to(torch.float32).contiguous()
+    if scale is None:
+        scale = Dk ** -0.5
+    if initial_state is not None:
+        if initial_state.shape != (B, H, Dk, Dv):
+            raise ValueError(f"initial_state must be [B,H,Dk,Dv], got {tuple(initial_state.shape)}")
+        if inplace_state:
+            if initial_state.dtype != torch.float32 or not initial_state.is_contiguous():
+                raise ValueError("inplace_state needs a contiguous fp32 initial_state")
+        else:
+            initial_state = initial_state.to(torch.float32).contiguous()
+    elif inplace_state:
+        raise ValueError("inplace_state needs an initial_state")
+    o = torch.empty((B, T, H, Dv), dtype=torch.bfloat16, device=dev)
+    if inplace_state:
+        final = initial_state
+    else:
+        final = torch.empty((B, H, Dk, Dv), dtype=torch.float32, device=dev) if output_final_state else None
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.daisy_kda_recurrent_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(),
+            g.data_ptr(), 1 if g.dtype == torch.bfloat16 else 0, beta.data_ptr(),
+            _lib.ptr(initial_state), o.data_ptr(), _lib.ptr(final),
+            B, T, H, Dk, Dv, float(scale), 1 if use_qk_l2norm_in_kernel else 0, float(l2_eps),
+            _lib.current_stream(dev))
+    _lib.check(rc, "daisy_kda_recurrent_fwd")
+    return o, final
+
+
 def kda_gate_fwd(g: torch.Tensor, A_log: torch.Tensor, head_k_dim: int,
                  g_bias: Optional[torch.Tensor] = None, beta: float = 1.0, threshold: float = 20.0) -> torch.Tensor:
     """``-exp(A_log[h]) * softplus(g + bias)``; ``g [..., H*Dk]`` -> ``[..., H, Dk]`` in ``g.dtype``."""

@@ -152,6 +152,21 @@ int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * Token-by-token KDA (the recurrence of daisy_kda_chunk_fwd evaluated one token
+ * at a time, state in registers).  This is the "fused_recurrent" mode that
+ * models/daisy/attention_kimi.py:70,144 names and leaves unsupported; a
+ * generation loop calls it with T = 1 per step, carrying the state.
+ *
+ * Tensors as in daisy_kda_chunk_fwd (contiguous [B, T, H, D]; Dk = Dv = 128).
+ * initial_state NULL = zeros; final_state NULL = not wanted; the two may alias.
+ */
+int daisy_kda_recurrent_fwd(const void* q, const void* k, const void* v,
+                            const void* g, int g_is_bf16, const float* beta,
+                            const float* initial_state, void* o, float* final_state,
+                            int B, int T, int H, int Dk, int Dv,
+                            float scale, int l2norm_qk, float l2_eps, void* stream);
+
+/* ---------------------------------------------------------------------------
  * KDA log-decay gate:  out[..., h, d] = -exp(A_log[h]) * softplus(g[..., h, d] + bias[h, d])
  * (softplus is the identity above `threshold`).  Replaces fused_kda_gate
  * (models/daisy/fla_custom_ops.py:71-103,190-200), forward only.

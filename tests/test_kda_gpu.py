@@ -113,3 +113,59 @@ def test_kda_rejects_unsupported_shapes():
     z = torch.zeros(1, 64, 1, 64, dtype=torch.bfloat16, device="cuda:0")
     with pytest.raises(RuntimeError, match="Dk"):
         ops.kda_chunk_fwd(z, z, z, z.float(), torch.zeros(1, 64, 1, device="cuda:0"))
+
+
+# ---- token-by-token kernel (decode steps, short prompts) ------------------------------------
+
+@pytest.mark.parametrize("B,T,H,g_scale,g_bf16", [
+    (2, 1, 3, 1.0, False),     # one decode step
+    (1, 17, 2, 1.0, False),
+    (2, 130, 2, 0.05, True),   # slow decay, bf16 gate
+    (1, 64, 1, 8.0, False),    # very fast decay
+])
+def test_kda_recurrent_matches_recurrence(B, T, H, g_scale, g_bf16):
+    from daisy_amd import fused_recurrent_kda
+    say(f"kda recurrent case B{B} T{T} H{H} g_scale{g_scale} g_bf16={g_bf16}")
+    q, k, v, gl, beta = _inputs(B, T, H, seed=100 + T + H, g_scale=g_scale)
+    if g_bf16:
+        gl = gl.bfloat16()
+    S0 = torch.randn(B, H, 128, 128, generator=torch.Generator().manual_seed(9)) * 0.1
+    o_ref, S_ref = oracle.kda_recurrent(q, k, v, gl.float(), beta, initial_state=S0)
+    o, S = fused_recurrent_kda(q.cuda(), k.cuda(), v.cuda(), gl.cuda(), beta.cuda(), initial_state=S0.cuda(),
+                               output_final_state=True, use_qk_l2norm_in_kernel=True)
+    torch.cuda.synchronize()
+    _check(o, S, o_ref, S_ref, "kda recurrent")
+    # no initial state, no final state wanted, no L2 norm (inputs are unit vectors already up to bf16 rounding)
+    o_ref2, _ = oracle.kda_recurrent(q, k, v, gl.float(), beta, use_qk_l2norm=False)
+    o2, S2 = fused_recurrent_kda(q.cuda(), k.cuda(), v.cuda(), gl.cuda(), beta.cuda())
+    assert S2 is None
+    assert_close_bf16(o2, o_ref2, "kda recurrent (no state): o")
+
+
+def test_kda_decode_steps_continue_a_chunked_prefill():
+    """Prefill T0 tokens with the chunked kernel, then decode token by token with the state carried in place:
+    outputs and final state equal one chunked run over all T tokens."""
+    from daisy_amd import fused_recurrent_kda
+    B, T0, n_steps, H = 2, 200, 24, 2
+    T = T0 + n_steps
+    q, k, v, gl, beta = (t.cuda() for t in _inputs(B, T, H, seed=77))
+    o_ref, S_ref = oracle.kda_recurrent(q.cpu(), k.cpu(), v.cpu(), gl.cpu(), beta.cpu())
+    o0, S = chunk_kda(q[:, :T0], k[:, :T0], v[:, :T0], gl[:, :T0], beta[:, :T0], output_final_state=True,
+                      use_qk_l2norm_in_kernel=True)
+    outs = [o0]
+    ptr = S.data_ptr()
+    for t in range(T0, T):
+        o_t, S_t = fused_recurrent_kda(q[:, t:t + 1], k[:, t:t + 1], v[:, t:t + 1], gl[:, t:t + 1], beta[:, t:t + 1],
+                                       initial_state=S, use_qk_l2norm_in_kernel=True, inplace_state=True)
+        assert S_t.data_ptr() == ptr
+        outs.append(o_t)
+    torch.cuda.synchronize()
+    _check(torch.cat(outs, 1), S, o_ref, S_ref, "kda prefill + decode steps")
+
+
+def test_kda_recurrent_rejects_bad_arguments():
+    q, k, v, gl, beta = (t.cuda() for t in _inputs(1, 4, 1, seed=3))
+    with pytest.raises(RuntimeError, match="not supported"):
+        ops.kda_recurrent_fwd(q[..., :64].contiguous(), k[..., :64].contiguous(), v, gl[..., :64].contiguous(), beta)
+    with pytest.raises(ValueError):
+        ops.kda_recurrent_fwd(q, k, v, gl, beta, inplace_state=True)

@@ -7,6 +7,7 @@ Hand-written gfx950 HIP kernels (``daisy_amd/csrc``, C ABI in
 """
 from .attention import (CausalSelfAttention, Rotary, WindowMask, build_window_mask,  # noqa: F401
                         dense_mask_to_window, doc_start_from_ids)
+from . import core  # noqa: F401
 from .functional import norm  # noqa: F401
 from .generate import Generator  # noqa: F401
 from .kda import chunk_kda, fused_kda_gate, fused_recurrent_kda  # noqa: F401
@@ -14,5 +15,5 @@ from .kv_cache import KVCache, RingContext  # noqa: F401
 
 __all__ = [
     "CausalSelfAttention", "Rotary", "WindowMask", "build_window_mask", "dense_mask_to_window",
-    "doc_start_from_ids", "norm", "Generator", "chunk_kda", "fused_kda_gate", "fused_recurrent_kda", "KVCache", "RingContext",
+    "doc_start_from_ids", "norm", "Generator", "chunk_kda", "fused_kda_gate", "fused_recurrent_kda", "KVCache", "RingContext", "core",
 ]

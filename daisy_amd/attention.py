@@ -115,10 +115,28 @@ class Rotary(nn.Module):
             active = (1 / base) ** torch.linspace(0, 1, steps=keep, dtype=torch.float32)
             angular_freq = torch.cat([active, active.new_zeros(half - keep)])
         self.inv_freq = nn.Buffer(angular_freq, persistent=False)
+        self._inv_freq_fp32 = angular_freq.clone()   # plain attribute: survives dtype casts of the module
         theta = torch.outer(torch.arange(max_seq_len, dtype=torch.float32), angular_freq)
         self.cos = nn.Buffer(theta.cos(), persistent=False)
         self.sin = nn.Buffer(theta.sin(), persistent=False)
         self._max_seq_len = int(max_seq_len)
+
+    def _apply(self, fn, recurse=True):
+        # Module-wide casts (model.bfloat16(), .half(), .to(dtype)) move the tables with the module
+        # but must not narrow them: the kernels take fp32 tables, and bf16 angles lose the position.
+        super()._apply(fn, recurse)
+        for name in ("inv_freq", "cos", "sin"):
+            buf = getattr(self, name)
+            if buf.dtype != torch.float32:
+                dev = buf.device
+                if name == "inv_freq":
+                    fresh = self._inv_freq_fp32.to(dev)
+                else:
+                    theta = torch.outer(torch.arange(self._max_seq_len, dtype=torch.float32, device=dev),
+                                        self._inv_freq_fp32.to(dev))
+                    fresh = theta.cos() if name == "cos" else theta.sin()
+                setattr(self, name, nn.Buffer(fresh, persistent=False))
+        return self
 
     def _get_cos_sin(self, L):
         torch._assert(L <= self.cos.shape[0], f"Rotary buffers too small {self.cos.shape[0]} < {L}")
@@ -136,6 +154,9 @@ class Rotary(nn.Module):
 
 class CausalSelfAttention(nn.Module):
     """Merged-QKVO sliding-window causal self-attention (models/daisy/attention.py:73-202)."""
+
+    # step() takes a KVCache layer handle (RingContext) in place of chronological k_ctx / v_ctx.
+    accepts_ring_context = True
 
     def __init__(self, dim: int, num_heads: int, head_dim, receives_ve: bool = False,
                  layer_idx: Optional[int] = None, max_seq_len: int = 131072):

@@ -1,0 +1,165 @@
+"""Prefill / step glue over a Daisy model (models/daisy/daisy_core.py:294-370), cache-aware.
+
+The reference's ``DaisyCore.prefill`` builds a dense ``[1, 1, T, T]`` mask, stacks every layer's
+keys and values into ``kv [2, L, B, H, T, D]`` and hands that to ``KVCache.bulk_write_packed``;
+``DaisyCore.step`` takes one token of one sequence.  The two functions here walk the same
+model attributes (``embed``, ``blocks``, ``skip_map``, ``skip_weights``, ``ve_module_map`` /
+``compute_value_embeddings``, ``lm_head_w``, ``window_size``, ``attn_window_size``,
+``eos_token_id``) with the same arithmetic, but
+
+* pass the window / document mask as a descriptor (no T x T tensor, no T <= 46340 cap),
+* write each layer's keys and values straight into the ring cache as the layer finishes
+  (nothing of size ``L * T`` is ever stacked), and
+* accept a batch of sequences (the cache has a batch dimension; the reference pins B = 1).
+
+They work on the reference's ``DaisyCore`` once its blocks hold this package's
+``CausalSelfAttention``, and on any module with the same attributes.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor
+
+from .attention import WindowMask, build_window_mask
+from .functional import norm
+from .kv_cache import KVCache
+
+
+def _value_embeddings(model, ids: Tensor) -> Dict[int, Tensor]:
+    if hasattr(model, "compute_value_embeddings"):
+        return model.compute_value_embeddings(ids)
+    return {i: m(ids) for i, m in getattr(model, "ve_module_map", {}).items()}
+
+
+def _mask_for(model, input_seq: Tensor) -> WindowMask:
+    window = getattr(model, "window_size", None)
+    if input_seq.size(0) == 1:
+        return build_window_mask(input_seq, window, model.eos_token_id)
+    # One descriptor serves the whole batch, so document boundaries (which differ per row)
+    # cannot be expressed: a batch must not contain the end-of-sequence token.
+    torch._assert(bool((input_seq != model.eos_token_id).all()),
+                  "batched prefill needs prompts without the end-of-sequence token")
+    return WindowMask(window, None)
+
+
+@torch.no_grad()
+def prefill(model, input_seq: Tensor, cache: Optional[KVCache] = None, debug: bool = False
+            ) -> Tuple[Tensor, Optional[Tensor]]:
+    """``DaisyCore.prefill`` (daisy_core.py:325-370) for ``input_seq [B, T]``.
+
+    With ``cache`` the keys/values of every layer go straight into it (``cache.t`` becomes T) and
+    ``(logits [B, V], None)`` is returned; without, ``(logits, kv [2, L, B, H, T, D])`` as the
+    reference does.
+    """
+    assert input_seq.ndim == 2
+    B, T = input_seq.shape
+    L = len(model.blocks)
+    x = x0 = norm(model.embed(input_seq))
+    skip_map, skip_weights = model.skip_map, model.skip_weights
+    ve_map = _value_embeddings(model, input_seq)
+    attn_mask = _mask_for(model, input_seq)
+    k_list: List[Optional[Tensor]] = []
+    v_list: List[Optional[Tensor]] = []
+    skip_connections = []
+    for i in range(L):
+        if i in skip_map:
+            gate = torch.sigmoid(skip_weights[skip_map[i]])
+            x = x * gate + (1 - gate) * skip_connections[skip_map[i]]
+        x, k, v = model.blocks[i].prefill(x, ve_map.get(i), x0, attn_mask=attn_mask, debug=debug)
+        skip_connections.append(x)
+        if cache is not None:
+            if k is not None:
+                cache.bulk_write_layer(i, k, v, T)
+        else:
+            k_list.append(k)
+            v_list.append(v)
+    x = norm(x)
+    logits = F.linear(x[:, -1].bfloat16(), model.lm_head_w.bfloat16()).float()
+    if cache is not None:
+        cache.t = T
+        cache._staged = [False] * cache.L
+        return logits, None
+    H, D = model.attn_num_heads, model.attn_head_dim
+    zeros = None
+    K, V = [], []
+    for k, v in zip(k_list, v_list):
+        if k is None:
+            if zeros is None:
+                zeros = torch.zeros(B, H, T, D, device=x.device, dtype=x.dtype)
+            k = v = zeros
+        K.append(k)
+        V.append(v)
+    return logits, torch.stack([torch.stack(K, dim=0), torch.stack(V, dim=0)], dim=0)
+
+
+@torch.no_grad()
+def step(model, token_ids: Tensor, cache: KVCache) -> Tensor:
+    """``DaisyCore.step`` (daisy_core.py:294-323) for one new token per sequence, ``token_ids [B]``
+    (or a 0-dim tensor when B = 1), at position ``cache.t``.
+
+    Each attention layer streams its ring in place and appends the new row itself (bf16 cache and
+    this package's attention), or gets the chronological view and the row is written here.
+    Advances the cache; returns ``logits [B, V]``.
+    """
+    token_ids = token_ids.reshape(-1, 1)
+    B = token_ids.size(0)
+    torch._assert(B == cache.B, "token batch does not match the cache")
+    pos = cache.t
+    L = len(model.blocks)
+    x = x0 = norm(model.embed(token_ids))
+    skip_map, skip_weights = model.skip_map, model.skip_weights
+    ve_map = _value_embeddings(model, token_ids)
+    window = getattr(model, "attn_window_size", cache.W)
+    in_place = cache.dtype == torch.bfloat16
+    skip_connections = []
+    for i in range(L):
+        if i in skip_map:
+            gate = torch.sigmoid(skip_weights[skip_map[i]])
+            x = x * gate + (1 - gate) * skip_connections[skip_map[i]]
+        blk = model.blocks[i]
+        if getattr(blk, "attn", None) is None:
+            k_ctx = v_ctx = None
+        elif in_place and getattr(blk.attn, "accepts_ring_context", False):
+            k_ctx = v_ctx = cache.ring(i)
+        else:
+            k_ctx, v_ctx = cache.view(i)
+        x, k_new, v_new = blk.step(x, ve_map.get(i), x0, k_ctx, v_ctx, pos, window)
+        skip_connections.append(x)
+        if k_new is not None and not cache._staged[i]:
+            cache.write(i, k_new.to(cache.dtype), v_new.to(cache.dtype))
+    cache.advance()
+    x = norm(x)
+    return F.linear(x.flatten(end_dim=1).bfloat16(), model.lm_head_w.bfloat16()).float()
+
+
+@torch.no_grad()
+def generate_greedy(model, prompt_ids: Tensor, max_new_tokens: int, window: Optional[int] = None,
+                    cache: Optional[KVCache] = None) -> Tensor:
+    """Greedy continuation of a batch of equally long prompts ``[B, T]`` -> ``[B, max_new_tokens]``.
+
+    Rows that produce the end-of-sequence token keep emitting it.  The cache (bf16 ring of
+    ``window`` slots, default the model's window) is created unless given.
+    """
+    assert prompt_ids.ndim == 2 and prompt_ids.size(1) > 0 and max_new_tokens > 0
+    B = prompt_ids.size(0)
+    dev = prompt_ids.device
+    if cache is None:
+        W = window if window is not None else model.attn_window_size
+        cache = KVCache(L=len(model.blocks), B=B, H=model.attn_num_heads, W=W, D=model.attn_head_dim,
+                        device=dev, dtype=torch.bfloat16)
+    vocab = model.embed.num_embeddings
+    logits, _ = prefill(model, prompt_ids, cache)
+    done = torch.zeros(B, dtype=torch.bool, device=dev)
+    eos = torch.tensor(model.eos_token_id, device=dev)
+    out = []
+    for i in range(max_new_tokens):
+        tok = torch.argmax(logits[..., :vocab], dim=-1)
+        tok = torch.where(done, eos, tok)
+        done = done | (tok == eos)
+        out.append(tok)
+        if i < max_new_tokens - 1:
+            logits = step(model, tok, cache)
+    return torch.stack(out, dim=1)

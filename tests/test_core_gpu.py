@@ -1,0 +1,210 @@
+"""Cache-aware prefill / step glue (daisy_amd.core) on a small Daisy-shaped model.
+
+The model below has the attributes of the reference's DaisyCore (models/daisy/daisy_core.py:96-175)
+and blocks with the arithmetic of models/daisy/block.py:33-81.  Checked: against an fp32-softmax CPU
+evaluation of the same model through the oracle's attention; that writing K/V straight into the ring
+equals the reference's stack-then-bulk_write_packed route bit for bit; that steps through the ring match
+steps over chronological views; and that a batch of sequences gives what each sequence gives alone.
+"""
+import os
+
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+os.environ["DISABLE_O_ZERO_INIT"] = "1"
+
+import oracle
+from daisy_amd import CausalSelfAttention, KVCache, core
+from daisy_amd.functional import norm
+from helpers import say
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+class _MLP(nn.Module):
+    def __init__(self, dim):
+        super().__init__()
+        self.fc = nn.Parameter((torch.randn(2 * dim, dim) * 0.05).bfloat16())
+        self.proj = nn.Parameter((torch.randn(dim, 2 * dim) * 0.05).bfloat16())
+
+    def forward(self, x):
+        return F.linear(F.relu(F.linear(x, self.fc)).square(), self.proj)
+
+
+class _Block(nn.Module):
+    def __init__(self, dim, H, D, has_attn, receives_ve, max_seq_len):
+        super().__init__()
+        self.g_x = nn.Parameter(torch.tensor(2.0))
+        self.attn = CausalSelfAttention(dim, H, D, receives_ve=receives_ve, max_seq_len=max_seq_len) if has_attn else None
+        if self.attn is not None:
+            with torch.no_grad():
+                self.attn.qkvo_w.copy_((torch.randn(4, dim, dim) * 0.04).bfloat16())
+        self.mlp = _MLP(dim)
+
+    def _mix(self, x, x0):
+        g = torch.sigmoid(self.g_x)
+        return g * x + (1.0 - g) * x0
+
+    def prefill(self, x, ve, x0, attn_mask=None, debug=False):
+        x = self._mix(x, x0)
+        k = v = None
+        if self.attn is not None:
+            y, k, v = self.attn.prefill(x, ve, attn_mask, debug=debug)
+            x = x + y
+        return x + self.mlp(norm(x)), k, v
+
+    def step(self, x, ve, x0, k_ctx, v_ctx, pos, window):
+        x = self._mix(x, x0)
+        k = v = None
+        if self.attn is not None:
+            y, k, v = self.attn.step(x, k_ctx, v_ctx, pos, ve, window=window)
+            x = x + y
+        return x + self.mlp(norm(x)), k, v
+
+
+class _Core(nn.Module):
+    """L = 4 layers, attention in layers 0, 1, 3 (layer 2 has none), value embeddings into 0 and 3, skip 1 -> 3."""
+
+    def __init__(self, vocab=96, dim=256, H=2, D=128, window=48, eos=1, max_seq_len=512):
+        super().__init__()
+        torch.manual_seed(0)
+        self.embed = nn.Embedding(vocab, dim)
+        self.attn_layers = [0, 1, 3]
+        self.blocks = nn.ModuleList([_Block(dim, H, D, i in self.attn_layers, i in (0, 3), max_seq_len) for i in range(4)])
+        self.ve_emb = nn.Embedding(vocab, dim)
+        self.ve_module_map = {0: self.ve_emb, 3: self.ve_emb}
+        self.skip_map = {3: 1}
+        self.skip_weights = nn.Parameter(torch.ones(4) * 1.5)
+        self.lm_head_w = nn.Parameter(torch.randn(128, dim) * 0.05)
+        self.window_size = self.attn_window_size = window
+        self.eos_token_id = eos
+        self.attn_num_heads, self.attn_head_dim = H, D
+        self.bfloat16()
+
+    def compute_value_embeddings(self, ids):
+        return {i: m(ids) for i, m in self.ve_module_map.items()}
+
+    # the reference's own step signature (daisy_core.py:294-323), used as the comparison route
+    def step(self, token_id, k_ctxs, v_ctxs, pos):
+        token_id = token_id.view(1, 1)
+        x = x0 = norm(self.embed(token_id))
+        ve_map = self.compute_value_embeddings(token_id)
+        skips, ks, vs = [], [], []
+        for i, blk in enumerate(self.blocks):
+            if i in self.skip_map:
+                gate = torch.sigmoid(self.skip_weights[self.skip_map[i]])
+                x = x * gate + (1 - gate) * skips[self.skip_map[i]]
+            x, k, v = blk.step(x, ve_map.get(i), x0, k_ctxs[i], v_ctxs[i], pos, self.attn_window_size)
+            skips.append(x)
+            ks.append(k)
+            vs.append(v)
+        return F.linear(norm(x).flatten(end_dim=1).bfloat16(), self.lm_head_w.bfloat16()).float(), ks, vs
+
+
+def _cpu_prefill_logits(model_cpu, ids):
+    """The same model evaluated on the CPU with the oracle's attention (fp32 softmax and contractions)."""
+    m = model_cpu
+    T = ids.size(1)
+    x = x0 = oracle.rms_norm(m.embed(ids))
+    ve_map = m.compute_value_embeddings(ids)
+    doc_start = oracle.doc_start_from_ids(ids, m.eos_token_id)
+    skips = []
+    for i, blk in enumerate(m.blocks):
+        if i in m.skip_map:
+            gate = torch.sigmoid(m.skip_weights[m.skip_map[i]])
+            x = x * gate + (1 - gate) * skips[m.skip_map[i]]
+        x = blk._mix(x, x0)
+        if blk.attn is not None:
+            a = blk.attn
+            ve = ve_map.get(i)
+            y, _, _ = oracle.attn_prefill(x, a.qkvo_w.detach(), a.num_heads, a.head_dim, a.rotary.cos[:T], a.rotary.sin[:T],
+                                          m.window_size, doc_start=doc_start, ve=ve,
+                                          g_ve=None if a.g_ve is None else float(a.g_ve))
+            x = x + y
+        x = x + blk.mlp(oracle.rms_norm(x))
+        skips.append(x)
+    return F.linear(oracle.rms_norm(x)[:, -1].bfloat16(), m.lm_head_w.bfloat16()).float()
+
+
+def _close(a, b, what, tol=3e-2):
+    err = (a.float().cpu() - b.float().cpu()).abs().max().item()
+    ref = b.float().abs().max().item()
+    say(f"{what}: max-abs diff {err:.3e} (scale {ref:.2f})")
+    assert err <= tol * max(ref, 1.0), f"{what}: {err:.3e}"
+
+
+def test_prefill_matches_cpu_model_and_fills_the_ring_like_the_reference_route():
+    with torch.no_grad():
+        model_cpu = _Core()
+        model = _Core().to(DEV)
+        model.load_state_dict(model_cpu.state_dict())
+        T, W = 150, model.window_size
+        ids = torch.randint(2, 96, (1, T), generator=torch.Generator().manual_seed(3))
+        ids[0, 40] = ids[0, 97] = model.eos_token_id          # three documents
+        logits_ref = _cpu_prefill_logits(model_cpu, ids)
+        logits, kv = core.prefill(model, ids.to(DEV))           # reference-style return value
+        assert kv.shape == (2, 4, 1, 2, T, 128)
+        assert torch.count_nonzero(kv[:, 2]) == 0              # the layer without attention packs zeros
+        _close(logits, logits_ref, "prefill logits vs CPU model")
+        # straight into the ring == stack + bulk_write_packed (inference/kv_cache.py:57-68)
+        c_ref = KVCache(4, 1, 2, W, 128, DEV, torch.bfloat16)
+        c_ref.bulk_write_packed(kv, T)
+        c_new = KVCache(4, 1, 2, W, 128, DEV, torch.bfloat16)
+        logits2, none = core.prefill(model, ids.to(DEV), c_new)
+        assert none is None and c_new.t == T == c_ref.t
+        assert torch.equal(logits2, logits)
+        assert torch.equal(c_new.k, c_ref.k) and torch.equal(c_new.v, c_ref.v)
+
+
+def test_steps_through_the_ring_match_steps_over_chronological_views():
+    with torch.no_grad():
+        model = _Core().to(DEV)
+        T, n_steps, W = 70, 60, model.window_size                  # the ring wraps during the steps
+        ids = torch.randint(2, 96, (1, T + n_steps), generator=torch.Generator().manual_seed(4)).to(DEV)
+        ring = KVCache(4, 1, 2, W, 128, DEV, torch.bfloat16)
+        chrono = KVCache(4, 1, 2, W, 128, DEV, torch.bfloat16)
+        core.prefill(model, ids[:, :T], ring)
+        core.prefill(model, ids[:, :T], chrono)
+        for s in range(n_steps):
+            tok = ids[0, T + s]
+            la = core.step(model, tok, ring)
+            views = [chrono.view(i) for i in range(4)]
+            lb, ks, vs = model.step(tok, [v[0] for v in views], [v[1] for v in views], chrono.t)
+            for i in range(4):
+                if ks[i] is not None:
+                    chrono.write(i, ks[i], vs[i])
+            chrono.advance()
+            _close(la, lb, f"step {s} logits", tol=2e-2)
+        assert ring.t == chrono.t == T + n_steps
+        # same rows in the same slots; the attention-less layer's slots stay zero in both
+        _close(ring.k, chrono.k, "ring keys", tol=2e-2)
+        _close(ring.v, chrono.v, "ring values", tol=2e-2)
+        assert torch.count_nonzero(ring.k[2]) == 0
+
+
+def test_batched_prefill_and_steps_match_single_sequences():
+    with torch.no_grad():
+        model = _Core().to(DEV)
+        B, T, n_steps, W = 3, 64, 8, model.window_size
+        ids = torch.randint(2, 96, (B, T + n_steps), generator=torch.Generator().manual_seed(5)).to(DEV)
+        cache = KVCache(4, B, 2, W, 128, DEV, torch.bfloat16)
+        lb = [core.prefill(model, ids[:, :T], cache)[0]]
+        for s in range(n_steps):
+            lb.append(core.step(model, ids[:, T + s], cache))
+        for b in range(B):
+            c1 = KVCache(4, 1, 2, W, 128, DEV, torch.bfloat16)
+            l1 = [core.prefill(model, ids[b:b + 1, :T], c1)[0]]
+            for s in range(n_steps):
+                l1.append(core.step(model, ids[b, T + s], c1))
+            for s in range(n_steps + 1):
+                _close(lb[s][b:b + 1], l1[s], f"row {b} call {s}", tol=2e-2)
+            _close(cache.k[:, b:b + 1], c1.k, f"row {b} ring keys", tol=2e-2)
+        out = core.generate_greedy(model, ids[:, :T], 6)
+        assert out.shape == (B, 6) and out.dtype == torch.long
+        with pytest.raises(Exception, match="end-of-sequence"):
+            bad = ids[:, :T].clone()
+            bad[1, 5] = model.eos_token_id
+            core.prefill(model, bad, KVCache(4, B, 2, W, 128, DEV, torch.bfloat16))

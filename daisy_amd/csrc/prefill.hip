@@ -559,15 +559,10 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
     asm volatile("" ::: "memory");
   };
 
-  // The first copy goes out before anything else so that its latency overlaps the Q loads.
+  // The first two K tiles go out before anything else so that their latency overlaps the Q loads.
+  auto tile_of = [&](int n) { const int t = t_first + n; return t <= t_hi ? t : t - n_tiles; };
   copy_k(t_first, 0);
-  // V buffer 1 is read (times a zero P) before anything was copied into it: clear it.
-  {
-    u32x4 z = {0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < TILE / 8 / kPrefillThreads; ++i)
-      *reinterpret_cast<u32x4*>(&Vs[1][8 * (tid + kPrefillThreads * i)]) = z;
-  }
+  if (n_tiles > 1) copy_k(tile_of(1), 1);
 
   // ---- Q fragment (B operand), RoPE fused ----------------------------------
   bf16x8 qreg[NS];
@@ -617,18 +612,19 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
   for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+  f32x16 sc[2];                    // S of the tile this step turns into P; refilled in place for the next tile
   float m_run = -INFINITY, l_run = 0.f;
   float alpha_pend = 1.f;          // rescale of O asked for by the last softmax, not applied yet
   bool rescale_pend = false;       // wave-uniform
+  bool pending = false;            // wave-uniform: pfrag holds a P that has not been multiplied into O yet
   bf16x8 pfrag[2][2];              // P of the previous tile (B operands of the delayed product)
-  auto clear_pfrag = [&]() {
+  {
     const u32x4 z = {0, 0, 0, 0};
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int m = 0; m < 2; ++m) pfrag[sb][m] = __builtin_bit_cast(bf16x8, z);
-  };
-  clear_pfrag();
+  }
 
   auto apply_pending_rescale = [&]() {
     if (rescale_pend) {
@@ -640,79 +636,50 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
     }
   };
 
-  // O^T += V^T P^T with the P left by the previous tile, V from buffer offset vofs (elements).
-  auto pv_product = [&](int vofs) {
+  // One 32-key half of S^T = K Q^T into sc[sb], K from buffer offset kofs (elements).
+  auto qk_half = [&](int kofs, int sb) {
+    constexpr int KPF = 3;   // K fragments are read KPF contraction slices ahead of their MFMAs
+    bf16x8 ka[KPF];
+    auto read_k = [&](int s) {
+      ka[s % KPF] = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(k_rd[s] + kofs + 32 * sb * D));
+    };
 #pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
+    for (int s = 0; s < KPF; ++s) read_k(s);
 #pragma unroll
-      for (int m = 0; m < 2; ++m) {
+    for (int r = 0; r < 16; ++r) sc[sb][r] = 0.f;
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-          lds_u16_ptr vp = v_rd[dt] + vofs;
-          const u32x2 a0 = lds_read_tr16_as3(vp + (32 * sb + 16 * m) * D);
-          const u32x2 a1 = lds_read_tr16_as3(vp + (32 * sb + 16 * m + 8) * D);
-          const u32x4 av = {a0.x, a0.y, a1.x, a1.y};
-          oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), pfrag[sb][m], oacc[dt], 0, 0, 0);
-        }
+    for (int s = 0; s < NS; ++s) {
+      sc[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[s % KPF], qreg[s], sc[sb], 0, 0, 0);
+      if (s + KPF < NS) read_k(s + KPF);
+    }
+  };
+
+  // Half of O^T += V^T P^T: the 32 keys of block sb, V from buffer offset vofs (elements).
+  auto pv_half = [&](int vofs, int sb) {
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) {
+        lds_u16_ptr vp = v_rd[dt] + vofs;
+        const u32x2 a0 = lds_read_tr16_as3(vp + (32 * sb + 16 * m) * D);
+        const u32x2 a1 = lds_read_tr16_as3(vp + (32 * sb + 16 * m + 8) * D);
+        const u32x4 av = {a0.x, a0.y, a1.x, a1.y};
+        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), pfrag[sb][m], oacc[dt], 0, 0, 0);
       }
     }
   };
 
-  // One tile of this wavefront: S = K Q^T, then (one basic block) the delayed product of the
-  // previous tile together with the softmax of this one.
-  auto wave_tile = [&](int tile, int par, auto masked_tag) {
-    constexpr bool MASKED = decltype(masked_tag)::value;
-    const int kv0 = tile * kBN;
-    const int kofs = par * TILE, vofs = (par ^ 1) * TILE;
-    f32x16 sc[2];
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sc[sb][r] = 0.f;
-    // K fragments are read KPF contraction slices ahead of the MFMAs that use them.
-    constexpr int KPF = 3;
-    bf16x8 ka[KPF][2];
-    auto read_k = [&](int s) {
-      lds_u16_ptr kp = k_rd[s] + kofs;
-#pragma unroll
-      for (int sb = 0; sb < 2; ++sb)
-        ka[s % KPF][sb] = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(kp + 32 * sb * D));
-    };
-#pragma unroll
-    for (int s = 0; s < KPF; ++s) read_k(s);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-#pragma unroll
-      for (int sb = 0; sb < 2; ++sb)
-        sc[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[s % KPF][sb], qreg[s], sc[sb], 0, 0, 0);
-      if (s + KPF < NS) read_k(s + KPF);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    apply_pending_rescale();
-    pv_product(vofs);
-    if constexpr (MASKED) {
-#pragma unroll
-      for (int sb = 0; sb < 2; ++sb) {
-        // element r of this lane is key kv0 + 32sb + 4lh + c_r with c_r = 8*(r/4) + r%4
-        const int hi = qrow - (kv0 + 32 * sb + 4 * lh);    // visible iff lo <= c_r <= hi
-        const int lo = lo_q - (kv0 + 32 * sb + 4 * lh);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int c = 8 * (r >> 2) + (r & 3);
-          if (c > hi || c < lo) sc[sb][r] = -INFINITY;
-        }
-      }
-    }
+  // Online-softmax bookkeeping for the tile held in sc (after masking): returns the exponent offset.
+  // Lazy rescale: the reference maximum only moves when some query of the wavefront sees a score
+  // more than 8 (log2 units) above it; until then probabilities stay below 2^8, which bf16 and
+  // the fp32 sums hold without loss, and O is not touched.
+  auto update_maximum = [&]() {
     float mt = -INFINITY;
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sc[sb][r]);
     mt = pair_max(mt) * p.scale_log2e;
-    // Lazy rescale: the reference maximum only moves when some query of the wavefront sees a
-    // score more than 8 (log2 units) above it; until then probabilities stay below 2^8, which
-    // bf16 and the fp32 sums hold without loss, and O is not touched.
     const bool move = __builtin_amdgcn_ballot_w64(mt > m_run + 8.f) != 0;
     const float m_new = move ? fmaxf(m_run, mt) : m_run;
     const float mu = (m_new == -INFINITY) ? 0.f : m_new;
@@ -720,84 +687,136 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
     m_run = m_new;
     alpha_pend = alpha;
     rescale_pend = move;
+    l_run *= alpha;
+    return mu;
+  };
+  // P of one 32-key half: exp2, row sums, bf16 B operands of the delayed product.
+  auto probabilities_half = [&](int sb, float mu) {
+    float pv[16];
     float lsum = 0.f;
 #pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      pv[r] = fast_exp2(fmaf(sc[sb][r], p.scale_log2e, -mu));
+      lsum += pv[r];
+    }
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      u32x4 pk;
+      pk.x = pack_bf16x2(pv[8 * m + 0], pv[8 * m + 1]);
+      pk.y = pack_bf16x2(pv[8 * m + 2], pv[8 * m + 3]);
+      pk.z = pack_bf16x2(pv[8 * m + 4], pv[8 * m + 5]);
+      pk.w = pack_bf16x2(pv[8 * m + 6], pv[8 * m + 7]);
+      pfrag[sb][m] = __builtin_bit_cast(bf16x8, pk);
+    }
+    l_run += lsum;
+  };
+  auto mask_scores = [&](int kv0) {
+#pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
-      float pv[16];
+      // element r of this lane is key kv0 + 32sb + 4lh + c_r with c_r = 8*(r/4) + r%4
+      const int hi = qrow - (kv0 + 32 * sb + 4 * lh);    // visible iff lo <= c_r <= hi
+      const int lo = lo_q - (kv0 + 32 * sb + 4 * lh);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        pv[r] = fast_exp2(fmaf(sc[sb][r], p.scale_log2e, -mu));
-        lsum += pv[r];
-      }
-#pragma unroll
-      for (int m = 0; m < 2; ++m) {
-        u32x4 pk;
-        pk.x = pack_bf16x2(pv[8 * m + 0], pv[8 * m + 1]);
-        pk.y = pack_bf16x2(pv[8 * m + 2], pv[8 * m + 3]);
-        pk.z = pack_bf16x2(pv[8 * m + 4], pv[8 * m + 5]);
-        pk.w = pack_bf16x2(pv[8 * m + 6], pv[8 * m + 7]);
-        pfrag[sb][m] = __builtin_bit_cast(bf16x8, pk);
+        const int c = 8 * (r >> 2) + (r & 3);
+        if (c > hi || c < lo) sc[sb][r] = -INFINITY;
       }
     }
-    l_run = l_run * alpha + lsum;
+  };
+
+  auto is_active = [&](int n) {
+    if (n < 0 || n >= n_tiles) return false;
+    const int t = tile_of(n);
+    return t >= tw_lo && t <= tw_hi;
+  };
+  // Step n: K(n+2) and V(n) start on their way; at the end they have landed and all wavefronts meet.
+  // K(n+1) was published by the previous step, V(n-1) too.
+  auto step_begin = [&](int n) {
+    if (n + 2 < n_tiles) copy_k(tile_of(n + 2), n & 1);
+    copy_v(tile_of(n), n & 1);
+  };
+  auto step_end = [&]() {
+    copies_landed();
+    __syncthreads();
+  };
+
+  // Generic step (tiles at the edges of a wavefront's range, masked tiles, idle steps): the three
+  // pieces one after the other.
+  auto generic_steps = [&](int from, int to) {
+    for (int n = from; n <= to; ++n) {
+      const int par = n & 1;
+      step_begin(n);
+      if (pending) {
+        apply_pending_rescale();
+        pv_half((par ^ 1) * TILE, 0);
+        pv_half((par ^ 1) * TILE, 1);
+        pending = false;
+      }
+      if (is_active(n)) {
+        const int kv0 = tile_of(n) * kBN;
+        if (!(kv0 + kBN - 1 <= q_w_min && kv0 >= lo_w_max)) mask_scores(kv0);
+        const float mu = update_maximum();
+        probabilities_half(0, mu);
+        probabilities_half(1, mu);
+        pending = true;
+      }
+      if (is_active(n + 1)) {
+        qk_half((par ^ 1) * TILE, 0);
+        qk_half((par ^ 1) * TILE, 1);
+      }
+      step_end();
+    }
+  };
+  // Hot step: tile n fully visible, the previous and the next tile belong to this wavefront too.
+  // One basic block holds the delayed product of tile n-1, the softmax of tile n and S of tile
+  // n+1 (written into the registers of S(n) as soon as each half has been turned into P), so
+  // that the matrix pipe has work all along the vector work of the same wavefront.
+  auto hot_steps = [&](int from, int to) {
+    for (int n = from; n <= to; ++n) {
+      const int par = n & 1;
+      const int other = (par ^ 1) * TILE;   // V(n-1) and K(n+1) both sit in the other buffer
+      step_begin(n);
+      apply_pending_rescale();
+      const float mu = update_maximum();
+      pv_half(other, 0);
+      probabilities_half(0, mu);   // frees sc[0] ...
+      pv_half(other, 1);
+      qk_half(other, 0);           // ... for S(n+1), first half
+      probabilities_half(1, mu);
+      qk_half(other, 1);
+      step_end();
+    }
   };
 
   copies_landed();
   __syncthreads();
+  if (is_active(0)) {
+    qk_half(0, 0);
+    qk_half(0, 1);
+  }
 
-  // Step n (parity par = n & 1) works on tile(n): K(tile(n)) is in K buffer par and V of the
-  // previous step's tile in V buffer par^1.  Within each of the two runs of the rotated order
-  // the tiles of a wavefront come as masked ones at the window / document edge, fully visible
-  // ones, masked ones at the diagonal; the fully visible ones get a loop with one code path.
-  bool pending = false;   // wave-uniform: P of the last tile has not been multiplied into O yet
-  auto start_copies = [&](int tile, int n) {
-    if (n + 1 < n_tiles) copy_k(tile == t_hi ? t_lo : tile + 1, (n & 1) ^ 1);
-    copy_v(tile, n & 1);
-  };
-  auto generic_tiles = [&](int from, int to, int n) {
-    for (int tile = from; tile <= to; ++tile, ++n) {
-      const int par = n & 1;
-      start_copies(tile, n);
-      if (tile >= tw_lo && tile <= tw_hi) {
-        wave_tile(tile, par, std::true_type{});
-        pending = true;
-      } else if (pending) {
-        // the product of this wavefront's last tile, before its V buffer is reused
-        apply_pending_rescale();
-        pv_product((par ^ 1) * TILE);
-        clear_pfrag();   // the wavefront may become active again after the wrap
-        pending = false;
-      }
-      copies_landed();
-      __syncthreads();
-    }
-  };
   // Fully visible tiles of this wavefront: first key >= every row's lower bound, last key <=
-  // the first row.
-  int c_lo = max((lo_w_max + kBN - 1) / kBN, max(tw_lo, t_lo));
-  int c_hi = min((q_w_min + 1) / kBN - 1, min(tw_hi, t_hi));
-  if (c_hi < c_lo) { c_lo = t_hi + 1; c_hi = t_hi; }   // none: everything runs in the generic loops
+  // the first row.  A hot step needs such a tile with active neighbours in the same run of
+  // consecutive tiles (the rotated order has two runs: t_first..t_hi, then t_lo..t_first-1).
+  const int c_lo = max((lo_w_max + kBN - 1) / kBN, max(tw_lo, t_lo));
+  const int c_hi = min((q_w_min + 1) / kBN - 1, min(tw_hi, t_hi));
 #pragma nounroll
   for (int run = 0; run < 2; ++run) {
     const int a = run == 0 ? t_first : t_lo;
     const int b = run == 0 ? t_hi : t_first - 1;
-    const int n0 = run == 0 ? 0 : t_hi - t_first + 1;
-    generic_tiles(a, min(b, c_lo - 1), n0);
-    const int ca = max(a, c_lo), cb = min(b, c_hi);
-    for (int tile = ca, n = n0 + ca - a; tile <= cb; ++tile, ++n) {
-      const int par = n & 1;
-      start_copies(tile, n);
-      wave_tile(tile, par, std::false_type{});
-      pending = true;
-      copies_landed();
-      __syncthreads();
-    }
-    const int g = max(a, c_hi + 1);
-    generic_tiles(g, b, n0 + g - a);
+    const int n0 = run == 0 ? 0 : t_hi - t_first + 1;     // step of tile a
+    if (b < a) continue;
+    int ha = max(max(c_lo, a + 1), tw_lo + 1);
+    int hb = min(min(c_hi, b - 1), tw_hi - 1);
+    if (hb < ha) { ha = b + 1; hb = b; }                   // no hot tile in this run
+    generic_steps(n0, n0 + ha - 1 - a);
+    hot_steps(n0 + ha - a, n0 + hb - a);
+    generic_steps(n0 + hb + 1 - a, n0 + b - a);
   }
   if (pending) {
     apply_pending_rescale();
-    pv_product(((n_tiles - 1) & 1) * TILE);
+    pv_half(((n_tiles - 1) & 1) * TILE, 0);
+    pv_half(((n_tiles - 1) & 1) * TILE, 1);
   }
 
   const float l_tot = pair_sum(l_run);

@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu]
 
-NAME is one of prefill | module | long | decode | kda | copy; "copy" runs a plain 1 GiB
+NAME is one of prefill | ceiling | module | long | decode | kda | copy; "copy" runs a plain 1 GiB
 device copy and nothing else (the known-size kernel against which the HBM
 counters FETCH_SIZE / WRITE_SIZE are calibrated under rocprofv3 --pmc).
 
@@ -290,7 +290,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", default=None, help="prefill | module | long | decode | kda | copy (default: all but copy)")
+    ap.add_argument("--only", default=None, help="prefill | ceiling | module | long | decode | kda | copy (default: all but copy)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -308,6 +308,13 @@ def main():
     cpu = not args.no_cpu
     extra = {}
     head = bench_prefill_c2(args.steps, args.warmup, cpu) if want("prefill") else None
+    if want("ceiling"):
+        from daisy_amd import ops
+        extra["matrix_pipe_ceiling"] = {
+            "what": "register-only v_mfma_f32_32x32x16_bf16 on every SIMD, 2 wavefronts each, ~25 ms per run",
+            "mfma_only": ops.probe_matrix_rate(False, 80000),
+            "mfma_with_attention_vector_mix": ops.probe_matrix_rate(True, 60000),
+        }
     if want("module"):
         extra["module_c2"] = bench_module_c2(max(args.steps // 2, 4), max(args.warmup // 2, 2))
     if want("long"):

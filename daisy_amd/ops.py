@@ -315,3 +315,31 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
             B, T, H, D, float(eps), _lib.current_stream(dev))
     _lib.check(rc, "daisy_qkv_prep_fwd")
     return qo, ko, vo
+
+
+def probe_matrix_rate(with_vector_mix: bool, iters: int = 50000, workgroups: int = 256, device="cuda:0") -> dict:
+    """Sustained rate of register-only bf16 MFMAs on every SIMD (optionally with the attention loop's vector mix).
+
+    Returns ``{"ms", "tflops", "clock_mhz"}``; see ``daisy_probe_matrix_rate`` in ``include/daisy_hip.h``.
+    """
+    import ctypes
+    dev = torch.device(device)
+    sink = torch.empty(4096, dtype=torch.float32, device=dev)
+    ticks = torch.zeros(2 * workgroups, dtype=torch.int64, device=dev)
+    lib = _lib.load()
+    flop = ctypes.c_double(0.0)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.device(dev):
+        stream = _lib.current_stream(dev)
+        rc = lib.daisy_probe_matrix_rate(int(with_vector_mix), workgroups, max(iters // 10, 1), sink.data_ptr(),
+                                         ticks.data_ptr(), ctypes.byref(flop), stream)   # warm-up
+        _lib.check(rc, "daisy_probe_matrix_rate")
+        start.record()
+        rc = lib.daisy_probe_matrix_rate(int(with_vector_mix), workgroups, iters, sink.data_ptr(),
+                                         ticks.data_ptr(), ctypes.byref(flop), stream)
+        end.record()
+        _lib.check(rc, "daisy_probe_matrix_rate")
+        torch.cuda.synchronize(dev)
+    ms = start.elapsed_time(end)
+    t = ticks.view(workgroups, 2).double().sum(0)
+    return {"ms": ms, "tflops": flop.value / ms / 1e9, "clock_mhz": float(t[0] / t[1] * 100.0)}

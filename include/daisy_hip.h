@@ -207,6 +207,18 @@ int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
                        void* v_out, const int64_t* v_out_strides,
                        int B, int T, int H, int D, float eps, void* stream);
 
+/* ---------------------------------------------------------------------------
+ * Diagnostic (no counterpart in the reference): launches `workgroups` workgroups
+ * of 8 wavefronts (two per SIMD) that each issue 8 * iters independent
+ * v_mfma_f32_32x32x16_bf16 from registers -- alone (with_vector_mix = 0) or with
+ * 5 fma + 1 exp2 between consecutive MFMAs, the ratio of the attention inner
+ * loop (1).  The caller times the launch; *flop_out receives the flop count.
+ * sink: 4096 floats of scratch; ticks: 2 uint64 per workgroup = (shader clock
+ * counter, 100 MHz counter) deltas over the loop, i.e. the clock the chip ran at.
+ */
+int daisy_probe_matrix_rate(int with_vector_mix, int workgroups, int iters,
+                            float* sink, unsigned long long* ticks, double* flop_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

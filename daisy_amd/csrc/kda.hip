@@ -537,19 +537,58 @@ __global__ __launch_bounds__(64 * KSW, 1) void kda_state_kernel(KdaParams p) {
     }
     lds_cptr sb = stage0 + st * kStageBytes;
 
+    // LDS operands are read in two batches ahead of the MFMAs that use them (one wavefront per
+    // SIMD has the registers for it) instead of each next to its MFMA, where every MFMA waited
+    // for a full LDS latency.
+    bf16x8 wa[4][4], qa[4][4], pa[4][2], kh[8][2], kl[8][2];
+    f32x4 dc[8];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int m = 0; m < 4; ++m) wa[mt][m] = lds_bf16x8(sb + kStageWn + 4096 * mt + rd256[m]);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int m = 0; m < 4; ++m) qa[mt][m] = lds_bf16x8(sb + kStageQg + 4096 * mt + rd256[m]);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
+        if (32 * m <= 16 * mt + 15) pa[mt][m] = lds_bf16x8(sb + kStagePm + 2048 * mt + rd128[m]);
+
     bf16x8 Sb[4];
 #pragma unroll
     for (int m = 0; m < 4; ++m) Sb[m] = pack_acc2(S[2 * m], S[2 * m + 1]);
+    __builtin_amdgcn_sched_barrier(0);
 
-    // U = U0 + (-W) S0; tile mt: rows (positions) 16*mt + 4*q4 + r, column vcol.
-    f32x4 U[4];
+    // U = U0 + (-W) S0 and O = Qg S0: eight independent accumulator chains.
+    // Tile mt: rows (positions) 16*mt + 4*q4 + r, column vcol.
+    f32x4 U[4], O[4];
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
       U[mt] = u0c[mt];
-#pragma unroll
-      for (int m = 0; m < 4; ++m)
-        U[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lds_bf16x8(sb + kStageWn + 4096 * mt + rd256[m]), Sb[m], U[mt], 0, 0, 0);
+      O[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        U[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[mt][m], Sb[m], U[mt], 0, 0, 0);
+        O[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[mt][m], Sb[m], O[mt], 0, 0, 0);
+      }
+    }
+    // The operands of the state update are read while those 32 MFMAs run.
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) {
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+        kh[dt][m] = lds_bf16x8(sb + kStageKtH + 2048 * dt + rd128[m]);
+        kl[dt][m] = lds_bf16x8(sb + kStageKtL + 2048 * dt + rd128[m]);
+      }
+      dc[dt] = *(const f32x4 __attribute__((address_space(3)))*)(sb + kStageDec + 4 * (16 * dt + 4 * q4));
+    }
+    __builtin_amdgcn_sched_barrier(0);
     bf16x8 Uh[2], Ul[2];
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
@@ -563,38 +602,36 @@ __global__ __launch_bounds__(64 * KSW, 1) void kda_state_kernel(KdaParams p) {
       Ul[m] = pack_acc2(l0, l1);
     }
 
-    // O = Qg S0 + Pm U  (scale already folded into Qg and Pm)
+    // O += Pm U  (scale already folded into Qg and Pm; columns up to the diagonal only)
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
-      f32x4 O = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int m = 0; m < 4; ++m)
-        O = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lds_bf16x8(sb + kStageQg + 4096 * mt + rd256[m]), Sb[m], O, 0, 0, 0);
 #pragma unroll
       for (int m = 0; m < 2; ++m) {
-        if (32 * m <= 16 * mt + 15)   // columns up to the diagonal only
-          O = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lds_bf16x8(sb + kStagePm + 2048 * mt + rd128[m]), Uh[m], O, 0, 0, 0);
-      }
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int t = n * KC + 16 * mt + 4 * q4 + r;
-        if (t < p.T) p.o[(((int64_t)b * p.T + t) * p.H + h) * KD + vcol] = (uint16_t)(pack_bf16x2(O[r], 0.f) & 0xffffu);
+        if (32 * m <= 16 * mt + 15)
+          O[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[mt][m], Uh[m], O[mt], 0, 0, 0);
       }
     }
-
     // S = exp(G_last) (.) S + Kt^T U, with both operands split into two bf16 terms.
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
-      const f32x4 dc = *(const f32x4 __attribute__((address_space(3)))*)(sb + kStageDec + 4 * (16 * dt + 4 * q4));
 #pragma unroll
-      for (int r = 0; r < 4; ++r) S[dt][r] *= dc[r];
+      for (int r = 0; r < 4; ++r) S[dt][r] *= dc[dt][r];
+    }
 #pragma unroll
-      for (int m = 0; m < 2; ++m) {
-        const bf16x8 ah = lds_bf16x8(sb + kStageKtH + 2048 * dt + rd128[m]);
-        const bf16x8 al = lds_bf16x8(sb + kStageKtL + 2048 * dt + rd128[m]);
-        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, Uh[m], S[dt], 0, 0, 0);
-        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, Ul[m], S[dt], 0, 0, 0);
-        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, Uh[m], S[dt], 0, 0, 0);
+    for (int m = 0; m < 2; ++m) {
+#pragma unroll
+      for (int dt = 0; dt < 8; ++dt) {
+        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kh[dt][m], Uh[m], S[dt], 0, 0, 0);
+        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kh[dt][m], Ul[m], S[dt], 0, 0, 0);
+        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kl[dt][m], Uh[m], S[dt], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = n * KC + 16 * mt + 4 * q4 + r;
+        if (t < p.T) p.o[(((int64_t)b * p.T + t) * p.H + h) * KD + vcol] = (uint16_t)(pack_bf16x2(O[mt][r], 0.f) & 0xffffu);
       }
     }
 

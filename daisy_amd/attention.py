@@ -58,6 +58,34 @@ def build_window_mask(input_seq: Tensor, window_size: Optional[int], eos_token_i
     return WindowMask(window_size, ds)
 
 
+def build_block_window_masks(input_seq: Tensor, sliding_window_num_blocks, num_layers: int,
+                             eos_token_id: int, block: int = 128):
+    """Per-layer descriptors equal to the reference's training-time block masks
+    (``DaisyCore.create_blockmasks``, models/daisy/daisy_core.py:182-229).
+
+    There the window is counted in key blocks of ``block`` tokens: a query block sees its own
+    block and the ``w - 1`` blocks before it, element-wise restricted to ``k <= q`` and the query's
+    document.  Per query that is the single range ``[max(doc_start[q], (q // block - w + 1) * block), q]``,
+    which the attention kernel takes as a per-row lower bound.  Layers cycle long, short, short,
+    short, ... with the last layer long; short = long // 2.  Returns a list of ``num_layers``
+    ``WindowMask`` objects (two distinct ones) for ``CausalSelfAttention.forward(block_mask=...)``.
+    """
+    ids = input_seq.reshape(-1)
+    T = ids.numel()
+    torch._assert(T % block == 0, f"input_seq length {T} must be divisible by BLOCK_SIZE {block}")
+    w_long = int(sliding_window_num_blocks)
+    ds = doc_start_from_ids(ids, eos_token_id)
+    qblk = torch.arange(T, device=ids.device, dtype=torch.int32) // block
+
+    def one(w: int) -> WindowMask:
+        lo_blk = torch.clamp_min(qblk - (max(w, 1) - 1), 0) * block
+        return WindowMask(None, torch.maximum(ds, lo_blk).to(torch.int32).contiguous())
+
+    long_m, short_m = one(w_long), one(w_long // 2)
+    cycle = [long_m] + [short_m] * 3
+    return (cycle * ((num_layers + 3) // 4))[:num_layers - 1] + [long_m]
+
+
 def dense_mask_to_window(attn_mask: Tensor) -> WindowMask:
     """Converts a reference-style additive mask ``[..., T, T]`` to a ``WindowMask``.
 

@@ -41,6 +41,8 @@ from .attention import (  # noqa: F401
     rms_norm,
     build_attn_mask,
     doc_start_from_ids,
+    block_mask_dense,
+    block_mask_cycle,
     window_mask,
     sdpa,
     windowed_attention,

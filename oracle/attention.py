@@ -102,6 +102,54 @@ def doc_start_from_ids(input_seq: torch.Tensor, eos_token_id: int) -> torch.Tens
     return out
 
 
+def block_mask_dense(input_seq: torch.Tensor, window_blocks: int, eos_token_id: int, block: int = 128) -> torch.Tensor:
+    """Boolean ``[T, T]`` visibility of one training-time block mask.
+
+    models/daisy/daisy_core.py:182-221 (``create_blockmasks`` / ``build_bm``), restated block by
+    block with the semantics of ``BlockMask.from_kv_blocks``: per query block the key blocks that
+    touch it causally and by document are split into *full* ones (strictly earlier, every row of
+    both blocks in one document) and *partial* ones; both lists are ordered from the most recent
+    block backwards; the first ``min(n_full, w - 1)`` full blocks are visible everywhere, the first
+    ``min(n_partial, max(w - n_full, 1))`` partial blocks where ``q >= k`` and ``docs[q] == docs[k]``.
+    """
+    ids = input_seq.reshape(-1)
+    T = ids.numel()
+    assert T % block == 0
+    nb = T // block
+    docs = torch.cumsum((ids == eos_token_id).to(torch.int64), 0)
+    lo = docs.view(nb, block)[:, 0]
+    hi = docs.view(nb, block)[:, -1]
+    pos = torch.arange(T)
+    allowed = torch.zeros(T, T, dtype=torch.bool)
+    for i in range(nb):
+        full, partial = [], []
+        for j in range(i, -1, -1):                       # most recent first
+            any_ = (i >= j) and bool(lo[i] <= hi[j]) and bool(hi[i] >= lo[j])
+            all_ = (i > j) and bool(lo[i] == hi[j]) and bool(hi[i] == lo[j])
+            if any_ and all_:
+                full.append(j)
+            elif any_:
+                partial.append(j)
+        n_full = len(full)
+        keep_partial = partial[:min(len(partial), max(window_blocks - n_full, 1))]
+        keep_full = full[:min(n_full, max(window_blocks - 1, 0))]
+        qs = pos[i * block:(i + 1) * block]
+        for j in keep_full:
+            allowed[i * block:(i + 1) * block, j * block:(j + 1) * block] = True
+        for j in keep_partial:
+            ks = pos[j * block:(j + 1) * block]
+            m = (qs[:, None] >= ks[None, :]) & (docs[qs][:, None] == docs[ks][None, :])
+            allowed[i * block:(i + 1) * block, j * block:(j + 1) * block] = m
+    return allowed
+
+
+def block_mask_cycle(num_layers: int, window_blocks: int):
+    """Per-layer window (in blocks): long, short, short, short, ... and long for the last layer
+    (models/daisy/daisy_core.py:224-229); short = long // 2."""
+    cycle = [window_blocks] + [window_blocks // 2] * 3
+    return (cycle * ((num_layers + 3) // 4))[:num_layers - 1] + [window_blocks]
+
+
 def window_mask(T: int, window: Optional[int], doc_start: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Same mask as ``build_attn_mask`` expressed through (window, doc_start)."""
     pos = torch.arange(T)

@@ -190,3 +190,27 @@ def test_generator_ring_path_matches_full_prefill():
         assert gen.cache.t == seq.numel()
         out = [int(t) for t in gen.generate(prompt, max_new_tokens=5)]
         assert len(out) == 5
+
+
+def test_forward_with_training_block_masks():
+    """forward(block_mask=...) with the descriptors of build_block_window_masks equals dense attention under the
+    reference's block-mask visibility (models/daisy/daisy_core.py:182-229), for the long and the short window."""
+    from daisy_amd import build_block_window_masks
+    dim, H, D, T, w_blocks, L = 256, 2, 128, 640, 3, 4
+    attn = _make(dim, H, D, seed=5).to(DEV)
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(1, T, dim, generator=g).bfloat16()
+    ids = torch.randint(2, 40, (T,), generator=g)
+    ids[[70, 300, 301, 511]] = 1
+    masks = build_block_window_masks(ids.to(DEV), w_blocks, L, eos_token_id=1)
+    widths = oracle.block_mask_cycle(L, w_blocks)
+    w = attn.qkvo_w.detach().cpu()
+    cos, sin = attn.rotary.cos.cpu(), attn.rotary.sin.cpu()
+    q, k, v = oracle.calc_qkv(x, w, H, D, cos, sin)
+    for layer in (0, 1):                       # long, short
+        vis = oracle.block_mask_dense(ids, widths[layer], eos_token_id=1)
+        add = torch.zeros(T, T).masked_fill(~vis, float("-inf"))
+        o = oracle.sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), add, 0.12).transpose(1, 2)
+        y_ref = torch.nn.functional.linear(o.reshape(1, T, dim).to(w.dtype), w[3])
+        y = attn(x.to(DEV), None, block_mask=masks[layer])
+        assert_close_bf16(y, y_ref, f"y (window of {widths[layer]} blocks)")

@@ -254,12 +254,82 @@ static int resolve_nsplit(int B, int H, int n_rows, int nsplit) {
   return (n_rows + rps - 1) / rps;
 }
 
+// Any even head dim up to 256 (the reference's unit tests use 2 and 8): one wavefront per
+// (batch, head), lane l owns channels l, l + 64, ...; rows are visited one after the other with a
+// wavefront-wide reduction per score.  Correctness path for small shapes, not a fast one.
+__global__ __launch_bounds__(64) void decode_scalar_kernel(DecodeParams p, int D) {
+  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+  const int half = D / 2;
+  const uint16_t* qp = p.q + b * p.q_sb + h * p.q_sh;
+  const uint16_t* knp = p.k_new + b * p.kn_sb + h * p.kn_sh;
+  const uint16_t* vnp = p.v_new + b * p.vn_sb + h * p.vn_sh;
+  uint16_t* kc = p.kc + b * p.kc_sb + h * p.kc_sh;
+  uint16_t* vc = p.vc + b * p.vc_sb + h * p.vc_sh;
+  float qv[4], kn[4], vn[4], acc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    qv[i] = kn[i] = vn[i] = acc[i] = 0.f;
+    if (d < D) {
+      float x = bf16lo_to_f32(qp[d]), y = bf16lo_to_f32(knp[d]);
+      if (p.cos_row != nullptr) {
+        const bool lower = d < half;
+        const int dp = lower ? d + half : d - half;   // RoPE partner channel
+        const float c = p.cos_row[lower ? d : dp], sn = p.sin_row[lower ? d : dp];
+        const float xp = bf16lo_to_f32(qp[dp]), yp = bf16lo_to_f32(knp[dp]);
+        x = round_bf16(lower ? rope_lo(x, xp, c, sn) : rope_hi(xp, x, c, sn));
+        y = round_bf16(lower ? rope_lo(y, yp, c, sn) : rope_hi(yp, y, c, sn));
+      }
+      qv[i] = x;
+      kn[i] = y;
+      vn[i] = bf16lo_to_f32(vnp[d]);
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+  for (int r = 0; r < p.n_rows; ++r) {
+    const bool is_new = r == p.new_idx;
+    float kr[4], vr[4], part = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      kr[i] = vr[i] = 0.f;
+      if (d < D) {
+        kr[i] = is_new ? kn[i] : bf16lo_to_f32(kc[(int64_t)r * p.kc_sr + d]);
+        vr[i] = is_new ? vn[i] : bf16lo_to_f32(vc[(int64_t)r * p.vc_sr + d]);
+      }
+      part += qv[i] * kr[i];
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) part += __shfl_xor(part, off);
+    const float s = part * p.scale_log2e;
+    const float m_new = fmaxf(m, s);
+    const float alpha = fast_exp2(m - m_new), pr = fast_exp2(s - m_new);
+    l = l * alpha + pr;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = acc[i] * alpha + pr * vr[i];
+    m = m_new;
+  }
+  uint16_t* op = p.o + b * p.o_sb + h * p.o_sh;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < D) {
+      op[d] = (uint16_t)(pack_bf16x2(acc[i] / l, 0.f) & 0xffffu);
+      if (p.write_back) {
+        kc[(int64_t)p.new_idx * p.kc_sr + d] = (uint16_t)(pack_bf16x2(kn[i], 0.f) & 0xffffu);
+        vc[(int64_t)p.new_idx * p.vc_sr + d] = (uint16_t)(pack_bf16x2(vn[i], 0.f) & 0xffffu);
+      }
+    }
+  }
+}
+
 }  // namespace daisy
 
 using namespace daisy;
 
 extern "C" size_t daisy_decode_workspace_bytes(int B, int H, int D, int n_rows, int nsplit) {
   if (B <= 0 || H <= 0 || D <= 0 || n_rows <= 0) return 0;
+  if (D != 64 && D != 128) return 0;   // the small-head-dim kernel never splits
   const int ns = resolve_nsplit(B, H, n_rows, nsplit);
   if (ns == 1) return 0;
   return (size_t)B * H * ns * (D + 2) * sizeof(float);
@@ -280,7 +350,8 @@ extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
   DAISY_CHECK_ARG(q_strides && k_new_strides && v_new_strides && o_strides, "decode: stride arrays must be non-NULL");
   DAISY_CHECK_ARG(B > 0 && H > 0, "decode: B=%d and H=%d must be positive", B, H);
   DAISY_CHECK_ARG(B <= 65535 && H <= 65535, "decode: B=%d and H=%d must each be <= 65535", B, H);
-  DAISY_CHECK_SUPPORTED(D == 64 || D == 128, "decode: head_dim %d not supported (64 or 128)", D);
+  DAISY_CHECK_SUPPORTED(D >= 2 && D <= 256 && D % 2 == 0, "decode: head_dim %d not supported (even, 2..256)", D);
+  const bool fast = D == 64 || D == 128;
   DAISY_CHECK_ARG(n_rows >= 1, "decode: n_rows=%d must be >= 1 (the new token is always attended)", n_rows);
   DAISY_CHECK_ARG(new_idx >= 0 && new_idx < n_rows, "decode: new_idx=%d outside [0, %d)", new_idx, n_rows);
   DAISY_CHECK_ARG((cos_row == nullptr) == (sin_row == nullptr), "decode: cos_row and sin_row must both be given or both NULL");
@@ -288,16 +359,16 @@ extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
                   "decode: cache pointers and strides are required when n_rows > 1");
   DAISY_CHECK_ARG(!write_back || (k_cache && v_cache), "decode: write_back needs cache pointers");
   auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
-  DAISY_CHECK_ARG(al16(q) && al16(k_new) && al16(v_new) && al16(o) && al16(k_cache) && al16(v_cache),
+  DAISY_CHECK_ARG(!fast || (al16(q) && al16(k_new) && al16(v_new) && al16(o) && al16(k_cache) && al16(v_cache)),
                   "decode: tensors must be 16-byte aligned");
   static const int64_t zero3[3] = {0, 0, 0};
   if (!k_cache_strides) k_cache_strides = zero3;
   if (!v_cache_strides) v_cache_strides = zero3;
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < 2 && fast; ++i) {
     DAISY_CHECK_ARG(q_strides[i] % 8 == 0 && k_new_strides[i] % 8 == 0 && v_new_strides[i] % 8 == 0 && o_strides[i] % 8 == 0,
                     "decode: vector strides must be multiples of 8 elements");
   }
-  for (int i = 0; i < 3; ++i) {
+  for (int i = 0; i < 3 && fast; ++i) {
     DAISY_CHECK_ARG(k_cache_strides[i] % 8 == 0 && v_cache_strides[i] % 8 == 0,
                     "decode: cache strides must be multiples of 8 elements");
   }
@@ -317,7 +388,7 @@ extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
   p.cos_row = cos_row; p.sin_row = sin_row;
   p.o = (uint16_t*)o; p.o_sb = o_strides[0]; p.o_sh = o_strides[1];
   p.B = B; p.H = H; p.n_rows = n_rows; p.new_idx = new_idx; p.write_back = write_back;
-  p.nsplit = resolve_nsplit(B, H, n_rows, nsplit);
+  p.nsplit = fast ? resolve_nsplit(B, H, n_rows, nsplit) : 1;
   p.rows_per_split = (n_rows + p.nsplit - 1) / p.nsplit;
   p.scale_log2e = scale * kLog2e;
   p.partials = nullptr;
@@ -331,6 +402,11 @@ extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
   }
 
   hipStream_t s = (hipStream_t)stream;
+  if (!fast) {
+    hipLaunchKernelGGL(decode_scalar_kernel, dim3(H, B), dim3(64), 0, s, p, D);
+    DAISY_CHECK_LAUNCH("decode_scalar_kernel");
+    return DAISY_OK;
+  }
   dim3 grid(p.nsplit, H, B);
   if (D == 128) {
     hipLaunchKernelGGL(decode_kernel<128>, grid, dim3(kDecodeThreads), 0, s, p);

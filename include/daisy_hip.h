@@ -107,7 +107,8 @@ int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
  * workspace          : >= daisy_decode_workspace_bytes(...) bytes, 256-byte
  *                      aligned; may be NULL when that function returns 0.
  * nsplit             : number of sequence splits per (b, h); 0 = choose.
- * D must be 64 or 128.
+ * D is 64 or 128 for the streaming kernel; any other even D <= 256 runs a
+ * one-wavefront-per-(batch, head) kernel meant for small test shapes (no splits).
  */
 size_t daisy_decode_workspace_bytes(int B, int H, int D, int n_rows, int nsplit);
 

@@ -70,7 +70,8 @@ def test_decode_argument_errors():
     def call(D=128, n_rows=4, new_idx=0, kc=p, ws=None, ws_bytes=0, nsplit=1):
         return lib.daisy_decode_fwd(p, s2, p, s2, p, s2, kc, s3, kc, s3, None, None, p, s2, 1, 1, D,
                                     n_rows, new_idx, 0, 0.12, nsplit, ws, ws_bytes, None)
-    assert call(D=32) == -2 and "head_dim" in _err()
+    assert call(D=33) == -2 and "head_dim" in _err()
+    assert call(D=258) == -2 and "head_dim" in _err()
     assert call(new_idx=4) == -1 and "new_idx" in _err()
     assert call(n_rows=0) == -1
     assert call(kc=None) == -1 and "cache pointers" in _err()

@@ -97,5 +97,31 @@ def test_decode_rejects_bad_arguments():
     with pytest.raises(RuntimeError, match="new_idx"):
         ops.decode_attention(z, z, z, rows, rows, n_rows=4, new_idx=4, write_back=False)
     with pytest.raises(RuntimeError, match="head_dim"):
-        y = torch.zeros(1, 1, 32, dtype=torch.bfloat16, device="cuda:0")
+        y = torch.zeros(1, 1, 33, dtype=torch.bfloat16, device="cuda:0")
         ops.decode_attention(y, y, y, None, None, n_rows=1, new_idx=0, write_back=False)
+
+
+@pytest.mark.parametrize("D,n_rows,rope", [(8, 13, True), (2, 5, True), (32, 70, False), (200, 9, True)])
+def test_decode_small_head_dims(D, n_rows, rope):
+    """Head dims other than 64/128 (the reference's own unit tests use 2 and 8): the one-wavefront kernel."""
+    B, H = 2, 3
+    g = torch.Generator().manual_seed(D + n_rows)
+    kc = torch.randn(B, H, n_rows, D, generator=g).bfloat16()
+    vc = torch.randn(B, H, n_rows, D, generator=g).bfloat16()
+    q, kn, vn = (torch.randn(B, H, D, generator=g).bfloat16() for _ in range(3))
+    new_idx = n_rows // 2
+    cos = sin = None
+    qr, knr = q, kn
+    if rope:
+        cos_t, sin_t = oracle.rope_tables(D, 40)
+        cos, sin = cos_t[17].contiguous(), sin_t[17].contiguous()
+        qr = oracle.apply_rope(q[:, None], cos[None], sin[None])[:, 0]
+        knr = oracle.apply_rope(kn[:, None], cos[None], sin[None])[:, 0]
+    ke, ve = kc.clone(), vc.clone()
+    ke[:, :, new_idx], ve[:, :, new_idx] = knr, vn
+    ref = oracle.sdpa(qr[:, :, None], ke, ve, None, 0.12)[:, :, 0]
+    dk, dv = kc.cuda(), vc.cuda()
+    o = ops.decode_attention(q.cuda(), kn.cuda(), vn.cuda(), dk, dv, n_rows=n_rows, new_idx=new_idx, write_back=True,
+                             cos_row=None if cos is None else cos.cuda(), sin_row=None if sin is None else sin.cuda())
+    assert_close_bf16(o, ref, f"o (D={D})")
+    assert torch.equal(dk.cpu(), ke) and torch.equal(dv.cpu(), ve), "the new row must be appended rotated, bit for bit"

@@ -214,3 +214,25 @@ def test_forward_with_training_block_masks():
         y_ref = torch.nn.functional.linear(o.reshape(1, T, dim).to(w.dtype), w[3])
         y = attn(x.to(DEV), None, block_mask=masks[layer])
         assert_close_bf16(y, y_ref, f"y (window of {widths[layer]} blocks)")
+
+
+@pytest.mark.parametrize("dim,H,D,T,W", [(2, 1, 2, 131, 128), (16, 2, 8, 12, 12), (16, 2, 8, 8, 16), (16, 2, 8, 20, 2)])
+def test_forward_equals_steps_at_the_reference_tests_shapes(dim, H, D, T, W):
+    """The shapes of the reference's own unit tests (tests/test_causal_self_attention_equivalence.py:15-52: H=1, D=2;
+    tests/test_attention.py:80-146: dim 16, H=2, D=8, window 2 included): head dims the fast kernels do not take."""
+    attn = _make(dim, H, D, seed=7).to(DEV)
+    with torch.no_grad():
+        attn.qkvo_w.copy_((torch.randn(4, dim, dim, generator=torch.Generator().manual_seed(8)) * 0.5).bfloat16())
+    x = torch.randn(1, T, dim, generator=torch.Generator().manual_seed(9)).bfloat16().to(DEV)
+    y_full = attn(x, None, attn_mask=WindowMask(W))
+    w = attn.qkvo_w.detach().cpu()
+    y_ref, _, _ = oracle.attn_prefill(x.cpu(), w, H, D, attn.rotary.cos.cpu()[:T], attn.rotary.sin.cpu()[:T], W)
+    assert_close_bf16(y_full, y_ref, "forward vs oracle", max_abs=3e-2, mean_abs=4e-3)
+    K = torch.empty(1, 0, H, D, device=DEV, dtype=torch.bfloat16)
+    V = torch.empty(1, 0, H, D, device=DEV, dtype=torch.bfloat16)
+    ys = []
+    for pos in range(T):
+        y, k_new, v_new = attn.step(x[:, pos:pos + 1], k_ctx=K, v_ctx=V, pos=pos, ve=None, window=W)
+        K, V = torch.cat([K, k_new], 1), torch.cat([V, v_new], 1)
+        ys.append(y)
+    assert torch.allclose(y_full.float(), torch.cat(ys, 1).float(), atol=2e-2, rtol=2e-2)

@@ -851,8 +851,10 @@ __global__ __launch_bounds__(256) void rope_k_kernel(PrefillParams p) {
   const uint16_t* kp = p.k + b * p.k_sb + (int64_t)t * p.k_st + h * p.k_sh + 8 * ch;
   uint16_t* op = p.k_out + b * p.ko_sb + (int64_t)t * p.ko_st + h * p.ko_sh + 8 * ch;
   float x1[8], x2[8], y1[8], y2[8];
-  unpack8(*reinterpret_cast<const u32x4*>(kp), x1);
-  unpack8(*reinterpret_cast<const u32x4*>(kp + HALF), x2);
+  // The unrotated keys are not needed again: read them past the caches, so that q, v and the
+  // rotated keys this pass writes are what the attention kernel finds there.
+  unpack8(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp)), x1);
+  unpack8(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp + HALF)), x2);
   const float* cr = p.cos + (int64_t)t * HALF + 8 * ch;
   const float* sr = p.sin + (int64_t)t * HALF + 8 * ch;
 #pragma unroll

@@ -1,0 +1,185 @@
+"""Kimi Delta Attention layer with the reference's module layout (models/daisy/attention_kimi.py:64-200).
+
+Same parameters and names as the reference's ``KimiLinearSelfAttention`` (``q_proj``, ``k_proj``,
+``v_proj``, ``q_conv1d.weight`` ..., ``f_proj``, ``b_proj``, ``A_log``, ``dt_bias``, ``g_proj``,
+``o_norm.weight``, ``o_proj``), the interface of ``AttentionProtocol``
+(models/daisy/attention_protocol.py:4-42) -- the reference's own ``forward`` / ``prefill`` /
+``step`` pass five arguments to a four-argument ``_forward_core`` and use an undefined
+``sa_lambdas``, so they cannot run as written -- and the arithmetic of ``_forward_core``:
+
+    q, k, v = silu(causal_conv4(proj(x)))          short depthwise convolutions, state kept for decode
+    g       = -exp(A_log) * softplus(f_proj(x) + dt_bias)       (``fused_kda_gate``)
+    beta    = sigmoid(b_proj(x)) in fp32
+    o, S    = chunk_kda(q, k, v, g, beta, S0, use_qk_l2norm_in_kernel=True)
+    y       = o_proj(rms_norm(o) * o_norm.weight * sigmoid(g_proj(x)))
+
+The delta-rule core runs on the HIP kernels (``chunk_kda`` for sequences, ``fused_recurrent_kda``
+with the state updated in place for single-token steps); projections, the four-tap convolution
+and the gated norm are PyTorch ops.  Three pieces of the reference come from the absent
+``flash-linear-attention`` package and are restated from their documented behaviour, not pinned
+against it: ``ShortConvolution`` (depthwise causal conv + SiLU with a ``[B, C, K]`` state) and
+the gated RMS norm (``FusedRMSNormGated(activation="sigmoid", eps=1e-5)``, the module the
+reference's ``CompilableFusedRMSNormGated`` stands in for), and ``chunk_kda``'s conventions.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from .kda import chunk_kda, fused_kda_gate, fused_recurrent_kda
+
+
+class ShortConvolution(nn.Module):
+    """Depthwise causal 1-D convolution + SiLU over ``[B, T, C]`` with a carried window.
+
+    ``weight [C, 1, K]`` like a grouped ``nn.Conv1d``.  ``cache [B, C, K]`` holds the last K
+    inputs (zeros before the sequence starts); the returned cache continues the sequence.
+    """
+
+    def __init__(self, hidden_size: int, kernel_size: int, activation: str = "silu", bias: bool = False,
+                 dtype=torch.bfloat16):
+        super().__init__()
+        assert activation == "silu"
+        self.hidden_size, self.kernel_size = hidden_size, kernel_size
+        w = torch.empty(hidden_size, 1, kernel_size, dtype=dtype)
+        nn.init.kaiming_uniform_(w, a=5 ** 0.5)
+        self.weight = nn.Parameter(w)
+        self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=dtype)) if bias else None
+
+    def forward(self, x: Tensor, cache: Optional[Tensor] = None, output_final_state: bool = False
+                ) -> Tuple[Tensor, Optional[Tensor]]:
+        B, T, C = x.shape
+        K = self.kernel_size
+        xt = x.transpose(1, 2)                                        # [B, C, T]
+        prev = cache[..., 1:] if cache is not None else xt.new_zeros(B, C, K - 1)
+        window = torch.cat([prev.to(xt.dtype), xt], dim=-1)           # [B, C, K - 1 + T]
+        y = F.conv1d(window, self.weight, self.bias, groups=C)        # [B, C, T]
+        new_cache = None
+        if output_final_state:
+            tail = window[..., -K:]
+            new_cache = tail if tail.shape[-1] == K else F.pad(tail, (K - tail.shape[-1], 0))
+        return F.silu(y).transpose(1, 2).contiguous(), new_cache
+
+
+class GatedRMSNorm(nn.Module):
+    """``rms_norm(x, eps) * weight * sigmoid(gate)`` over the last dim (fp32 statistics)."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-5, dtype=torch.bfloat16):
+        super().__init__()
+        self.hidden_size, self.eps = hidden_size, eps
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype))
+
+    def forward(self, x: Tensor, gate: Tensor) -> Tensor:
+        xf = x.float()
+        normed = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()
+        return (normed * torch.sigmoid(gate.float())).to(x.dtype)
+
+
+class KimiLinearSelfAttention(nn.Module):
+    """Linear-attention layer on the KDA kernels; see the module docstring.
+
+    ``ve`` is accepted for interface compatibility; it is mixed into v as in ``CausalSelfAttention``
+    (``sigmoid(g_ve) * v + (1 - sigmoid(g_ve)) * ve``) when ``receives_ve`` is set and ignored
+    otherwise (the reference leaves this as a TODO).  ``attn_mask`` is accepted and ignored (the
+    recurrence is causal by construction, a window does not apply, and variable-length packing
+    through a padding mask is not supported); ``block_mask`` must be None as in the reference.
+    """
+
+    def __init__(self, dim: int, num_heads: int, max_seq_len: int, head_dim: int, expand_v: float = 1.0,
+                 mode: str = "chunk", use_short_conv: bool = True, allow_neg_eigval: bool = False, conv_size: int = 4,
+                 conv_bias: bool = False, layer_idx: int = 0, receives_ve: bool = False):
+        assert not allow_neg_eigval, "allow_neg_eigval is not supported"
+        assert mode == "chunk", "mode must be 'chunk' (single-token steps use the recurrent kernel by themselves)"
+        super().__init__()
+        self.hidden_size, self.num_heads, self.head_dim = dim, num_heads, head_dim
+        self.head_k_dim, self.head_v_dim = head_dim, int(head_dim * expand_v)
+        torch._assert(self.head_k_dim == 128 and self.head_v_dim == 128, "the KDA kernels need head_dim 128 and expand_v 1")
+        self.key_dim, self.value_dim = num_heads * self.head_k_dim, num_heads * self.head_v_dim
+        self.use_short_conv, self.conv_size, self.layer_idx = use_short_conv, conv_size, layer_idx
+        bf = torch.bfloat16
+        self.q_proj = nn.Linear(dim, self.key_dim, bias=False, dtype=bf)
+        self.k_proj = nn.Linear(dim, self.key_dim, bias=False, dtype=bf)
+        self.v_proj = nn.Linear(dim, self.value_dim, bias=False, dtype=bf)
+        if use_short_conv:
+            self.q_conv1d = ShortConvolution(self.key_dim, conv_size, bias=conv_bias, dtype=bf)
+            self.k_conv1d = ShortConvolution(self.key_dim, conv_size, bias=conv_bias, dtype=bf)
+            self.v_conv1d = ShortConvolution(self.value_dim, conv_size, bias=conv_bias, dtype=bf)
+        self.f_proj = nn.Sequential(nn.Linear(dim, self.head_v_dim, bias=False, dtype=bf),
+                                    nn.Linear(self.head_v_dim, self.key_dim, bias=False, dtype=bf))
+        self.b_proj = nn.Linear(dim, num_heads, bias=False, dtype=bf)
+        self.A_log = nn.Parameter(torch.log(torch.empty(num_heads, dtype=torch.float32).uniform_(1, 16)).view(1, 1, -1, 1))
+        self.A_log._no_weight_decay = True
+        self.dt_bias = nn.Parameter(torch.zeros(self.key_dim, dtype=torch.float32))
+        self.dt_bias._no_weight_decay = True
+        self.g_proj = nn.Sequential(nn.Linear(dim, self.head_v_dim, bias=False, dtype=bf),
+                                    nn.Linear(self.head_v_dim, self.value_dim, bias=True, dtype=bf))
+        self.o_norm = GatedRMSNorm(self.head_v_dim, eps=1e-5, dtype=bf)
+        self.o_proj = nn.Linear(self.value_dim, dim, bias=False, dtype=bf)
+        self.receives_ve = receives_ve
+        self.g_ve = nn.Parameter(torch.tensor(0.0)) if receives_ve else None
+        self._recurrent_state: Optional[Tensor] = None
+        self._conv_state = None
+        self._seen = 0
+
+    def _apply(self, fn, recurse=True):
+        # The decay parameters stay fp32 under module-wide casts, as the reference creates them.
+        super()._apply(fn, recurse)
+        for name in ("A_log", "dt_bias"):
+            prm = getattr(self, name)
+            if prm.dtype != torch.float32:
+                prm.data = prm.data.float()
+        return self
+
+    def reset_history(self):
+        self._recurrent_state = None
+        self._conv_state = None
+        self._seen = 0
+
+    def _core(self, x: Tensor, ve: Optional[Tensor], use_cache: bool) -> Tensor:
+        B, T, _ = x.shape
+        H, Dk, Dv = self.num_heads, self.head_k_dim, self.head_v_dim
+        x = x.to(self.q_proj.weight.dtype)
+        state = self._recurrent_state if use_cache else None
+        convs = self._conv_state if (use_cache and self._conv_state is not None) else (None, None, None)
+        if self.use_short_conv:
+            q, cq = self.q_conv1d(self.q_proj(x), convs[0], use_cache)
+            k, ck = self.k_conv1d(self.k_proj(x), convs[1], use_cache)
+            v, cv = self.v_conv1d(self.v_proj(x), convs[2], use_cache)
+        else:
+            q, k, v = F.silu(self.q_proj(x)), F.silu(self.k_proj(x)), F.silu(self.v_proj(x))
+            cq = ck = cv = None
+        q, k, v = q.view(B, T, H, Dk), k.view(B, T, H, Dk), v.view(B, T, H, Dv)
+        if self.receives_ve:
+            torch._assert(ve is not None, "ve must be provided when receives_ve=True")
+            g_x = torch.sigmoid(self.g_ve).to(v.dtype)
+            v = g_x * v + (1.0 - g_x) * ve.view_as(v).to(v.dtype)
+        g = fused_kda_gate(self.f_proj(x), self.A_log, Dk, self.dt_bias)
+        beta = torch.sigmoid(self.b_proj(x)).to(torch.float32)
+        if use_cache and T == 1 and state is not None:
+            o, state = fused_recurrent_kda(q, k, v, g, beta, initial_state=state, use_qk_l2norm_in_kernel=True,
+                                           inplace_state=True)
+        else:
+            o, state = chunk_kda(q, k, v, g, beta, initial_state=state, output_final_state=use_cache,
+                                 use_qk_l2norm_in_kernel=True)
+        if use_cache:
+            self._recurrent_state = state
+            self._conv_state = (cq, ck, cv)
+            self._seen += T
+        gate = self.g_proj(x).view(B, T, H, Dv)
+        o = self.o_norm(o.to(gate.dtype), gate)
+        return self.o_proj(o.reshape(B, T, H * Dv))
+
+    def forward(self, x: Tensor, ve: Optional[Tensor], attn_mask=None, block_mask=None) -> Tensor:
+        assert block_mask is None, "block_mask not supported for KimiLinearSelfAttention"
+        return self._core(x, ve, use_cache=False)
+
+    def prefill(self, x: Tensor, ve: Optional[Tensor], attn_mask=None, debug: bool = False):
+        """Runs the prompt and keeps the recurrent and convolution states; there is no K/V to cache."""
+        return self._core(x, ve, use_cache=True), None, None
+
+    def step(self, x: Tensor, k_ctx, v_ctx, pos: int, ve: Optional[Tensor], window: Optional[int]):
+        torch._assert(x.size(1) == 1, "step() requires single position only")
+        return self._core(x, ve, use_cache=True), None, None

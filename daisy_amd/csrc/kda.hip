@@ -79,22 +79,19 @@ __host__ __device__ constexpr int perm32_inv(int p) { return (p & ~0x1c) | ((p &
 
 __device__ __forceinline__ f32x4 lds_f4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 
-// Packed storage of A^T (AT[j][i] = A_ij, j < i): row j keeps the entries i >= at_first(j), the
-// multiple of 4 at or below j + 1, so that every row starts 16-byte aligned; rows follow each other.
-__host__ __device__ constexpr int at_first(int j) { return 4 * ((j + 1) >> 2); }
-__host__ __device__ constexpr int at_off(int j) {
-  const int m = (j + 1) >> 2;
-  const int before = (m >= 1) ? 192 + 256 * (m - 1) - 8 * m * (m - 1) : 0;
-  const int idx = (m == 0) ? j : ((j + 1) & 3);
-  return before + idx * (KC - 4 * m);
-}
-constexpr int kAtPacked = at_off(KC - 2) + 4;   // row 62 is the last one with entries
+// Off-diagonal 16x16 blocks of A in LDS: block (I, J), J < I, has index I(I-1)/2 + J.
+__host__ __device__ constexpr int off_block(int I, int J) { return I * (I - 1) / 2 + J; }
+
+// A float as two bf16 terms (value = hi + lo up to 2^-17 relative).
+__device__ __forceinline__ void split_bf16(float x, float& hi, float& lo) { hi = round_bf16(x); lo = x - hi; }
 
 __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   __shared__ __attribute__((aligned(16))) float G[KC][KD];           // inclusive running log-decay; later staging for Wn
   __shared__ __attribute__((aligned(16))) uint16_t Kr[KC][KD + 8];   // k as given (bf16)
   __shared__ __attribute__((aligned(16))) uint16_t QV[KC][KD + 8];   // q as given; v as given once A and P are done
-  __shared__ __attribute__((aligned(16))) float ATp[kAtPacked];      // A^T, strictly lower part, rows packed (at_off)
+  __shared__ __attribute__((aligned(16))) float Ad[4][16][16];       // diagonal blocks of A, [block][column j][row i]; later T = (I + A_II)^-1 as bf16 hi | lo
+  __shared__ __attribute__((aligned(16))) uint16_t AoH[6][16][16];   // -A, off-diagonal blocks (off_block), [row][column], bf16 high term
+  __shared__ __attribute__((aligned(16))) uint16_t AoL[6][16][16];   //   ... low term
   __shared__ float rk[KC], rq[KC], bt[KC];                           // 1/|k|, 1/|q|, beta (0 for padded rows)
   __shared__ int steep[4];                                           // per 16-row block: total decay beyond exp(-80)
   auto& Qr = QV;
@@ -248,12 +245,25 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
     // accumulator: lane holds column j = 16J + li, rows i = 16I + 4*q4 + r
     const int j = 16 * J + li;
     const float rkj = rk[j];
+    f32x4 av;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int i = 16 * I + 4 * q4 + r;
-      if (j < i) ATp[at_off(j) + i - at_first(j)] = bt[i] * rk[i] * rkj * accA[r];
+      av[r] = bt[i] * rk[i] * rkj * accA[r];
       const float pv = (j <= i) ? p.scale * rq[i] * rkj * accP[r] : 0.f;
       p.Pm[(ci * KC + i) * KC + perm32(j)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
+    }
+    if (I == J) {
+      *reinterpret_cast<f32x4*>(&Ad[I][li][4 * q4]) = av;   // entries with i <= j are never read
+    } else {
+      const int ob = off_block(I, J);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float hi, lo;
+        split_bf16(-av[r], hi, lo);
+        AoH[ob][4 * q4 + r][li] = (uint16_t)(pack_bf16x2(hi, 0.f) & 0xffffu);
+        AoL[ob][4 * q4 + r][li] = (uint16_t)(pack_bf16x2(lo, 0.f) & 0xffffu);
+      }
     }
   };
   {
@@ -328,7 +338,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       if ((j & 3) == dq) {
         const int rj = 16 * I + j;
         const float rkj = rk[rj];
-        if (j < il) ATp[at_off(rj) + ri - at_first(rj)] = bi * rkj * av;
+        if (j < il) Ad[I][j][il] = bi * rkj * av;
         pv = (j <= il) ? qs * rkj * pv : 0.f;
         p.Pm[(ci * KC + ri) * KC + perm32(rj)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
       }
@@ -361,53 +371,128 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   }
   __syncthreads();   // V is in place
 
-  // ---- phase 4: forward substitution (I + A) X = diag(beta) [exp(G) K | V] ----
-  // One thread per right-hand-side column; the column lives in registers.
+  // ---- phase 4: (I + A) X = diag(beta) [exp(G) K | V] by blocks of 16 rows on MFMA ----
+  //     X_I = T_I (B_I - sum_{J<I} A_IJ X_J),   T_I = (I + A_II)^-1.
+  // The 256 right-hand-side columns form 16 tiles of 16; wavefront w solves tiles w, w+4 (W part)
+  // and w+8, w+12 (U part).  In the 16x16x32 MFMA a lane's accumulator holds rows 4q..4q+3 of a
+  // block for one column; the same four values, split into two bf16 terms, are that lane's
+  // share of the next product's right operand when contraction slot (q, e) stands for row
+  // 4q+e of block J (e < 4) and of block J+1 (e >= 4) -- so X never leaves the registers.  The left
+  // operands (T and -A, two bf16 terms each) come from LDS in that slot order; every product is
+  // three MFMAs (hi*hi, hi*lo, lo*hi).
   {
-    float X[KC];
-    const int c = tid;
-    if (c < KD) {
+    const int li = lane & 15, q4 = lane >> 4;
+    // 4a: T of diagonal block `wave`, one column per lane (lanes 16.. repeat the work of lane & 15).
+    {
+      float tc[16];
 #pragma unroll
-      for (int i = 0; i < KC; ++i) X[i] = bt[i] * rk[i] * __expf(G[i][c]) * bf16lo_to_f32(Kr[i][c]);
-    } else {
+      for (int i = 0; i < 16; ++i) tc[i] = (i == li) ? 1.f : 0.f;
 #pragma unroll
-      for (int i = 0; i < KC; ++i) X[i] = bt[i] * bf16lo_to_f32(Vr[i][c - KD]);
-    }
-    __syncthreads();   // every thread has read G: its space becomes the staging tile for Wn
-    // Right-looking elimination: once X[j] is final, remove it from every later row.  Row j of
-    // A^T is the same for all threads (an LDS broadcast); rows are fetched one step ahead of
-    // their use so that the LDS latency is hidden behind the multiply-adds of the current step.
-    f32x4 arow[2][KC / 4];
+      for (int j = 0; j < 15; ++j) {
+        f32x4 ar[4];
 #pragma unroll
-    for (int i4 = 0; i4 < KC / 4; ++i4) arow[0][i4] = lds_f4(&ATp[at_off(0) + 4 * i4 - at_first(0)]);
+        for (int i4 = (j + 1) / 4; i4 < 4; ++i4) ar[i4] = lds_f4(&Ad[wave][j][4 * i4]);
+        const float xj = tc[j];
 #pragma unroll
-    for (int j = 0; j < KC - 1; ++j) {
-      if (j + 1 < KC - 1) {
-#pragma unroll
-        for (int i4 = (j + 2) / 4; i4 < KC / 4; ++i4)
-          arow[(j + 1) & 1][i4] = lds_f4(&ATp[at_off(j + 1) + 4 * i4 - at_first(j + 1)]);
+        for (int i = j + 1; i < 16; ++i) tc[i] = fmaf(-ar[i >> 2][i & 3], xj, tc[i]);
       }
-      const float xj = X[j];
+      // The wavefront has read all of its block before any lane writes: T replaces A_II in place.
+      uint16_t* Th = reinterpret_cast<uint16_t*>(&Ad[wave][0][0]);   // [16][16] high terms, then [16][16] low terms
+      if (lane < 16) {
 #pragma unroll
-      for (int i4 = (j + 1) / 4; i4 < KC / 4; ++i4) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = 4 * i4 + e;
-          if (i > j) X[i] = fmaf(-arow[j & 1][i4][e], xj, X[i]);
+        for (int i = 0; i < 16; ++i) {
+          float hi, lo;
+          split_bf16(tc[i], hi, lo);
+          Th[i * 16 + li] = (uint16_t)(pack_bf16x2(hi, 0.f) & 0xffffu);
+          Th[256 + i * 16 + li] = (uint16_t)(pack_bf16x2(lo, 0.f) & 0xffffu);
         }
       }
     }
+    // 4b: right-hand sides in accumulator layout: C[tile][block][r] = B[16*block + 4*q4 + r][column].
+    f32x4 C[4][4];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+      const int col = 16 * (wave + 4 * (tt & 1)) + li;
+#pragma unroll
+      for (int I = 0; I < 4; ++I) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = 16 * I + 4 * q4 + r;
+          C[tt][I][r] = (tt < 2) ? bt[i] * rk[i] * __expf(G[i][col]) * bf16lo_to_f32(Kr[i][col])
+                                 : bt[i] * bf16lo_to_f32(Vr[i][col]);
+        }
+      }
+    }
+    __syncthreads();   // G has been read by everyone (it becomes the staging tile for Wn); T is in place
+    // 4c: left operands.  Slot (q4, e): e < 4 -> column 4*q4+e of the first block, e >= 4 -> of the second.
+    auto lds_half = [&](const uint16_t* row) -> u32x2 { return *reinterpret_cast<const u32x2*>(row + 4 * q4); };
+    auto frag = [&](u32x2 a, u32x2 b) -> bf16x8 { u32x4 w = {a.x, a.y, b.x, b.y}; return __builtin_bit_cast(bf16x8, w); };
+    const u32x2 none = {0u, 0u};
+    bf16x8 Tf[4][2], Af[4][2];   // Af: (1,0) | (2,0)(2,1) | (3,0)(3,1) | (3,2)
+#pragma unroll
+    for (int I = 0; I < 4; ++I) {
+      const uint16_t* Th = reinterpret_cast<const uint16_t*>(&Ad[I][0][0]);
+      Tf[I][0] = frag(lds_half(Th + li * 16), none);
+      Tf[I][1] = frag(lds_half(Th + 256 + li * 16), none);
+    }
+    Af[0][0] = frag(lds_half(&AoH[off_block(1, 0)][li][0]), none);
+    Af[0][1] = frag(lds_half(&AoL[off_block(1, 0)][li][0]), none);
+    Af[1][0] = frag(lds_half(&AoH[off_block(2, 0)][li][0]), lds_half(&AoH[off_block(2, 1)][li][0]));
+    Af[1][1] = frag(lds_half(&AoL[off_block(2, 0)][li][0]), lds_half(&AoL[off_block(2, 1)][li][0]));
+    Af[2][0] = frag(lds_half(&AoH[off_block(3, 0)][li][0]), lds_half(&AoH[off_block(3, 1)][li][0]));
+    Af[2][1] = frag(lds_half(&AoL[off_block(3, 0)][li][0]), lds_half(&AoL[off_block(3, 1)][li][0]));
+    Af[3][0] = frag(lds_half(&AoH[off_block(3, 2)][li][0]), none);
+    Af[3][1] = frag(lds_half(&AoL[off_block(3, 2)][li][0]), none);
+
+    // Two bf16 terms of an accumulator as halves of a right operand.
+    auto split_acc = [&](const f32x4& x, u32x2& hi, u32x2& lo) {
+      float h[4], l[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) split_bf16(x[e], h[e], l[e]);
+      hi.x = pack_bf16x2(h[0], h[1]); hi.y = pack_bf16x2(h[2], h[3]);
+      lo.x = pack_bf16x2(l[0], l[1]); lo.y = pack_bf16x2(l[2], l[3]);
+    };
+    // acc += L * R with L = Lf[0] + Lf[1], R = (hi | lo)
+    auto mul3 = [&](const bf16x8 (&Lf)[2], bf16x8 Rh, bf16x8 Rl, f32x4 acc) -> f32x4 {
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Lf[1], Rh, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Lf[0], Rl, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(Lf[0], Rh, acc, 0, 0, 0);
+      return acc;
+    };
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     uint16_t* Wst = reinterpret_cast<uint16_t*>(&G[0][0]);   // [64][128] bf16 staging
-    if (c < KD) {
-      const int pc = perm32(c);
 #pragma unroll
-      for (int i = 0; i < KC; ++i) Wst[i * KD + pc] = (uint16_t)(pack_bf16x2(-X[i], 0.f) & 0xffffu);
-    } else {
-      float* dst = p.U0T + (ci * KD + (c - KD)) * KC;
+    for (int tt = 0; tt < 4; ++tt) {
+      f32x4 X[4];
+      u32x2 xh[4], xl[4], ch, cl;
+      split_acc(C[tt][0], ch, cl);
+      X[0] = mul3(Tf[0], frag(ch, none), frag(cl, none), zero4);
+      split_acc(X[0], xh[0], xl[0]);
+      C[tt][1] = mul3(Af[0], frag(xh[0], none), frag(xl[0], none), C[tt][1]);
+      split_acc(C[tt][1], ch, cl);
+      X[1] = mul3(Tf[1], frag(ch, none), frag(cl, none), zero4);
+      split_acc(X[1], xh[1], xl[1]);
+      C[tt][2] = mul3(Af[1], frag(xh[0], xh[1]), frag(xl[0], xl[1]), C[tt][2]);
+      C[tt][3] = mul3(Af[2], frag(xh[0], xh[1]), frag(xl[0], xl[1]), C[tt][3]);
+      split_acc(C[tt][2], ch, cl);
+      X[2] = mul3(Tf[2], frag(ch, none), frag(cl, none), zero4);
+      split_acc(X[2], xh[2], xl[2]);
+      C[tt][3] = mul3(Af[3], frag(xh[2], none), frag(xl[2], none), C[tt][3]);
+      split_acc(C[tt][3], ch, cl);
+      X[3] = mul3(Tf[3], frag(ch, none), frag(cl, none), zero4);
+
+      const int col = 16 * (wave + 4 * (tt & 1)) + li;
+      if (tt < 2) {
+        const int pc = perm32(col);
 #pragma unroll
-      for (int i4 = 0; i4 < KC / 4; ++i4) {
-        f32x4 w = {X[4 * i4], X[4 * i4 + 1], X[4 * i4 + 2], X[4 * i4 + 3]};
-        *reinterpret_cast<f32x4*>(dst + 4 * i4) = w;
+        for (int I = 0; I < 4; ++I)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            Wst[(16 * I + 4 * q4 + r) * KD + pc] = (uint16_t)(pack_bf16x2(-X[I][r], 0.f) & 0xffffu);
+      } else {
+        float* dst = p.U0T + (ci * KD + col) * KC + 4 * q4;
+#pragma unroll
+        for (int I = 0; I < 4; ++I) *reinterpret_cast<f32x4*>(dst + 16 * I) = X[I];
       }
     }
     __syncthreads();
@@ -417,7 +502,6 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       *reinterpret_cast<u32x4*>(p.Wn + ci * KC * KD + 8 * ch) = *reinterpret_cast<const u32x4*>(Wst + 8 * ch);
     }
   }
-
 }
 
 __device__ __forceinline__ bf16x8 pack_acc2(const f32x4& t0, const f32x4& t1) {

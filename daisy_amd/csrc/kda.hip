@@ -1,5 +1,6 @@
 // Kernel 3: chunked Kimi Delta Attention forward and its log-decay gate (gfx950).
 #include "common.h"
+#include <type_traits>
 
 namespace daisy {
 
@@ -517,160 +518,226 @@ __device__ __forceinline__ bf16x8 pack_acc2(const f32x4& t0, const f32x4& t1) {
 // c ^ f(r)) so that the 16-byte operand reads of 16 consecutive rows fall into 16 different
 // slots of the 256-byte bank window: f(r) = r & 15 for 256-byte rows, (r >> 1) & 7 for 128-byte
 // rows (two rows per window).
-constexpr int KSW = 2;                        // wavefronts per workgroup (16 value columns each)
+constexpr int KCT = 2;                        // tiles of 16 value columns per workgroup
+constexpr int KSW = 2 * KCT;                  // computing wavefronts per workgroup: two per column tile
+constexpr int KPW = 4;                        // data-moving wavefronts per workgroup
 constexpr int kStageWn = 0;                   // [64][128] bf16
 constexpr int kStageQg = 16384;               // [64][128] bf16
 constexpr int kStageKtH = 32768;              // [128][64] bf16
 constexpr int kStageKtL = 49152;              // [128][64] bf16
-constexpr int kStagePm = 65536;               // [64][64]  bf16
-constexpr int kStageDec = 73728;              // [128] fp32
-constexpr int kStageBytes = 74240;
+constexpr int kStageBytes = 65536;
 
 typedef __attribute__((address_space(3))) const char* lds_cptr;
 __device__ __forceinline__ bf16x8 lds_bf16x8(lds_cptr p) {
   return __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)p);
 }
 
-__global__ __launch_bounds__(64 * KSW, 1) void kda_state_kernel(KdaParams p) {
+// The chunk-to-chunk chain sets the time of this kernel.  Two measures shorten a link:
+//  * the work of one tile of 16 value columns is shared by two wavefronts: wavefront `hf` keeps
+//    the state rows (key channels) [64 hf, 64 hf + 64) and produces the output rows (positions)
+//    [32 hf, 32 hf + 32) of the chunk.  Both need all of U = U0 - W S0, whose contraction runs
+//    over every key channel: each computes it in full (16 MFMAs, duplicated) from its own half of
+//    the state and a bf16 copy of the partner's half, handed over through LDS at the barrier
+//    that ends a chunk -- no barrier inside a chunk;
+//  * a fifth wavefront does nothing but move data: it issues the global->LDS copies of the next
+//    chunk (a CU takes in only ~30 bytes per cycle, so issuing 64 KB blocks a wavefront for
+//    longer than the arithmetic of a chunk lasts) and stores the previous chunk's output rows,
+//    which the computing wavefronts leave in LDS, as whole 64-byte row pieces.
+__global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParams p) {
   __shared__ __attribute__((aligned(1024))) char stage[2][kStageBytes];
+  __shared__ __attribute__((aligned(16))) u32x4 xch[2][KSW][2][64];           // [chunk parity][wavefront][k-group][lane]
+  __shared__ __attribute__((aligned(16))) uint16_t ost[2][KC][KVS * KCT];      // [chunk parity][position][value column]
 
   // Keep the column groups of one (batch, head) on one XCD: they read the same chunk data.
   int vid = blockIdx.x;
   if ((gridDim.x & 7) == 0) vid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  constexpr int NGRP = KD / (KVS * KSW);
+  constexpr int NGRP = KD / (KVS * KCT);
   const int grp = vid % NGRP, bh = vid / NGRP;
   const int h = bh % p.H, b = bh / p.H;
   const int lane = threadIdx.x & 63, ln = lane & 15, q4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int vcol = KVS * (KSW * grp + wave) + ln;
 
-  // ---- copies of one chunk into a stage (this wavefront's share) --------------------------
-  const uint32_t stage_lds = lds_address(&stage[0][0]);
-  // 256-byte rows: a wavefront copy moves 4 rows; lane i lands at row i/16, position i%16.
-  // 128-byte rows: 8 rows per copy; lane i lands at row i/8, position i%8.
-  int src256[4], src128[2];   // source byte offsets inside a group of 16 rows, by (copy index & 3) / (& 1)
+  if (wave >= KSW) {
+    const int pw = wave - KSW;
+    // ================= data-moving wavefront =================
+    const uint32_t stage_lds = lds_address(&stage[0][0]);
+    // 256-byte rows: a wavefront copy moves 4 rows; lane i lands at row i/16, position i%16.
+    // 128-byte rows: 8 rows per copy; lane i lands at row i/8, position i%8.
+    int src256[4], src128[2];   // source byte offsets inside a group of 16 rows, by (copy index & 3) / (& 1)
 #pragma unroll
-  for (int v = 0; v < 4; ++v) src256[v] = (4 * v + (lane >> 4)) * 256 + 16 * ((lane & 15) ^ ((4 * v + (lane >> 4)) & 15));
+    for (int v = 0; v < 4; ++v) src256[v] = (4 * v + (lane >> 4)) * 256 + 16 * ((lane & 15) ^ ((4 * v + (lane >> 4)) & 15));
 #pragma unroll
-  for (int v = 0; v < 2; ++v) src128[v] = (8 * v + (lane >> 3)) * 128 + 16 * ((lane & 7) ^ ((4 * v + (lane >> 4)) & 7));
-
-  auto issue_copies = [&](int n, int st) {
-    const int64_t ci = (int64_t)bh * p.NC + n;
-    const uint32_t dst = stage_lds + st * kStageBytes;
-    const uint16_t* wn = p.Wn + ci * KC * KD;
-    const uint16_t* qg = p.Qg + ci * KC * KD;
-    const uint16_t* kh = p.KtH + ci * KD * KC;
-    const uint16_t* kl = p.KtL + ci * KD * KC;
-    const uint16_t* pm = p.Pm + ci * KC * KC;
+    for (int v = 0; v < 2; ++v) src128[v] = (8 * v + (lane >> 3)) * 128 + 16 * ((lane & 7) ^ ((4 * v + (lane >> 4)) & 7));
+    auto issue_copies = [&](int n, int st) {
+      const int64_t ci = (int64_t)bh * p.NC + n;
+      const uint32_t dst = stage_lds + st * kStageBytes;
+      const uint16_t* wn = p.Wn + ci * KC * KD;
+      const uint16_t* qg = p.Qg + ci * KC * KD;
+      const uint16_t* kh = p.KtH + ci * KD * KC;
+      const uint16_t* kl = p.KtL + ci * KD * KC;
 #pragma unroll
-    for (int j = wave; j < 16; j += KSW) {   // 16 copies of 4 rows x 256 B each
-      copy16_to_lds_async(wn + (j >> 2) * 2048, src256[j & 3], dst + kStageWn + j * 1024);
-      copy16_to_lds_async(qg + (j >> 2) * 2048, src256[j & 3], dst + kStageQg + j * 1024);
-    }
+      for (int j = pw; j < 16; j += KPW) {
+        copy16_to_lds_async(wn + (j >> 2) * 2048, src256[j & 3], dst + kStageWn + j * 1024);
+        copy16_to_lds_async(qg + (j >> 2) * 2048, src256[j & 3], dst + kStageQg + j * 1024);
+      }
 #pragma unroll
-    for (int j = wave; j < 16; j += KSW) {   // 16 copies of 8 rows x 128 B each
-      copy16_to_lds_async(kh + (j >> 1) * 1024, src128[j & 1], dst + kStageKtH + j * 1024);
-      copy16_to_lds_async(kl + (j >> 1) * 1024, src128[j & 1], dst + kStageKtL + j * 1024);
-    }
+      for (int j = pw; j < 16; j += KPW) {
+        copy16_to_lds_async(kh + (j >> 1) * 1024, src128[j & 1], dst + kStageKtH + j * 1024);
+        copy16_to_lds_async(kl + (j >> 1) * 1024, src128[j & 1], dst + kStageKtL + j * 1024);
+      }
+    };
+    // The four workgroups of a (batch, head) copy the same 64 KB per chunk at about the same
+    // time and would all wait out the full HBM latency.  Each touches a quarter of a later chunk
+    // (this wavefront 4 KB of it, one dword per 64 bytes) so that the copies find their lines in
+    // L2.  The touching load is the youngest of an iteration: vmcnt(1) then means that every copy
+    // has landed (loads return in order) while the touch stays in flight.  Its target register
+    // is tied up for the whole loop.
+    uint32_t touched = 0;
+    constexpr int kAhead = 3;
+    auto touch_ahead = [&](int n) {
+      const int64_t ci = (int64_t)bh * p.NC + n;
+      const uint16_t* base = (grp == 0) ? p.Wn + ci * KC * KD : (grp == 1) ? p.Qg + ci * KC * KD
+                           : (grp == 2) ? p.KtH + ci * KD * KC : p.KtL + ci * KD * KC;
+      asm volatile("global_load_dword %0, %1, %2" : "+v"(touched) : "v"(pw * 4096 + lane * 64), "s"(base) : "memory");
+    };
+    // Output rows of chunk n: 64 rows x 64 bytes, 16 bytes per lane and pass.
+    auto store_o = [&](int n) {
 #pragma unroll
-    for (int j = wave; j < 8; j += KSW)
-      copy16_to_lds_async(pm + (j >> 1) * 1024, src128[j & 1], dst + kStagePm + j * 1024);
-    if (wave == 0 && lane < 32)
-      copy16_to_lds_async(reinterpret_cast<const uint16_t*>(p.dec + ci * KD), 16 * lane, dst + kStageDec);
-  };
-  auto copies_landed = [&]() {
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), visible to the compiler's wait-count model
+      for (int k = pw; k < 4; k += KPW) {
+        const int idx = 64 * k + lane, row = idx >> 2, piece = idx & 3;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(&ost[n & 1][row][8 * piece]);
+        const int t = n * KC + row;
+        if (t < p.T)
+          *reinterpret_cast<u32x4*>(p.o + (((int64_t)b * p.T + t) * p.H + h) * KD + KVS * KCT * grp + 8 * piece) = v;
+      }
+    };
+    issue_copies(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     asm volatile("" ::: "memory");
-  };
+    __syncthreads();
+    for (int n = 0; n < p.NC; ++n) {
+      if (n > 0) store_o(n - 1);
+      if (n + 1 < p.NC) issue_copies(n + 1, (n + 1) & 1);
+      if (NGRP == 4 && n + kAhead < p.NC) {
+        touch_ahead(n + kAhead);
+        __builtin_amdgcn_s_waitcnt(0x0F71);   // vmcnt(1)
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+      }
+      asm volatile("" ::: "memory");
+      __syncthreads();
+    }
+    store_o(p.NC - 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" :: "v"(touched));
+    return;
+  }
+
+  // ================= computing wavefronts =================
+  const int ct = wave >> 1, hf = wave & 1;
+  const int vcol = KVS * (KCT * grp + ct) + ln;
 
   // ---- per-lane LDS read offsets (bytes, inside a stage) ------------------------------------
   // A operand of a 16x16x32 MFMA: lane (row ln, k-group q4) reads chunk 4m + q4 of its row.
-  int rd256[4], rd128[2];
+  // Groups of 32 key channels are taken own half first: local group mm is channel group
+  // 2 hf + mm for mm < 2 and 2 (1 - hf) + mm - 2 after that.
+  int rdk[4], rd128[2];
 #pragma unroll
-  for (int m = 0; m < 4; ++m) rd256[m] = ln * 256 + 16 * ((4 * m + q4) ^ ln);
+  for (int mm = 0; mm < 4; ++mm) {
+    const int m = (mm < 2) ? 2 * hf + mm : 2 * (1 - hf) + (mm - 2);
+    rdk[mm] = ln * 256 + 16 * ((4 * m + q4) ^ ln);
+  }
 #pragma unroll
   for (int m = 0; m < 2; ++m) rd128[m] = ln * 128 + 16 * ((4 * m + q4) ^ ((ln >> 1) & 7));
   lds_cptr stage0 = (lds_cptr)&stage[0][0];
 
-  // State tile dt: rows (key channels) 16*dt + 4*q4 + r, column vcol.
-  f32x4 S[8];
+  // State tile i: rows (key channels) 16*(4 hf + i) + 4*q4 + r, column vcol.
+  f32x4 S[4];
 #pragma unroll
-  for (int dt = 0; dt < 8; ++dt) {
+  for (int i = 0; i < 4; ++i) {
 #pragma unroll
     for (int r = 0; r < 4; ++r)
-      S[dt][r] = p.s0 ? p.s0[((int64_t)bh * KD + 16 * dt + 4 * q4 + r) * KD + vcol] : 0.f;
+      S[i][r] = p.s0 ? p.s0[((int64_t)bh * KD + 16 * (4 * hf + i) + 4 * q4 + r) * KD + vcol] : 0.f;
   }
 
-  // U0 (accumulator initial value of U) comes straight from global memory, one chunk ahead.
-  auto load_u0 = [&](int n, f32x4* dst) {
-    const float* src = p.U0T + (((int64_t)bh * p.NC + n) * KD + vcol) * KC + 4 * q4;
+  // What depends on the value column or is small comes straight from global memory, one chunk
+  // ahead: U0 (accumulator initial value of U), the chunk's total decay of this wavefront's
+  // state rows, and this wavefront's rows of P as left operand.
+  auto load_direct = [&](int n, f32x4* u0, f32x4* dcy, bf16x8 (*pa)[2]) {
+    const int64_t ci = (int64_t)bh * p.NC + n;
+    const float* src = p.U0T + (ci * KD + vcol) * KC + 4 * q4;
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) dst[mt] = *reinterpret_cast<const f32x4*>(src + 16 * mt);
-  };
-  f32x4 u0c[4], u0n[4];
-  issue_copies(0, 0);
-  load_u0(0, u0c);
-  copies_landed();
-  __syncthreads();
-
-  for (int n = 0; n < p.NC; ++n) {
-    const int st = n & 1;
-    if (n + 1 < p.NC) {
-      issue_copies(n + 1, st ^ 1);
-      load_u0(n + 1, u0n);
-    }
-    lds_cptr sb = stage0 + st * kStageBytes;
-
-    // LDS operands are read in two batches ahead of the MFMAs that use them (one wavefront per
-    // SIMD has the registers for it) instead of each next to its MFMA, where every MFMA waited
-    // for a full LDS latency.
-    bf16x8 wa[4][4], qa[4][4], pa[4][2], kh[8][2], kl[8][2];
-    f32x4 dc[8];
+    for (int mt = 0; mt < 4; ++mt) u0[mt] = *reinterpret_cast<const f32x4*>(src + 16 * mt);
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int i = 0; i < 4; ++i) dcy[i] = *reinterpret_cast<const f32x4*>(p.dec + ci * KD + 16 * (4 * hf + i) + 4 * q4);
 #pragma unroll
-      for (int m = 0; m < 4; ++m) wa[mt][m] = lds_bf16x8(sb + kStageWn + 4096 * mt + rd256[m]);
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-      for (int m = 0; m < 4; ++m) qa[mt][m] = lds_bf16x8(sb + kStageQg + 4096 * mt + rd256[m]);
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int m = 0; m < 2; ++m)
-        if (32 * m <= 16 * mt + 15) pa[mt][m] = lds_bf16x8(sb + kStagePm + 2048 * mt + rd128[m]);
+        pa[i][m] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(p.Pm + (ci * KC + 16 * (2 * hf + i) + ln) * KC + 32 * m + 8 * q4));
+  };
+  // Two sets, used in turn by even and odd chunks (the chunk loop is unrolled by two so that no
+  // register copy, which would have to wait for the loads, sits between them and their use).
+  f32x4 u0[2][4], dcy[2][4];
+  bf16x8 pa[2][2][2];
+  bf16x8 Sb[4];   // the state as right operand, by local channel group
+  Sb[0] = pack_acc2(S[0], S[1]);
+  Sb[1] = pack_acc2(S[2], S[3]);
+  xch[0][wave][0][lane] = __builtin_bit_cast(u32x4, Sb[0]);
+  xch[0][wave][1][lane] = __builtin_bit_cast(u32x4, Sb[1]);
+  load_direct(0, u0[0], dcy[0], pa[0]);
+  __syncthreads();
 
-    bf16x8 Sb[4];
+  auto chunk_step = [&](int n, auto parity) {
+    constexpr int st = decltype(parity)::value;
+    f32x4 (&u0c)[4] = u0[st];
+    f32x4 (&dcc)[4] = dcy[st];
+    bf16x8 (&pac)[2][2] = pa[st];
+    // The direct loads of the next chunk go out first thing, ahead of the burst of copies of the
+    // data-moving wavefronts (the memory pipeline of a CU is one queue: behind that burst they
+    // would block this wavefront for thousands of cycles), and are waited for at the end of the
+    // chunk, so that no wait for them can end up behind newer loads.
+    if (n + 1 < p.NC) load_direct(n + 1, u0[st ^ 1], dcy[st ^ 1], pa[st ^ 1]);
+    __builtin_amdgcn_sched_barrier(0);
+    lds_cptr sb = stage0 + st * kStageBytes;
+
+    // LDS operands are read in two batches ahead of the MFMAs that use them instead of each next
+    // to its MFMA, where every MFMA waited for a full LDS latency.
+    Sb[2] = __builtin_bit_cast(bf16x8, xch[st][wave ^ 1][0][lane]);
+    Sb[3] = __builtin_bit_cast(bf16x8, xch[st][wave ^ 1][1][lane]);
+    bf16x8 wa[4][4], qa[2][4], kh[4][2], kl[4][2];
 #pragma unroll
-    for (int m = 0; m < 4; ++m) Sb[m] = pack_acc2(S[2 * m], S[2 * m + 1]);
+    for (int mm = 0; mm < 4; ++mm) {
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) wa[mt][mm] = lds_bf16x8(sb + kStageWn + 4096 * mt + rdk[mm]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) qa[i][mm] = lds_bf16x8(sb + kStageQg + 4096 * (2 * hf + i) + rdk[mm]);
+    }
     __builtin_amdgcn_sched_barrier(0);
 
-    // U = U0 + (-W) S0 and O = Qg S0: eight independent accumulator chains.
-    // Tile mt: rows (positions) 16*mt + 4*q4 + r, column vcol.
-    f32x4 U[4], O[4];
+    // U = U0 + (-W) S0 (all four row tiles) and O = Qg S0 (this wavefront's two row tiles).
+    // Row tile mt: positions 16*mt + 4*q4 + r, column vcol.
+    f32x4 U[4], O[2];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-      U[mt] = u0c[mt];
-      O[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < 4; ++mt) U[mt] = u0c[mt];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) O[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int mm = 0; mm < 4; ++mm) {
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) U[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[mt][mm], Sb[mm], U[mt], 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) O[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[i][mm], Sb[mm], O[i], 0, 0, 0);
     }
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
-        U[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[mt][m], Sb[m], U[mt], 0, 0, 0);
-        O[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[mt][m], Sb[m], O[mt], 0, 0, 0);
-      }
-    }
-    // The operands of the state update are read while those 32 MFMAs run.
+    // The operands of the state update are read while those MFMAs run.
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt) {
+    for (int i = 0; i < 4; ++i) {
 #pragma unroll
       for (int m = 0; m < 2; ++m) {
-        kh[dt][m] = lds_bf16x8(sb + kStageKtH + 2048 * dt + rd128[m]);
-        kl[dt][m] = lds_bf16x8(sb + kStageKtL + 2048 * dt + rd128[m]);
+        kh[i][m] = lds_bf16x8(sb + kStageKtH + 2048 * (4 * hf + i) + rd128[m]);
+        kl[i][m] = lds_bf16x8(sb + kStageKtL + 2048 * (4 * hf + i) + rd128[m]);
       }
-      dc[dt] = *(const f32x4 __attribute__((address_space(3)))*)(sb + kStageDec + 4 * (16 * dt + 4 * q4));
     }
     __builtin_amdgcn_sched_barrier(0);
     bf16x8 Uh[2], Ul[2];
@@ -686,50 +753,53 @@ __global__ __launch_bounds__(64 * KSW, 1) void kda_state_kernel(KdaParams p) {
       Ul[m] = pack_acc2(l0, l1);
     }
 
-    // O += Pm U  (scale already folded into Qg and Pm; columns up to the diagonal only)
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-#pragma unroll
-      for (int m = 0; m < 2; ++m) {
-        if (32 * m <= 16 * mt + 15)
-          O[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[mt][m], Uh[m], O[mt], 0, 0, 0);
-      }
-    }
     // S = exp(G_last) (.) S + Kt^T U, with both operands split into two bf16 terms.
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt) {
+    for (int i = 0; i < 4; ++i) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) S[dt][r] *= dc[dt][r];
+      for (int r = 0; r < 4; ++r) S[i][r] *= dcc[i][r];
     }
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
 #pragma unroll
-      for (int dt = 0; dt < 8; ++dt) {
-        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kh[dt][m], Uh[m], S[dt], 0, 0, 0);
-        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kh[dt][m], Ul[m], S[dt], 0, 0, 0);
-        S[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kl[dt][m], Uh[m], S[dt], 0, 0, 0);
+      for (int i = 0; i < 4; ++i) {
+        S[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kh[i][m], Uh[m], S[i], 0, 0, 0);
+        S[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kh[i][m], Ul[m], S[i], 0, 0, 0);
+        S[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kl[i][m], Uh[m], S[i], 0, 0, 0);
       }
     }
+    // O += Pm U (scale already folded into Qg and Pm).  Positions 32..63 of U only reach the
+    // output rows of the second half (P is zero above the diagonal).
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int i = 0; i < 2; ++i) O[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pac[i][0], Uh[0], O[i], 0, 0, 0);
+    if (hf) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int t = n * KC + 16 * mt + 4 * q4 + r;
-        if (t < p.T) p.o[(((int64_t)b * p.T + t) * p.H + h) * KD + vcol] = (uint16_t)(pack_bf16x2(O[mt][r], 0.f) & 0xffffu);
-      }
+      for (int i = 0; i < 2; ++i) O[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pac[i][1], Uh[1], O[i], 0, 0, 0);
+    }
+    // The new state goes to the partner as soon as it exists.
+    Sb[0] = pack_acc2(S[0], S[1]);
+    Sb[1] = pack_acc2(S[2], S[3]);
+    xch[st ^ 1][wave][0][lane] = __builtin_bit_cast(u32x4, Sb[0]);
+    xch[st ^ 1][wave][1][lane] = __builtin_bit_cast(u32x4, Sb[1]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        ost[st][16 * (2 * hf + i) + 4 * q4 + r][KVS * ct + ln] = (uint16_t)(pack_bf16x2(O[i][r], 0.f) & 0xffffu);
     }
 
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) u0c[mt] = u0n[mt];
-    copies_landed();
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the direct loads of the next chunk
     __syncthreads();
+  };
+  for (int n = 0; n < p.NC; n += 2) {
+    chunk_step(n, std::integral_constant<int, 0>{});
+    if (n + 1 < p.NC) chunk_step(n + 1, std::integral_constant<int, 1>{});
   }
-
   if (p.s_out != nullptr) {
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) p.s_out[((int64_t)bh * KD + 16 * dt + 4 * q4 + r) * KD + vcol] = S[dt][r];
+      for (int r = 0; r < 4; ++r) p.s_out[((int64_t)bh * KD + 16 * (4 * hf + i) + 4 * q4 + r) * KD + vcol] = S[i][r];
   }
 }
 
@@ -800,7 +870,7 @@ extern "C" int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(kda_prep_kernel, dim3(p.NC, H, B), dim3(256), 0, s, p);
   DAISY_CHECK_LAUNCH("kda_prep_kernel");
-  hipLaunchKernelGGL(kda_state_kernel, dim3((unsigned)(B * H * (KD / (KVS * KSW)))), dim3(64 * KSW), 0, s, p);
+  hipLaunchKernelGGL(kda_state_kernel, dim3((unsigned)(B * H * (KD / (KVS * KCT)))), dim3(64 * (KSW + KPW)), 0, s, p);
   DAISY_CHECK_LAUNCH("kda_state_kernel");
   return DAISY_OK;
 }

@@ -105,8 +105,13 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   auto row_off = [&](int r) -> int64_t { return (((int64_t)b * p.T + t0 + r) * p.H + h) * KD; };
 
   // ---- phase 0a: G = cumsum(g) -----------------------------------------------
+  // Every global load of the chunk (g here, then q, k, v and beta of phase 0b) goes out before
+  // the first result is used, so that the memory latency is paid once.
   if (tid < 4) steep[tid] = 0;
   __syncthreads();
+  const int cc = tid & 15, r4 = tid >> 4;
+  u32x4 qraw[4], vraw[4], kraw[4];
+  float btv[4];
   {
     const int d = tid & 127, half = tid >> 7;
     float gv[32];
@@ -119,6 +124,17 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       const float x = p.g_bf16 ? bf16lo_to_f32(((const uint16_t*)p.g)[off]) : ((const float*)p.g)[off];
       gv[i] = (t0 + r < p.T) ? x : 0.f;
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = r4 + 16 * i;
+      const int rc = min(r, p.T - 1 - t0);
+      const int64_t off = row_off(rc) + 8 * cc;
+      kraw[i] = *reinterpret_cast<const u32x4*>(p.k + off);
+      vraw[i] = *reinterpret_cast<const u32x4*>(p.v + off);
+      qraw[i] = *reinterpret_cast<const u32x4*>(p.q + off);
+      btv[i] = p.beta[((int64_t)b * p.T + t0 + rc) * p.H + h];
+    }
+    __builtin_amdgcn_sched_barrier(0);
     float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
@@ -141,21 +157,15 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   }
 
   // ---- phase 0b: raw q, k to LDS, row norms, beta ---------------------------
-  const int cc = tid & 15, r4 = tid >> 4;
-  u32x4 qraw[4], vraw[4];
   float rqv[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = r4 + 16 * i;
     const bool live = t0 + r < p.T;
-    const int64_t off = row_off(min(r, p.T - 1 - t0)) + 8 * cc;
     const u32x4 zero4 = {0, 0, 0, 0};
-    u32x4 kraw = *reinterpret_cast<const u32x4*>(p.k + off);
-    vraw[i] = *reinterpret_cast<const u32x4*>(p.v + off);
-    qraw[i] = *reinterpret_cast<const u32x4*>(p.q + off);
-    if (!live) { kraw = zero4; vraw[i] = zero4; qraw[i] = zero4; }
+    if (!live) { kraw[i] = zero4; vraw[i] = zero4; qraw[i] = zero4; }
     float kf[8], qf[8];
-    unpack8(kraw, kf);
+    unpack8(kraw[i], kf);
     unpack8(qraw[i], qf);
     float sk = 0.f, sq = 0.f;
 #pragma unroll
@@ -167,9 +177,9 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
     if (cc == 0) {
       rk[r] = nk;
       rq[r] = rqv[i];
-      bt[r] = live ? p.beta[((int64_t)b * p.T + t0 + r) * p.H + h] : 0.f;
+      bt[r] = live ? btv[i] : 0.f;
     }
-    *reinterpret_cast<u32x4*>(&Kr[r][8 * cc]) = kraw;
+    *reinterpret_cast<u32x4*>(&Kr[r][8 * cc]) = kraw[i];
     *reinterpret_cast<u32x4*>(&Qr[r][8 * cc]) = qraw[i];
   }
   __syncthreads();

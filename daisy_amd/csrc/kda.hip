@@ -361,25 +361,6 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(&Vr[r4 + 16 * i][8 * cc]) = vraw[i];
 
-  // ---- phase 3: (exp(G_last - G) k/|k|)^T as two bf16 terms, position permuted ----
-  {
-    const int d = tid & 127, gh = tid >> 7;
-    const float glast = G[KC - 1][d];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int g8 = 4 * gh + i;   // group of 8 stored positions
-      float hi[8], lo[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int pos = perm32_inv(8 * g8 + e);
-        const float val = __expf(glast - G[pos][d]) * bf16lo_to_f32(Kr[pos][d]) * rk[pos];
-        hi[e] = round_bf16(val);
-        lo[e] = val - hi[e];
-      }
-      *reinterpret_cast<u32x4*>(p.KtH + (ci * KD + d) * KC + 8 * g8) = pack8(hi);
-      *reinterpret_cast<u32x4*>(p.KtL + (ci * KD + d) * KC + 8 * g8) = pack8(lo);
-    }
-  }
   __syncthreads();   // V is in place
 
   // ---- phase 4: (I + A) X = diag(beta) [exp(G) K | V] by blocks of 16 rows on MFMA ----
@@ -434,7 +415,38 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
         }
       }
     }
-    __syncthreads();   // G has been read by everyone (it becomes the staging tile for Wn); T is in place
+    // ---- phase 3 (placed here, where few registers are live): (exp(G_last - G) k/|k|)^T as two
+    // bf16 terms, position permuted.  Thread (d, gh) makes four 16-byte pieces of row d; stored
+    // from here they would hit 64 different lines per instruction, so they go through LDS (the
+    // space of G and of K, both dead after the barrier) and leave as whole rows.
+    u32x4 kth[4], ktl[4];
+    const int kd = tid & 127, kgh = tid >> 7;
+    {
+      const float glast = G[KC - 1][kd];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int g8 = 4 * kgh + i;   // group of 8 stored positions
+        float hi[8], lo[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int pos = perm32_inv(8 * g8 + e);
+          const float val = __expf(glast - G[pos][kd]) * bf16lo_to_f32(Kr[pos][kd]) * rk[pos];
+          hi[e] = round_bf16(val);
+          lo[e] = val - hi[e];
+        }
+        kth[i] = pack8(hi);
+        ktl[i] = pack8(lo);
+      }
+    }
+    __syncthreads();   // G, K and V have been read by everyone (their space becomes staging); T is in place
+    char* KtHst = reinterpret_cast<char*>(&G[0][0]) + KC * KD * 2;   // [128][64] bf16 behind the Wn tile
+    char* KtLst = reinterpret_cast<char*>(&Kr[0][0]);                // [128][64] bf16
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int off = kd * 128 + 16 * ((4 * kgh + i) ^ (kd & 7));    // pieces of a row swizzled against bank conflicts
+      *reinterpret_cast<u32x4*>(KtHst + off) = kth[i];
+      *reinterpret_cast<u32x4*>(KtLst + off) = ktl[i];
+    }
     // 4c: left operands.  Slot (q4, e): e < 4 -> column 4*q4+e of the first block, e >= 4 -> of the second.
     auto lds_half = [&](const uint16_t* row) -> u32x2 { return *reinterpret_cast<const u32x2*>(row + 4 * q4); };
     auto frag = [&](u32x2 a, u32x2 b) -> bf16x8 { u32x4 w = {a.x, a.y, b.x, b.y}; return __builtin_bit_cast(bf16x8, w); };
@@ -511,6 +523,13 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
     for (int i = 0; i < 4; ++i) {
       const int ch = tid + 256 * i;   // 16-byte chunk of the [64][128] bf16 tile
       *reinterpret_cast<u32x4*>(p.Wn + ci * KC * KD + 8 * ch) = *reinterpret_cast<const u32x4*>(Wst + 8 * ch);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ch = tid + 256 * i;   // 16-byte chunk of a [128][64] bf16 tile
+      const int off = (ch >> 3) * 128 + 16 * ((ch & 7) ^ ((ch >> 3) & 7));
+      *reinterpret_cast<u32x4*>(p.KtH + ci * KD * KC + 8 * ch) = *reinterpret_cast<const u32x4*>(KtHst + off);
+      *reinterpret_cast<u32x4*>(p.KtL + ci * KD * KC + 8 * ch) = *reinterpret_cast<const u32x4*>(KtLst + off);
     }
   }
 }

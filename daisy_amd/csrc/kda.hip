@@ -43,10 +43,11 @@ __global__ __launch_bounds__(256) void kda_gate_kernel(const void* g, const floa
 //   KtH + KtL = (exp(G_last - G) (.) K)^T split into two bf16 terms, [128][64], position permuted
 //   U0T = U0^T                      fp32 [128][64]
 //   dec = exp(G_last)               fp32 [128]
-// kda_state_kernel (one wavefront per (batch, head, 16 value columns), two wavefronts per
-// workgroup sharing the chunk data through double-buffered LDS stages) then
-// walks the chunks in order with the fp32 state in registers; every product in
-// it is a v_mfma_f32_16x16x32_bf16 whose B operand is an accumulator (S0 or U)
+// kda_state_kernel (one workgroup per (batch, head, 32 value columns): two computing
+// wavefronts per tile of 16 columns, four data-moving wavefronts that fill the
+// double-buffered LDS stages with the chunk data) then walks the chunks in order
+// with the fp32 state in registers; every product in it is a
+// v_mfma_f32_16x16x32_bf16 whose B operand is an accumulator (S0 or U)
 // converted to bf16 in place: in the 16x16 accumulator layout lane l holds
 // column l%16 and rows 4*(l/16)+r of each tile, so two stacked tiles give the
 // lane 8 contraction indices 16*t + 4*(l/16) + r (t = 0,1; r = 0..3).  The A
@@ -54,12 +55,14 @@ __global__ __launch_bounds__(256) void kda_gate_kernel(const void* g, const floa
 // aligned group of 32 (perm32) so that those 8 indices are 8 consecutive
 // elements, one 16-byte load.
 //
-// Numerics: off-diagonal 16x16 blocks of A and P run on MFMA with both operands
-// referenced to the row before the block (every exponent <= 0); diagonal blocks
-// are accumulated in fp32 from running products of exp(g) (no exponent is ever
-// positive, so strong decays cannot overflow).  The triangular solve is fp32.
-// The state update uses a two-term bf16 split of both operands (three MFMAs),
-// which keeps the state error near fp32.
+// Numerics: the 16x16 blocks of A and P run on MFMA with both operands
+// referenced to the row before the block (every exponent <= 0 off the diagonal);
+// a diagonal block whose total decay exceeds exp(-80) is instead accumulated in
+// fp32 from running products of exp(g) (no exponent is ever positive, so strong
+// decays cannot overflow).  The triangular solve works on 16-row blocks: fp32
+// inverses of the diagonal blocks, everything else as products of two-term bf16
+// splits (three MFMAs each, relative error ~2^-17).  The state update uses the
+// same two-term split of both operands, which keeps the state error near fp32.
 // ===========================================================================
 constexpr int KC = 64;    // chunk length
 constexpr int KD = 128;   // Dk = Dv

@@ -138,10 +138,12 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       btv[i] = p.beta[((int64_t)b * p.T + t0 + rc) * p.H + h];
     }
     __builtin_amdgcn_sched_barrier(0);
+    // G holds the running sum in units of log 2 (g * log2(e)): every exponential below is a bare
+    // v_exp_f32.
     float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
-      acc += gv[i];
+      acc += gv[i] * kLog2e;
       G[32 * half + i][d] = acc;
     }
 #pragma unroll
@@ -199,8 +201,8 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       const float sc = p.scale * rqv[i];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        o8[e] = sc * __expf(g0[e]) * qf[e];
-        o8[4 + e] = sc * __expf(g1[e]) * qf[4 + e];
+        o8[e] = sc * __builtin_amdgcn_exp2f(g0[e]) * qf[e];
+        o8[4 + e] = sc * __builtin_amdgcn_exp2f(g1[e]) * qf[4 + e];
       }
       const u32x4 pk = pack8(o8);
       uint16_t* dst = p.Qg + (ci * KC + r) * KD + pos0;
@@ -212,7 +214,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       const f32x4 g0 = lds_f4(&G[KC - 1][8 * cc]), g1 = lds_f4(&G[KC - 1][8 * cc + 4]);
       f32x4 d0, d1;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) { d0[e] = __expf(g0[e]); d1[e] = __expf(g1[e]); }
+      for (int e = 0; e < 4; ++e) { d0[e] = __builtin_amdgcn_exp2f(g0[e]); d1[e] = __builtin_amdgcn_exp2f(g1[e]); }
       float* dd = p.dec + ci * KD + 8 * cc;
       *reinterpret_cast<f32x4*>(dd) = d0;
       *reinterpret_cast<f32x4*>(dd + 4) = d1;
@@ -224,37 +226,56 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   // factor exp(G_i - G_ref) is <= 1 and, for J < I, so is the column factor exp(G_ref - G_j).
   // For a diagonal block (J == I) the column factor grows to exp(total decay of the block); the
   // block takes this path only when that total stays below 80 (flag `steep` otherwise).
-  auto mfma_block = [&](int I, int J) {
+  // The row operands (k_i f_i, q_i f_i with f_i = exp(G_i - G_ref)) of a block row are made once
+  // and serve every block of the row.
+  bf16x8 va[4], vq[4];
+  auto row_operands = [&](int I) {
     const int li = lane & 15, q4 = lane >> 4;
     const int ref = 16 * I - 1;   // -1 for the first block: G_ref = 0
-    const int ri = 16 * I + li, rj = 16 * J + li;
+    const int ri = 16 * I + li;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int d0 = 32 * m + 8 * q4;
+      float ki[8], qi[8], ak[8], aq[8];
+      unpack8(*reinterpret_cast<const u32x4*>(&Kr[ri][d0]), ki);
+      unpack8(*reinterpret_cast<const u32x4*>(&Qr[ri][d0]), qi);
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+        const f32x4 gi = lds_f4(&G[ri][d0 + 4 * hf]);
+        const f32x4 gr = (ref >= 0) ? lds_f4(&G[max(ref, 0)][d0 + 4 * hf]) : zero;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float fi = __builtin_amdgcn_exp2f(gi[e] - gr[e]);
+          ak[4 * hf + e] = ki[4 * hf + e] * fi;
+          aq[4 * hf + e] = qi[4 * hf + e] * fi;
+        }
+      }
+      va[m] = __builtin_bit_cast(bf16x8, pack8(ak));
+      vq[m] = __builtin_bit_cast(bf16x8, pack8(aq));
+    }
+  };
+  auto mfma_block = [&](int I, int J) {
+    const int li = lane & 15, q4 = lane >> 4;
+    const int ref = 16 * I - 1;
+    const int rj = 16 * J + li;
     f32x4 accA = {0.f, 0.f, 0.f, 0.f}, accP = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
       const int d0 = 32 * m + 8 * q4;
-      float ki[8], qi[8], kj[8], ak[8], aq[8], bk[8];
-      unpack8(*reinterpret_cast<const u32x4*>(&Kr[ri][d0]), ki);
-      unpack8(*reinterpret_cast<const u32x4*>(&Qr[ri][d0]), qi);
+      float kj[8], bk[8];
       unpack8(*reinterpret_cast<const u32x4*>(&Kr[rj][d0]), kj);
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf) {
         const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-        const f32x4 gi = lds_f4(&G[ri][d0 + 4 * hf]), gj = lds_f4(&G[rj][d0 + 4 * hf]);
+        const f32x4 gj = lds_f4(&G[rj][d0 + 4 * hf]);
         const f32x4 gr = (ref >= 0) ? lds_f4(&G[max(ref, 0)][d0 + 4 * hf]) : zero;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float fi = __expf(gi[e] - gr[e]);
-          const float fj = __expf(gr[e] - gj[e]);
-          ak[4 * hf + e] = ki[4 * hf + e] * fi;
-          aq[4 * hf + e] = qi[4 * hf + e] * fi;
-          bk[4 * hf + e] = kj[4 * hf + e] * fj;
-        }
+        for (int e = 0; e < 4; ++e) bk[4 * hf + e] = kj[4 * hf + e] * __builtin_amdgcn_exp2f(gr[e] - gj[e]);
       }
-      const bf16x8 va = __builtin_bit_cast(bf16x8, pack8(ak));
-      const bf16x8 vq = __builtin_bit_cast(bf16x8, pack8(aq));
       const bf16x8 vb = __builtin_bit_cast(bf16x8, pack8(bk));
-      accA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, vb, accA, 0, 0, 0);
-      accP = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vq, vb, accP, 0, 0, 0);
+      accA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[m], vb, accA, 0, 0, 0);
+      accP = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vq[m], vb, accP, 0, 0, 0);
     }
     // accumulator: lane holds column j = 16J + li, rows i = 16I + 4*q4 + r
     const int j = 16 * J + li;
@@ -280,31 +301,12 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       }
     }
   };
-  {
-    for (int bi = wave; bi < 6; bi += 4) {
-      // off-diagonal blocks in the order (1,0) (2,0) (2,1) (3,0) (3,1) (3,2)
-      const int I = (bi == 0) ? 1 : (bi < 3 ? 2 : 3);
-      const int J = (bi == 0) ? 0 : (bi < 3 ? bi - 1 : bi - 3);
-      mfma_block(I, J);
-    }
-    // The state kernel reads P in 16x32 pieces; blocks (0,1) and (2,3) lie above the diagonal.
-    if (wave >= 2) {
-      const int li = lane & 15, q4 = lane >> 4;
-      const int I = (wave == 2) ? 0 : 2, J = I + 1;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) p.Pm[(ci * KC + 16 * I + 4 * q4 + r) * KC + perm32(16 * J + li)] = 0;
-    }
-  }
-
-  // ---- phase 2b: diagonal 16x16 blocks ----------------------------------------
-  // Wavefront w owns diagonal block w.  Usual case: the MFMA path above.  If some channel
-  // decays by more than exp(-80) across the block, the column factors of that path could
-  // overflow; the block is then accumulated in fp32 from running products of exp(g), where no
-  // exponent is ever positive.
-  if (!steep[wave]) {
-    mfma_block(wave, wave);
-  } else {
-    const int I = wave, il = lane >> 2, dq = lane & 3;
+  // Blocks by wavefront: 0 -> (0,0), (3,3); 1 -> (1,0), (1,1); 2 -> (2,0), (2,1), (2,2);
+  // 3 -> (3,0), (3,1), (3,2).  A diagonal block whose decay is too steep for the MFMA path (some
+  // channel beyond exp(-80) across the block: the column factors could overflow) is accumulated
+  // in fp32 from running products of exp(g), where no exponent is ever positive.
+  auto steep_diagonal = [&](int I) {
+    const int il = lane >> 2, dq = lane & 3;
     const int ri = 16 * I + il;
     float a[16], pp[16];
 #pragma unroll
@@ -328,7 +330,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
           const f32x4 gb0 = lds_f4(&G[rj][d0]), gb1 = lds_f4(&G[rj][d0 + 4]);
           f32x4 e0, e1;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) { e0[e] = __expf(ga0[e] - gb0[e]); e1[e] = __expf(ga1[e] - gb1[e]); }
+          for (int e = 0; e < 4; ++e) { e0[e] = __builtin_amdgcn_exp2f(ga0[e] - gb0[e]); e1[e] = __builtin_amdgcn_exp2f(ga1[e] - gb1[e]); }
           const bool live = j < il;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -356,6 +358,26 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
         pv = (j <= il) ? qs * rkj * pv : 0.f;
         p.Pm[(ci * KC + ri) * KC + perm32(rj)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
       }
+    }
+  };
+  {
+    const int nseg = (wave == 0) ? 2 : 1;
+    for (int sg = 0; sg < nseg; ++sg) {
+      const int I = (wave == 0) ? 3 * sg : wave;
+      const int jlo = (wave == 0) ? I : 0, jhi = (wave == 3) ? 2 : I;
+      row_operands(I);
+      for (int J = jlo; J <= jhi; ++J) {
+        if (J == I && steep[I]) steep_diagonal(I);
+        else mfma_block(I, J);
+      }
+    }
+    // The state kernel reads P in 16x32 pieces; blocks (0,1) and (2,3) lie above the diagonal.
+    if (wave == 1) {
+      const int li = lane & 15, q4 = lane >> 4;
+#pragma unroll
+      for (int I = 0; I < 4; I += 2)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) p.Pm[(ci * KC + 16 * I + 4 * q4 + r) * KC + perm32(16 * (I + 1) + li)] = 0;
     }
   }
   __syncthreads();
@@ -413,7 +435,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int i = 16 * I + 4 * q4 + r;
-          C[tt][I][r] = (tt < 2) ? bt[i] * rk[i] * __expf(G[i][col]) * bf16lo_to_f32(Kr[i][col])
+          C[tt][I][r] = (tt < 2) ? bt[i] * rk[i] * __builtin_amdgcn_exp2f(G[i][col]) * bf16lo_to_f32(Kr[i][col])
                                  : bt[i] * bf16lo_to_f32(Vr[i][col]);
         }
       }
@@ -433,7 +455,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int pos = perm32_inv(8 * g8 + e);
-          const float val = __expf(glast - G[pos][kd]) * bf16lo_to_f32(Kr[pos][kd]) * rk[pos];
+          const float val = __builtin_amdgcn_exp2f(glast - G[pos][kd]) * bf16lo_to_f32(Kr[pos][kd]) * rk[pos];
           hi[e] = round_bf16(val);
           lo[e] = val - hi[e];
         }

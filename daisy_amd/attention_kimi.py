@@ -49,8 +49,23 @@ class ShortConvolution(nn.Module):
         self.weight = nn.Parameter(w)
         self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=dtype)) if bias else None
 
-    def forward(self, x: Tensor, cache: Optional[Tensor] = None, output_final_state: bool = False
-                ) -> Tuple[Tensor, Optional[Tensor]]:
+    def forward(self, x: Tensor, cache: Optional[Tensor] = None, output_final_state: bool = False,
+                cu_seqlens: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
+        if cu_seqlens is not None:
+            # Sequences packed along T of a batch of one: the window must not reach across a
+            # boundary, so every sequence is convolved by itself; caches are [N, C, K].
+            bounds = [int(v) for v in cu_seqlens.tolist()]
+            ys, caches = [], []
+            for i in range(len(bounds) - 1):
+                c_i = cache[i:i + 1] if cache is not None else None
+                if bounds[i + 1] == bounds[i]:
+                    if output_final_state:
+                        caches.append(c_i.clone() if c_i is not None else x.new_zeros(1, x.size(2), self.kernel_size))
+                    continue
+                y_i, nc_i = self.forward(x[:, bounds[i]:bounds[i + 1]], c_i, output_final_state)
+                ys.append(y_i)
+                caches.append(nc_i)
+            return torch.cat(ys, dim=1), (torch.cat(caches, dim=0) if output_final_state else None)
         B, T, C = x.shape
         K = self.kernel_size
         xt = x.transpose(1, 2)                                        # [B, C, T]
@@ -83,9 +98,12 @@ class KimiLinearSelfAttention(nn.Module):
 
     ``ve`` is accepted for interface compatibility; it is mixed into v as in ``CausalSelfAttention``
     (``sigmoid(g_ve) * v + (1 - sigmoid(g_ve)) * ve``) when ``receives_ve`` is set and ignored
-    otherwise (the reference leaves this as a TODO).  ``attn_mask`` is accepted and ignored (the
-    recurrence is causal by construction, a window does not apply, and variable-length packing
-    through a padding mask is not supported); ``block_mask`` must be None as in the reference.
+    otherwise (the reference leaves this as a TODO).  A two-dimensional ``attn_mask [B, S]`` is a
+    padding mask as in the reference (models/daisy/attention_kimi.py:150-154, 1 = token,
+    0 = padding): the tokens are packed into one row, every sequence runs by itself
+    (``cu_seqlens``), and the padded positions of the result are zero.  Any other ``attn_mask``
+    (window descriptors, dense attention masks) is ignored: the recurrence is causal by
+    construction and a window does not apply.  ``block_mask`` must be None as in the reference.
     """
 
     def __init__(self, dim: int, num_heads: int, max_seq_len: int, head_dim: int, expand_v: float = 1.0,
@@ -138,16 +156,27 @@ class KimiLinearSelfAttention(nn.Module):
         self._conv_state = None
         self._seen = 0
 
-    def _core(self, x: Tensor, ve: Optional[Tensor], use_cache: bool) -> Tensor:
-        B, T, _ = x.shape
+    def _core(self, x: Tensor, ve: Optional[Tensor], use_cache: bool, attn_mask=None) -> Tensor:
+        B0, S0, _ = x.shape
         H, Dk, Dv = self.num_heads, self.head_k_dim, self.head_v_dim
         x = x.to(self.q_proj.weight.dtype)
+        indices = cu_seqlens = None
+        if isinstance(attn_mask, Tensor) and attn_mask.ndim == 2:
+            # get_unpad_data of the reference's dependency, restated: positions of the tokens in the
+            # flattened batch and the running sequence lengths.
+            keep = attn_mask[:, -S0:].to(torch.bool)
+            indices = torch.nonzero(keep.flatten(), as_tuple=False).flatten()
+            cu_seqlens = F.pad(torch.cumsum(keep.sum(-1), 0), (1, 0)).to(torch.int32)
+            x = x.flatten(0, 1)[indices].unsqueeze(0)
+            if ve is not None:
+                ve = ve.reshape(B0 * S0, -1)[indices].unsqueeze(0)
+        B, T, _ = x.shape
         state = self._recurrent_state if use_cache else None
         convs = self._conv_state if (use_cache and self._conv_state is not None) else (None, None, None)
         if self.use_short_conv:
-            q, cq = self.q_conv1d(self.q_proj(x), convs[0], use_cache)
-            k, ck = self.k_conv1d(self.k_proj(x), convs[1], use_cache)
-            v, cv = self.v_conv1d(self.v_proj(x), convs[2], use_cache)
+            q, cq = self.q_conv1d(self.q_proj(x), convs[0], use_cache, cu_seqlens)
+            k, ck = self.k_conv1d(self.k_proj(x), convs[1], use_cache, cu_seqlens)
+            v, cv = self.v_conv1d(self.v_proj(x), convs[2], use_cache, cu_seqlens)
         else:
             q, k, v = F.silu(self.q_proj(x)), F.silu(self.k_proj(x)), F.silu(self.v_proj(x))
             cq = ck = cv = None
@@ -158,27 +187,32 @@ class KimiLinearSelfAttention(nn.Module):
             v = g_x * v + (1.0 - g_x) * ve.view_as(v).to(v.dtype)
         g = fused_kda_gate(self.f_proj(x), self.A_log, Dk, self.dt_bias)
         beta = torch.sigmoid(self.b_proj(x)).to(torch.float32)
-        if use_cache and T == 1 and state is not None:
+        if use_cache and T == 1 and state is not None and cu_seqlens is None:
             o, state = fused_recurrent_kda(q, k, v, g, beta, initial_state=state, use_qk_l2norm_in_kernel=True,
                                            inplace_state=True)
         else:
             o, state = chunk_kda(q, k, v, g, beta, initial_state=state, output_final_state=use_cache,
-                                 use_qk_l2norm_in_kernel=True)
+                                 use_qk_l2norm_in_kernel=True, cu_seqlens=cu_seqlens)
         if use_cache:
             self._recurrent_state = state
             self._conv_state = (cq, ck, cv)
             self._seen += T
         gate = self.g_proj(x).view(B, T, H, Dv)
         o = self.o_norm(o.to(gate.dtype), gate)
-        return self.o_proj(o.reshape(B, T, H * Dv))
+        y = self.o_proj(o.reshape(B, T, H * Dv))
+        if indices is not None:   # back to the padded layout, zeros where the mask was 0
+            padded = y.new_zeros(B0 * S0, y.size(-1))
+            padded[indices] = y[0]
+            y = padded.view(B0, S0, -1)
+        return y
 
     def forward(self, x: Tensor, ve: Optional[Tensor], attn_mask=None, block_mask=None) -> Tensor:
         assert block_mask is None, "block_mask not supported for KimiLinearSelfAttention"
-        return self._core(x, ve, use_cache=False)
+        return self._core(x, ve, use_cache=False, attn_mask=attn_mask)
 
     def prefill(self, x: Tensor, ve: Optional[Tensor], attn_mask=None, debug: bool = False):
         """Runs the prompt and keeps the recurrent and convolution states; there is no K/V to cache."""
-        return self._core(x, ve, use_cache=True), None, None
+        return self._core(x, ve, use_cache=True, attn_mask=attn_mask), None, None
 
     def step(self, x: Tensor, k_ctx, v_ctx, pos: int, ve: Optional[Tensor], window: Optional[int]):
         torch._assert(x.size(1) == 1, "step() requires single position only")

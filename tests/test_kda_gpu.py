@@ -8,7 +8,7 @@ import torch
 import torch.nn.functional as F
 
 import oracle
-from daisy_amd import chunk_kda, fused_kda_gate, ops
+from daisy_amd import chunk_kda, fused_kda_gate, fused_recurrent_kda, ops
 from helpers import assert_close_bf16, say
 
 pytestmark = pytest.mark.gpu
@@ -169,3 +169,27 @@ def test_kda_recurrent_rejects_bad_arguments():
         ops.kda_recurrent_fwd(q[..., :64].contiguous(), k[..., :64].contiguous(), v, gl[..., :64].contiguous(), beta)
     with pytest.raises(ValueError):
         ops.kda_recurrent_fwd(q, k, v, gl, beta, inplace_state=True)
+
+
+def test_kda_cu_seqlens_packs_independent_sequences():
+    """Sequences packed along T with ``cu_seqlens`` (the call of models/daisy/attention_kimi.py:133-134
+    passes it): each runs from its own initial state, empty ones included."""
+    H = 2
+    lens = [100, 64, 0, 136]
+    T = sum(lens)
+    q, k, v, gl, beta = _inputs(1, T, H, seed=11)
+    cu = torch.tensor([0, 100, 164, 164, 300], dtype=torch.int32)
+    S0 = torch.randn(len(lens), H, 128, 128, generator=torch.Generator().manual_seed(12)) * 0.1
+    o, S = chunk_kda(q.cuda(), k.cuda(), v.cuda(), gl.cuda(), beta.cuda(), initial_state=S0.cuda(),
+                     output_final_state=True, use_qk_l2norm_in_kernel=True, cu_seqlens=cu.cuda())
+    assert o.shape == (1, T, H, 128) and S.shape == (len(lens), H, 128, 128)
+    o_r, S_r = fused_recurrent_kda(q.cuda(), k.cuda(), v.cuda(), gl.cuda(), beta.cuda(), initial_state=S0.cuda(),
+                                   output_final_state=True, use_qk_l2norm_in_kernel=True, cu_seqlens=cu.cuda())
+    for i, n in enumerate(lens):
+        s, e = int(cu[i]), int(cu[i + 1])
+        if n == 0:
+            assert torch.equal(S[i].cpu(), S0[i]) and torch.equal(S_r[i].cpu(), S0[i])
+            continue
+        o_ref, S_ref = oracle.kda_recurrent(q[:, s:e], k[:, s:e], v[:, s:e], gl[:, s:e], beta[:, s:e], initial_state=S0[i:i + 1])
+        _check(o[:, s:e], S[i:i + 1], o_ref, S_ref, f"chunked, sequence {i}")
+        _check(o_r[:, s:e], S_r[i:i + 1], o_ref, S_ref, f"recurrent, sequence {i}")

@@ -105,3 +105,33 @@ def test_parameter_names_and_dtypes_follow_the_reference():
     assert m.q_conv1d.weight.shape == (256, 1, 4)
     with pytest.raises(AssertionError):
         m.to(DEV)(torch.zeros(1, 4, 256, device=DEV, dtype=torch.bfloat16), None, block_mask=object())
+
+
+def test_padding_mask_packs_sequences():
+    """A [B, S] padding mask (models/daisy/attention_kimi.py:150-154): every row runs as its own
+    sequence on its tokens only, padded positions come back as zeros."""
+    with torch.no_grad():
+        m = _layer(seed=4).to(DEV)
+        B, S = 3, 160
+        x = torch.randn(B, S, 256, generator=torch.Generator().manual_seed(5)).bfloat16().to(DEV)
+        lens = [160, 97, 1]
+        mask = torch.zeros(B, S, dtype=torch.int32)
+        for b, n in enumerate(lens):
+            mask[b, S - n:] = 1          # left padding
+        y = m(x, None, attn_mask=mask.to(DEV))
+        assert y.shape == (B, S, 256)
+        for b, n in enumerate(lens):
+            y_b = m(x[b:b + 1, S - n:], None)
+            _close(y[b, S - n:], y_b[0], f"row {b} ({n} tokens) vs the row alone", 2e-2)
+            assert not y[b, :S - n].any(), "padded positions must be zero"
+        # with a state: prefill on the padded batch, then a step, equals the rows one by one
+        m.reset_history()
+        m.prefill(x, None, attn_mask=mask.to(DEV))
+        assert m._recurrent_state.shape[0] == B
+        x1 = torch.randn(B, 1, 256, generator=torch.Generator().manual_seed(6)).bfloat16().to(DEV)
+        y1, _, _ = m.step(x1, None, None, S, None, None)
+        for b, n in enumerate(lens):
+            m.reset_history()
+            m.prefill(x[b:b + 1, S - n:], None)
+            y1_b, _, _ = m.step(x1[b:b + 1], None, None, n, None, None)
+            _close(y1[b], y1_b[0], f"step after padded prefill, row {b}", 2e-2)

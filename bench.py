@@ -321,6 +321,8 @@ def main():
         extra["prefill_c3_B1_T65536_H16_D128"] = bench_prefill_c3(max(args.steps // 5, 4), max(args.warmup // 2, 2))
     if want("decode"):
         extra["decode_c4"] = bench_decode_c4(256, 16, cpu)
+        from daisy_amd import ops
+        extra["hbm_read_ceiling"] = dict(ops.probe_read_rate(), what="read-only stream of 2 GiB, 8192 workgroups, 128 B in flight per lane")
     if want("kda"):
         try:
             extra["kda_c5"] = bench_kda_c5(max(args.steps // 5, 4), max(args.warmup // 2, 2), cpu)

@@ -60,6 +60,7 @@ SIGNATURES = {
         c_float, c_float, c_void_p]),                           # softplus beta, threshold, stream
     "daisy_probe_matrix_rate": (c_int, [
         c_int, c_int, c_int, c_void_p, c_void_p, POINTER(ctypes.c_double), c_void_p]),
+    "daisy_probe_read_rate": (c_int, [c_void_p, ctypes.c_size_t, c_int, c_void_p, c_void_p]),
     "daisy_qkv_prep_fwd": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q, k, v (+ strides)
         c_void_p, _I64P, c_void_p,                               # ve, ve strides, gate

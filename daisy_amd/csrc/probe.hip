@@ -50,9 +50,37 @@ __global__ __launch_bounds__(512) void matrix_rate_kernel(float* sink, unsigned 
   }
 }
 
+// Read-only streaming: every workgroup sums its contiguous slab of the buffer with 8 x 16 bytes in
+// flight per lane (non-temporal loads).  The rate this reaches is the practical ceiling of any
+// kernel that only streams from HBM, such as the decode kernel.
+__global__ __launch_bounds__(256) void read_rate_kernel(const u32x4* buf, size_t vec_per_wg, uint32_t* sink) {
+  const u32x4* p = buf + (size_t)blockIdx.x * vec_per_wg + threadIdx.x;
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  for (size_t i = 0; i < vec_per_wg; i += 256 * 8) {
+    u32x4 r[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) r[u] = __builtin_nontemporal_load(p + i + 256 * u);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += r[u];
+  }
+  // The sum only keeps the loads alive; it is stored when it takes one particular value.
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[blockIdx.x & 4095] = acc.x;
+}
+
 }  // namespace daisy
 
 using namespace daisy;
+
+extern "C" int daisy_probe_read_rate(const void* buf, size_t bytes, int workgroups, void* sink, void* stream) {
+  DAISY_CHECK_ARG(buf && sink, "probe: buf and sink (4096 x 4 bytes) must be non-NULL");
+  DAISY_CHECK_ARG((reinterpret_cast<uintptr_t>(buf) & 15) == 0, "probe: buf must be 16-byte aligned");
+  DAISY_CHECK_ARG(workgroups > 0 && bytes > 0 && bytes % ((size_t)workgroups * 256 * 8 * 16) == 0,
+                  "probe: bytes=%zu must be a multiple of workgroups (%d) x 32 KiB", bytes, workgroups);
+  hipLaunchKernelGGL(read_rate_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream,
+                     reinterpret_cast<const u32x4*>(buf), bytes / 16 / (size_t)workgroups, reinterpret_cast<uint32_t*>(sink));
+  DAISY_CHECK_LAUNCH("read_rate_kernel");
+  return DAISY_OK;
+}
 
 extern "C" int daisy_probe_matrix_rate(int with_vector_mix, int workgroups, int iters,
                                        float* sink, unsigned long long* ticks, double* flop_out, void* stream) {

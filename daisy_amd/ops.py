@@ -343,3 +343,26 @@ def probe_matrix_rate(with_vector_mix: bool, iters: int = 50000, workgroups: int
     ms = start.elapsed_time(end)
     t = ticks.view(workgroups, 2).double().sum(0)
     return {"ms": ms, "tflops": flop.value / ms / 1e9, "clock_mhz": float(t[0] / t[1] * 100.0)}
+
+
+def probe_read_rate(gib: int = 2, workgroups: int = 8192, repeats: int = 5, device="cuda:0") -> dict:
+    """Read-only streaming rate of the GPU over a ``gib`` GiB buffer (``daisy_probe_read_rate``).
+
+    Returns ``{"ms", "bytes", "gbs"}`` (mean over ``repeats`` launches after one warm-up).
+    """
+    dev = torch.device(device)
+    nbytes = gib << 30
+    buf = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
+    sink = torch.empty(4096, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.device(dev):
+        stream = _lib.current_stream(dev)
+        _lib.check(lib.daisy_probe_read_rate(buf.data_ptr(), nbytes, workgroups, sink.data_ptr(), stream), "daisy_probe_read_rate")
+        start.record()
+        for _ in range(repeats):
+            _lib.check(lib.daisy_probe_read_rate(buf.data_ptr(), nbytes, workgroups, sink.data_ptr(), stream), "daisy_probe_read_rate")
+        end.record()
+        torch.cuda.synchronize(dev)
+    ms = start.elapsed_time(end) / repeats
+    return {"ms": ms, "bytes": nbytes, "gbs": nbytes / ms / 1e6}

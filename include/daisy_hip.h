@@ -220,6 +220,14 @@ int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
 int daisy_probe_matrix_rate(int with_vector_mix, int workgroups, int iters,
                             float* sink, unsigned long long* ticks, double* flop_out, void* stream);
 
+/* Diagnostic (no counterpart in the reference): `workgroups` workgroups of 256 threads read
+ * `bytes` bytes of `buf` once (contiguous slab each, 8 x 16 bytes in flight per lane) and keep
+ * nothing.  The caller times the launch: bytes / time is the read-only streaming rate of the
+ * GPU, the practical ceiling for the decode kernel.  bytes must be a multiple of
+ * workgroups x 32 KiB; sink: 4096 x 4 bytes of scratch.
+ */
+int daisy_probe_read_rate(const void* buf, size_t bytes, int workgroups, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

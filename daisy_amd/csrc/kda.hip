@@ -109,7 +109,8 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
 
   // ---- phase 0a: G = cumsum(g) -----------------------------------------------
   // Every global load of the chunk (g here, then q, k, v and beta of phase 0b) goes out before
-  // the first result is used, so that the memory latency is paid once.
+  // the first result is used, so that the memory latency is paid once.  Inputs are read once and
+  // the workspace is written once: both as streaming (non-temporal) accesses.
   if (tid < 4) steep[tid] = 0;
   __syncthreads();
   const int cc = tid & 15, r4 = tid >> 4;
@@ -124,7 +125,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       // Rows past the end re-read the last row (always valid) and are zeroed afterwards, so
       // that the loads carry no branches and all go out together.
       const int64_t off = row_off(min(r, p.T - 1 - t0)) + d;
-      const float x = p.g_bf16 ? bf16lo_to_f32(((const uint16_t*)p.g)[off]) : ((const float*)p.g)[off];
+      const float x = p.g_bf16 ? bf16lo_to_f32(((const uint16_t*)p.g)[off]) : __builtin_nontemporal_load(((const float*)p.g) + off);
       gv[i] = (t0 + r < p.T) ? x : 0.f;
     }
 #pragma unroll
@@ -132,9 +133,9 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       const int r = r4 + 16 * i;
       const int rc = min(r, p.T - 1 - t0);
       const int64_t off = row_off(rc) + 8 * cc;
-      kraw[i] = *reinterpret_cast<const u32x4*>(p.k + off);
-      vraw[i] = *reinterpret_cast<const u32x4*>(p.v + off);
-      qraw[i] = *reinterpret_cast<const u32x4*>(p.q + off);
+      kraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.k + off));
+      vraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.v + off));
+      qraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.q + off));
       btv[i] = p.beta[((int64_t)b * p.T + t0 + rc) * p.H + h];
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -207,8 +208,8 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       const u32x4 pk = pack8(o8);
       uint16_t* dst = p.Qg + (ci * KC + r) * KD + pos0;
       u32x2 lo2 = {pk.x, pk.y}, hi2 = {pk.z, pk.w};
-      *reinterpret_cast<u32x2*>(dst) = lo2;        // channels 8cc+0..3
-      *reinterpret_cast<u32x2*>(dst + 8) = hi2;    // channels 8cc+4..7
+      __builtin_nontemporal_store(lo2, reinterpret_cast<u32x2*>(dst));        // channels 8cc+0..3
+      __builtin_nontemporal_store(hi2, reinterpret_cast<u32x2*>(dst + 8));    // channels 8cc+4..7
     }
     if (r4 == 0) {
       const f32x4 g0 = lds_f4(&G[KC - 1][8 * cc]), g1 = lds_f4(&G[KC - 1][8 * cc + 4]);
@@ -540,21 +541,21 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       } else {
         float* dst = p.U0T + (ci * KD + col) * KC + 4 * q4;
 #pragma unroll
-        for (int I = 0; I < 4; ++I) *reinterpret_cast<f32x4*>(dst + 16 * I) = X[I];
+        for (int I = 0; I < 4; ++I) __builtin_nontemporal_store(X[I], reinterpret_cast<f32x4*>(dst + 16 * I));
       }
     }
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int ch = tid + 256 * i;   // 16-byte chunk of the [64][128] bf16 tile
-      *reinterpret_cast<u32x4*>(p.Wn + ci * KC * KD + 8 * ch) = *reinterpret_cast<const u32x4*>(Wst + 8 * ch);
+      __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(Wst + 8 * ch), reinterpret_cast<u32x4*>(p.Wn + ci * KC * KD + 8 * ch));
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int ch = tid + 256 * i;   // 16-byte chunk of a [128][64] bf16 tile
       const int off = (ch >> 3) * 128 + 16 * ((ch & 7) ^ ((ch >> 3) & 7));
-      *reinterpret_cast<u32x4*>(p.KtH + ci * KD * KC + 8 * ch) = *reinterpret_cast<const u32x4*>(KtHst + off);
-      *reinterpret_cast<u32x4*>(p.KtL + ci * KD * KC + 8 * ch) = *reinterpret_cast<const u32x4*>(KtLst + off);
+      __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(KtHst + off), reinterpret_cast<u32x4*>(p.KtH + ci * KD * KC + 8 * ch));
+      __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(KtLst + off), reinterpret_cast<u32x4*>(p.KtL + ci * KD * KC + 8 * ch));
     }
   }
 }

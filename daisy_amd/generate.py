@@ -1,105 +1,146 @@
-"""``Generator`` with the reference's interface (inference/generate.py:61-285).
+"""Token generation over a ring KV cache, with the interface of the reference's ``Generator``
+(inference/generate.py:61-285): same constructor arguments, ``generate`` is a Python generator
+that yields ids and returns ``(history, prefill_seconds, decode_seconds)``, and ``_prefill`` /
+``_step`` talk to the model through ``model.prefill(ids[1, T]) -> (logits, kv[2, L, B, H, T, D])``
+and ``model.step(token, k_ctxs, v_ctxs, pos) -> (logits, k_list, v_list)``.
 
-``_prefill`` runs ``model.prefill`` and fills the ring cache, ``_step`` hands the
-per-layer context to ``model.step`` and appends the new rows, ``generate``
-yields sampled tokens.  Differences from the reference, none visible to a
-caller: nothing is wrapped in ``torch.compile`` (the hot ops are HIP kernels),
-and when every attention layer is this package's ``CausalSelfAttention`` the
-step passes ``RingContext`` handles so the decode kernel streams the cache in
-place and appends the new row itself (no chronological copy, no second write).
+What is arranged differently here:
+
+* nothing is wrapped in ``torch.compile``: the hot operations are HIP kernels already;
+* when every block's attention is this package's ``CausalSelfAttention`` and the cache is bf16, a
+  step hands each layer a handle on its ring (``KVCache.ring``) instead of a chronological copy:
+  the decode kernel streams the ring where it lies and appends the new row itself, so a step moves
+  no cache bytes on the host's behalf.  The handles are made once, not per token;
+* the token history lives in a preallocated buffer that grows geometrically, not in a tensor that
+  is re-concatenated for every token.
+
+Sampling follows the reference's arithmetic (inference/generate.py:13-58): temperature, top-k,
+nucleus filter, Gumbel-max draw, and the distance-decayed repetition penalty over the last 128
+tokens; the random numbers are drawn with the same call, so a seed gives the same tokens.
 """
 from __future__ import annotations
 
 import time
-from typing import Generator as _GeneratorType
+from typing import Iterator, List, Optional, Tuple
 
 import torch
-import torch.nn.functional as F
+from torch import Tensor
 
 from .attention import CausalSelfAttention
 from .kv_cache import KVCache
 
-
-def _topk_filter(x, k):
-    if k is None or k <= 0 or k >= x.size(-1):
-        return x
-    vals, idx = torch.topk(x, k)
-    return torch.full_like(x, float("-inf")).scatter_(-1, idx, vals)
+_NEG_INF = float("-inf")
+_PENALTY_LOOKBACK = 128      # tokens of history the repetition penalty looks at (generate.py:271)
 
 
-def _topp_filter(x, p):
-    if p is None or p <= 0.0 or p >= 1.0:
-        return x
-    sorted_p, order = torch.sort(F.softmax(x, dim=-1), dim=-1, descending=True)
-    keep_sorted = torch.cumsum(sorted_p, dim=-1) <= p
-    keep_sorted[..., 0] = True
-    keep = torch.zeros_like(keep_sorted).scatter(-1, order, keep_sorted)
-    return x.masked_fill(~keep, float("-inf"))
+# ----------------------------------------------------------------------------------------------
+# sampling
+# ----------------------------------------------------------------------------------------------
+def keep_top_k(scores: Tensor, k: Optional[int]) -> Tensor:
+    """Everything but the k largest entries of the last dim becomes -inf (no-op for k outside 1..V-1)."""
+    vocab = scores.size(-1)
+    if not k or k < 0 or k >= vocab:
+        return scores
+    drop = torch.ones_like(scores, dtype=torch.bool)
+    drop.scatter_(-1, scores.topk(k, dim=-1).indices, False)
+    return scores.masked_fill(drop, _NEG_INF)
 
 
-def _gumbel(shape, device, dtype):
-    u = torch.rand(shape, device=device, dtype=dtype)
-    return -torch.log(-torch.log(u.clamp_min_(1e-6)))
+def keep_nucleus(scores: Tensor, p: Optional[float]) -> Tensor:
+    """Nucleus filter: in order of falling probability, tokens stay while the running mass is <= p;
+    the most likely token always stays (no-op for p outside (0, 1))."""
+    if p is None or not (0.0 < p < 1.0):
+        return scores
+    ranked, order = scores.sort(dim=-1, descending=True)
+    mass = ranked.softmax(dim=-1).cumsum(dim=-1)
+    out_ranked = mass > p
+    out_ranked[..., 0] = False
+    out = torch.empty_like(out_ranked).scatter_(-1, order, out_ranked)
+    return scores.masked_fill(out, _NEG_INF)
 
 
-def _sample(logits, temperature=1.0, top_k=None, top_p=None):
-    """Greedy at temperature 0, else Gumbel-max over the filtered logits (generate.py:36-45)."""
+def gumbel_noise(like: Tensor) -> Tensor:
+    """Standard Gumbel noise, uniform draw clamped away from 0 at 1e-6."""
+    u = torch.rand(like.shape, device=like.device, dtype=like.dtype)
+    return u.clamp_min_(1e-6).log_().neg_().log_().neg_()
+
+
+def sample_token(logits: Tensor, temperature: float = 1.0, top_k: Optional[int] = None,
+                 top_p: Optional[float] = None) -> Tensor:
+    """Arg-max at temperature 0; otherwise one draw from softmax(filtered logits / temperature)
+    by the Gumbel-max identity (arg-max of scores + Gumbel noise)."""
     if temperature == 0.0:
-        return torch.argmax(logits, dim=-1)
-    x = logits / max(temperature, 1e-6)
-    x = _topp_filter(_topk_filter(x, top_k), top_p)
-    return torch.argmax(x + _gumbel(x.shape, x.device, x.dtype), dim=-1)
+        return logits.argmax(dim=-1)
+    scores = keep_nucleus(keep_top_k(logits / max(temperature, 1e-6), top_k), top_p)
+    return (scores + gumbel_noise(scores)).argmax(dim=-1)
 
 
-def _repetition_penalty(logits, prev: torch.Tensor, rep_p: torch.Tensor, _one: torch.Tensor, rep_h=140.0, cap=3.0):
-    """Distance-decayed repetition penalty (generate.py:47-58)."""
-    dist = torch.arange(prev.numel(), 0, -1, device=logits.device, dtype=logits.dtype)
-    hits = torch.zeros_like(logits).scatter_add_(0, prev, 0.5 ** (dist / rep_h)).clamp_max_(cap)
-    scale = torch.pow(rep_p, hits)
-    return logits * torch.where(logits > 0, 1.0 / scale, scale)
+def penalise_repeats(logits: Tensor, recent: Tensor, strength: Tensor, _one: Optional[Tensor] = None,
+                     half_life: float = 140.0, cap: float = 3.0) -> Tensor:
+    """A token seen ``d`` positions ago (1 = the last one) counts ``0.5 ** (d / half_life)``; counts
+    add up per token and saturate at ``cap``; the token's logit is divided by ``strength ** count``
+    when positive and multiplied by it otherwise.  ``_one`` is unused (kept for the call shape)."""
+    age = torch.arange(recent.numel(), 0, -1, device=logits.device, dtype=logits.dtype)
+    count = torch.zeros_like(logits).index_add_(0, recent, torch.pow(0.5, age / half_life)).clamp_(max=cap)
+    scale = torch.pow(strength, count)
+    return logits * torch.where(logits > 0, scale.reciprocal(), scale)
 
 
+# ----------------------------------------------------------------------------------------------
+# generator
+# ----------------------------------------------------------------------------------------------
 class Generator:
     def __init__(self, model, window, seed, device=None, dtype=torch.float16, max_seq_len: int = 65536,
                  temperature=1.0, top_k=None, top_p=None, repetition_penalty=1.0, eos_token_id=None):
-        if eos_token_id is None:
-            eos_token_id = getattr(model, "eos_token_id", None)
-        assert eos_token_id is not None
+        eos = eos_token_id if eos_token_id is not None else getattr(model, "eos_token_id", None)
+        if eos is None:
+            raise AssertionError("eos_token_id must be given or be an attribute of the model")
         self.model = model.eval()
-        self.device = next(model.parameters()).device if device is None else device
-        self.dtype = dtype
-        assert self.device is not None
-        h = d = None
-        attn_modules = []
-        for b in self.model.blocks:
-            a = getattr(b, "attn", None)
-            if a is not None:
-                attn_modules.append(a)
-                if h is None:
-                    h, d = a.num_heads, a.head_dim
-        self.cache = KVCache(L=len(self.model.blocks), B=1, H=h, W=window, D=d, device=self.device, dtype=dtype)
-        # In-place decode needs every layer's attention to understand RingContext
-        # and a bf16 cache (the kernels' storage type).
-        self.use_ring_context = (dtype == torch.bfloat16 and len(attn_modules) == len(self.model.blocks)
-                                 and all(isinstance(a, CausalSelfAttention) for a in attn_modules))
-        self.temperature = temperature
-        self.top_k = top_k
-        self.top_p = top_p
+        self.device = device if device is not None else next(model.parameters()).device
+        self.dtype, self.seed, self.max_seq_len = dtype, seed, max_seq_len
+        self.temperature, self.top_k, self.top_p = temperature, top_k, top_p
+        self.vocab_size = model.embed.num_embeddings
+        self.eos_token_id = torch.tensor(eos, device=self.device)
         self.rep_p_t = torch.tensor(repetition_penalty, device=self.device, dtype=dtype)
-        self.eos_token_id = torch.tensor(eos_token_id, device=self.device)
-        self.max_seq_len = max_seq_len
-        self.vocab_size = self.model.embed.num_embeddings
         self._one = torch.tensor(1, device=self.device, dtype=dtype)
-        self.seed = seed
-        torch.manual_seed(self.seed)
-        self.history = torch.empty(0, dtype=torch.long, device=self.device)
-        self.sample = _sample
-        self.apply_repetition_penalty = _repetition_penalty
+        self.sample = sample_token
+        self.apply_repetition_penalty = penalise_repeats
 
-    def _sync(self):
-        if str(self.device).startswith("cuda") and torch.cuda.is_available():
-            torch.cuda.synchronize()
+        # Cache geometry comes from the first block that has attention (generate.py:71-76).
+        layers = list(model.blocks)
+        attn = [getattr(blk, "attn", None) for blk in layers]
+        first = next(a for a in attn if a is not None)
+        self.cache = KVCache(L=len(layers), B=1, H=first.num_heads, W=window, D=first.head_dim,
+                             device=self.device, dtype=dtype)
+        # In-place decode: every layer must understand ring handles and the ring must be bf16.
+        self.use_ring_context = dtype == torch.bfloat16 and all(isinstance(a, CausalSelfAttention) for a in attn)
+        self._rings = [self.cache.ring(i) for i in range(len(layers))] if self.use_ring_context else None
 
+        torch.manual_seed(seed)
+        self._tokens = torch.empty(256, dtype=torch.long, device=self.device)
+        self._n_tokens = 0
+
+    # -- history ---------------------------------------------------------------------------
+    @property
+    def history(self) -> Tensor:
+        return self._tokens[:self._n_tokens]
+
+    @history.setter
+    def history(self, ids: Tensor) -> None:
+        self._n_tokens = 0
+        self._remember(ids)
+
+    def _remember(self, ids: Tensor) -> None:
+        ids = ids.reshape(-1).to(device=self.device, dtype=torch.long)
+        need = self._n_tokens + ids.numel()
+        if need > self._tokens.numel():
+            grown = torch.empty(max(need, 2 * self._tokens.numel()), dtype=torch.long, device=self.device)
+            grown[:self._n_tokens] = self._tokens[:self._n_tokens]
+            self._tokens = grown
+        self._tokens[self._n_tokens:need] = ids
+        self._n_tokens = need
+
+    # -- small setters of the reference's interface ----------------------------------------
     def set_temperature(self, temperature: float):
         self.temperature = float(temperature)
         return self
@@ -111,66 +152,80 @@ class Generator:
     def reset_history(self):
         self.model.reset_history()
         self.cache.reset_history()
-        self.history = torch.empty(0, dtype=torch.long, device=self.device)
+        self._n_tokens = 0
 
-    def _prefill(self, prompt_ids: torch.Tensor):
-        """``model.prefill(ids[1, T]) -> (logits, kv[2, L, B, H, T, D])``; fills the cache."""
-        ids = prompt_ids[None, :]
-        assert ids.size(1) > 0
-        logits, kv = self.model.prefill(ids)
-        logits = logits.to(self.dtype)[..., :self.vocab_size]
-        self.cache.bulk_write_packed(kv, prompt_ids.numel())
-        self.history = torch.cat([self.history, prompt_ids.to(dtype=torch.long, device=self.device)], dim=0)
-        return logits
+    def _sync(self):
+        if torch.cuda.is_available() and torch.device(self.device).type == "cuda":
+            torch.cuda.synchronize()
 
-    def _step(self, token: torch.Tensor):
-        L = len(self.model.blocks)
-        k_ctxs, v_ctxs = [], []
-        for i in range(L):
-            if self.use_ring_context:
-                ctx = self.cache.ring(i)
-                k_ctxs.append(ctx)
-                v_ctxs.append(ctx)
-            else:
-                kc, vc = self.cache.view(i)
-                assert kc.dtype == self.dtype and vc.dtype == self.dtype
-                k_ctxs.append(kc)
-                v_ctxs.append(vc)
-        logits, k_new, v_new = self.model.step(token, k_ctxs, v_ctxs, self.cache.t)
-        logits = logits.to(self.dtype)[..., :self.vocab_size]
-        # Layers without attention return None; the first layer always has attention.
-        k_new = [x.to(self.dtype) if x is not None else torch.zeros_like(k_new[0]) for x in k_new]
-        v_new = [x.to(self.dtype) if x is not None else torch.zeros_like(v_new[0]) for x in v_new]
-        for i in range(L):
-            if not self.cache._staged[i]:  # the decode kernel may already have appended this row
-                self.cache.write(i, k_new[i], v_new[i])
+    def _trim(self, logits: Tensor) -> Tensor:
+        return logits.to(self.dtype)[..., :self.vocab_size]
+
+    # -- model calls -----------------------------------------------------------------------
+    def _prefill(self, prompt_ids: Tensor) -> Tensor:
+        """Runs the prompt, stores its keys and values (the last ``W - 1`` positions fit) and
+        returns the logits of its last position, ``[1, vocab]``."""
+        n = prompt_ids.numel()
+        assert n > 0
+        logits, kv = self.model.prefill(prompt_ids.view(1, n))
+        self.cache.bulk_write_packed(kv, n)
+        self._remember(prompt_ids)
+        return self._trim(logits)
+
+    def _contexts(self) -> Tuple[List, List]:
+        if self._rings is not None:
+            for ring in self._rings:      # the handles are reused; only the position moves
+                ring.t = self.cache.t
+            return self._rings, self._rings
+        views = [self.cache.view(i) for i in range(self.cache.L)]
+        for k, v in views:
+            assert k.dtype == self.dtype and v.dtype == self.dtype
+        return [k for k, _ in views], [v for _, v in views]
+
+    def _step(self, token: Tensor) -> Tensor:
+        """One decode step: the model sees every layer's context as it was before this token,
+        the new rows go into slot ``t % W`` (unless the decode kernel has already put them
+        there), the cache moves on by one position."""
+        k_ctxs, v_ctxs = self._contexts()
+        logits, k_rows, v_rows = self.model.step(token, k_ctxs, v_ctxs, self.cache.t)
+        # A layer without attention returns None; its slot is filled with zeros shaped like the
+        # first layer's row, as the reference does (generate.py:240-241).
+        blank = None
+        for layer, (k_row, v_row) in enumerate(zip(k_rows, v_rows)):
+            if self.cache._staged[layer]:
+                continue
+            if k_row is None or v_row is None:
+                if blank is None:
+                    blank = torch.zeros_like(k_rows[0], dtype=self.dtype)
+                k_row = v_row = blank
+            self.cache.write(layer, k_row.to(self.dtype), v_row.to(self.dtype))
         self.cache.advance()
-        self.history = torch.cat([self.history, token.view(1)], dim=0)
-        return logits
+        self._remember(token)
+        return self._trim(logits)
 
+    # -- the loop --------------------------------------------------------------------------
     @torch.inference_mode()
-    def generate(self, prompt_ids: torch.Tensor, max_new_tokens) -> _GeneratorType[torch.Tensor, None, tuple]:
-        """Yields generated ids; returns ``(history, prefill_seconds, step_seconds)``."""
-        assert prompt_ids.ndim == 1
-        assert prompt_ids.size(0) > 0
-        assert max_new_tokens > 0
+    def generate(self, prompt_ids: Tensor, max_new_tokens) -> Iterator[Tensor]:
+        """Yields one ``[1]`` id tensor per generated token and stops at the end-of-sequence token
+        (not yielded) or after ``max_new_tokens``; the generator's return value is
+        ``(history, prefill_seconds, decode_seconds)``."""
+        assert prompt_ids.ndim == 1 and prompt_ids.numel() > 0 and max_new_tokens > 0
         self.reset_history()
-        self._sync(); t0 = time.perf_counter()
+        self._sync()
+        t_start = time.perf_counter()
         logits = self._prefill(prompt_ids)
-        self._sync(); t1 = time.perf_counter()
-        for i in range(max_new_tokens):
-            logits = logits[-1]
-            prev_ids = self.history[-128:]
-            logits = self.apply_repetition_penalty(logits, prev_ids, self.rep_p_t, self._one)
-            tok = self.sample(logits, self.temperature, self.top_k, self.top_p)
-            if tok == self.eos_token_id:
+        self._sync()
+        t_prompt = time.perf_counter()
+        for produced in range(1, max_new_tokens + 1):
+            scores = self.apply_repetition_penalty(logits[-1], self.history[-_PENALTY_LOOKBACK:], self.rep_p_t, self._one)
+            token = self.sample(scores, self.temperature, self.top_k, self.top_p)
+            if token == self.eos_token_id:
                 break
-            yield tok.view(1)
-            if i < max_new_tokens - 1:
-                logits = self._step(tok)
+            yield token.view(1)
+            if produced < max_new_tokens:
+                logits = self._step(token)
             else:
-                t = tok.to(device=self.device, dtype=torch.long).reshape(())
-                self.history = torch.cat([self.history, t.view(1)], dim=0)
-                logits = None
-        self._sync(); t2 = time.perf_counter()
-        return self.history.detach().clone(), t1 - t0, t2 - t1
+                self._remember(token)     # the last token is recorded but not run through the model
+        self._sync()
+        t_end = time.perf_counter()
+        return self.history.detach().clone(), t_prompt - t_start, t_end - t_prompt

@@ -1,16 +1,20 @@
-"""Ring-buffer KV cache with the reference's interface (inference/kv_cache.py:4-68).
+"""Ring-buffer KV cache with the public surface of the reference's ``KVCache``
+(inference/kv_cache.py:4-68): storage ``k, v [L, B, H, W, D]``, the token at
+position ``p`` lives in slot ``p % W``, ``view`` returns the live rows in
+chronological order, ``write`` stages the row of position ``t`` and ``advance``
+moves on by one position.
 
-Storage is ``k, v [L, B, H, W, D]``; the token at absolute position ``p`` lives
-in slot ``p % W``.  On top of the reference's methods the cache hands out a
-``RingContext`` per layer so that the decode kernel can stream the ring in place
-(physical order) and append the new row itself, instead of receiving a
-chronological copy.
+``ring(layer)`` is an addition for the HIP decode kernel: it hands out the layer's
+storage as it lies (slot order) so that a decode step reads the ring in place,
+writes the new row itself, and no chronological copy is ever made.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
+from typing import Optional, Tuple
 
 import torch
+from torch import Tensor
 
 
 @dataclass
@@ -23,8 +27,8 @@ class RingContext:
     """
     cache: "KVCache"
     layer: int
-    k: torch.Tensor
-    v: torch.Tensor
+    k: Tensor
+    v: Tensor
     t: int
     W: int
 
@@ -33,76 +37,89 @@ class RingContext:
 
 
 class KVCache:
+    """``t`` positions have been committed; a layer whose row for position ``t`` has been written
+    but not yet committed is *staged* (``advance`` commits all layers at once)."""
+
     def __init__(self, L, B, H, W, D, device, dtype):
-        self.H = H
-        self.B = B
-        self.D = D
-        self.W = W
-        self.L = L
+        self.L, self.B, self.H, self.W, self.D = L, B, H, W, D
+        self.device, self.dtype = device, dtype
+        self.k = torch.zeros((L, B, H, W, D), device=device, dtype=dtype)
+        self.v = torch.zeros_like(self.k)
         self.t = 0
-        self.device = device
-        self.dtype = dtype
-        self.k = torch.zeros(L, B, H, W, D, device=device, dtype=dtype)
-        self.v = torch.zeros(L, B, H, W, D, device=device, dtype=dtype)
         self._staged = [False] * L
 
     def reset_history(self):
-        # The reference allocates fresh zero tensors here (kv_cache.py:19-23); the
-        # storage is reused instead so that a long-lived cache never reallocates.
-        self.k.zero_()
-        self.v.zero_()
+        # The reference allocates fresh zero tensors here (kv_cache.py:19-23); the storage is
+        # reused instead so that a long-lived cache never reallocates.
+        for store in (self.k, self.v):
+            store.zero_()
         self.t = 0
         self._staged = [False] * self.L
 
-    def view(self, layer):
-        """Chronological last ``min(t + staged, W)`` rows as ``[B, n, H, D]``."""
-        staged = 1 if self._staged[layer] else 0
-        m = self.t + staged
-        n = min(m, self.W)
-        if n == 0:
-            return self.k[layer, :, :, :0, :].transpose(1, 2), self.v[layer, :, :, :0, :].transpose(1, 2)
-        end = (self.t + staged) % self.W
-        start = (end - n) % self.W
-        if start < end:
-            k = self.k[layer, :, :, start:end, :]
-            v = self.v[layer, :, :, start:end, :]
-        else:
-            k = torch.cat([self.k[layer, :, :, start:, :], self.k[layer, :, :, :end, :]], dim=2)
-            v = torch.cat([self.v[layer, :, :, start:, :], self.v[layer, :, :, :end, :]], dim=2)
-        return k.transpose(1, 2), v.transpose(1, 2)
+    # -- reading -----------------------------------------------------------------------------
+    def _live_rows(self, layer) -> Tuple[int, int]:
+        """(first position, number of rows) that ``view`` shows: the newest ``min(written, W)``."""
+        written = self.t + (1 if self._staged[layer] else 0)
+        rows = min(written, self.W)
+        return written - rows, rows
+
+    def view(self, layer) -> Tuple[Tensor, Tensor]:
+        """The live rows of a layer, oldest first, as ``[B, n, H, D]`` (``n = 0`` for an empty
+        cache).  A run of slots that does not wrap is returned as a view; a run that wraps is
+        the tail of the ring followed by its head (a copy)."""
+        first, rows = self._live_rows(layer)
+        lo = first % self.W if rows else 0
+        hi = lo + rows
+        out = []
+        for store in (self.k[layer], self.v[layer]):          # [B, H, W, D]
+            if hi <= self.W:
+                run = store[:, :, lo:hi]
+            else:
+                run = torch.cat((store[:, :, lo:], store[:, :, :hi - self.W]), dim=2)
+            out.append(run.transpose(1, 2))
+        return out[0], out[1]
 
     def ring(self, layer) -> RingContext:
         """In-place handle for the decode kernel (no copy)."""
         return RingContext(self, layer, self.k[layer], self.v[layer], self.t, self.W)
 
+    # -- writing -----------------------------------------------------------------------------
     def write(self, layer, k_new, v_new):
-        """Stages the row of position ``t``; accepts ``[B, 1, H, D]`` or ``[B, H, 1, D]``."""
-        if k_new.size(1) == 1:
-            k_new = k_new.transpose(1, 2)
-            v_new = v_new.transpose(1, 2)
-        i = self.t % self.W
-        self.k[layer, :, :, i:i + 1, :] = k_new
-        self.v[layer, :, :, i:i + 1, :] = v_new
+        """Stages the row of position ``t`` in slot ``t % W``.  A row may come as ``[B, 1, H, D]``
+        or ``[B, H, 1, D]``; as in the reference, a size-1 second dim marks the former."""
+        slot = self.t % self.W
+        for store, row in ((self.k, k_new), (self.v, v_new)):
+            if row.size(1) == 1:
+                row = row.transpose(1, 2)
+            store[layer, :, :, slot] = row[:, :, 0]
         self._staged[layer] = True
 
     def advance(self):
+        """Commits the staged rows of all layers: position ``t`` is done."""
         self.t += 1
         self._staged = [False] * self.L
 
+    def _prompt_slots(self, pos) -> Tuple[slice, Optional[Tensor]]:
+        """A prompt of ``pos`` tokens leaves room for the token that follows: only its last
+        ``min(pos, W - 1)`` positions are kept.  Returns their source range and target slots."""
+        kept = min(pos, max(self.W - 1, 0))
+        if kept == 0:
+            return slice(0, 0), None
+        positions = torch.arange(pos - kept, pos, device=self.k.device)
+        return slice(pos - kept, pos), positions.remainder_(self.W)
+
     def bulk_write_packed(self, kv, pos):
-        """Stores the last ``min(pos, W - 1)`` positions of ``kv [2, L, B, H, T, D]``."""
-        r = min(pos, max(self.W - 1, 0))
-        if r > 0:
-            idx = torch.arange(pos - r, pos, device=self.k.device) % self.W
-            self.k[:, :, :, idx, :] = kv[0][:, :, :, pos - r:pos, :].to(self.dtype)
-            self.v[:, :, :, idx, :] = kv[1][:, :, :, pos - r:pos, :].to(self.dtype)
+        """Stores a prompt's keys and values from ``kv [2, L, B, H, T, D]`` and sets ``t = pos``."""
+        src, slots = self._prompt_slots(pos)
+        if slots is not None:
+            self.k.index_copy_(3, slots, kv[0][:, :, :, src].to(self.dtype))
+            self.v.index_copy_(3, slots, kv[1][:, :, :, src].to(self.dtype))
         self.t = pos
         self._staged = [False] * self.L
 
     def bulk_write_layer(self, layer, k, v, pos):
         """Per-layer form of ``bulk_write_packed`` for ``k, v [B, H, T, D]``; does not move ``t``."""
-        r = min(pos, max(self.W - 1, 0))
-        if r > 0:
-            idx = torch.arange(pos - r, pos, device=self.k.device) % self.W
-            self.k[layer][:, :, idx, :] = k[:, :, pos - r:pos, :].to(self.dtype)
-            self.v[layer][:, :, idx, :] = v[:, :, pos - r:pos, :].to(self.dtype)
+        src, slots = self._prompt_slots(pos)
+        if slots is not None:
+            self.k[layer].index_copy_(2, slots, k[:, :, src].to(self.dtype))
+            self.v[layer].index_copy_(2, slots, v[:, :, src].to(self.dtype))

@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu]
 
-NAME is one of prefill | ceiling | module | long | decode | kda | copy; "copy" runs a plain 1 GiB
+NAME is one of prefill | ceiling | module | long | decode | kda | next | copy; "copy" runs a plain 1 GiB
 device copy and nothing else (the known-size kernel against which the HBM
 counters FETCH_SIZE / WRITE_SIZE are calibrated under rocprofv3 --pmc).
 
@@ -285,12 +285,126 @@ def bench_kda_c5(steps, warmup, cpu_baseline=True):
     return out
 
 
+def bench_next_rows(steps, warmup):
+    """The callers either side of the kernels: model-level prefill / step glue on an attention stack,
+    attention under training-time block masks, and the KDA layer."""
+    import torch.nn as nn
+    import torch.nn.functional as F
+    from daisy_amd import CausalSelfAttention, KVCache, KimiLinearSelfAttention, build_block_window_masks, core, ops
+    dev = "cuda:0"
+    out = {}
+
+    # ---- glue: 4 attention layers, 16 sequences, prompt 2048, window 4096 ------------------------
+    class Block(nn.Module):
+        def __init__(self, dim, H, D, max_len):
+            super().__init__()
+            self.attn = CausalSelfAttention(dim, H, D, max_seq_len=max_len)
+            with torch.no_grad():
+                self.attn.qkvo_w.copy_((torch.randn(4, dim, dim) * 0.02).bfloat16())
+
+        def prefill(self, x, ve, x0, attn_mask=None, debug=False):
+            y, k, v = self.attn.prefill(x, ve, attn_mask, debug=debug)
+            return x + y, k, v
+
+        def step(self, x, ve, x0, k_ctx, v_ctx, pos, window):
+            y, k, v = self.attn.step(x, k_ctx, v_ctx, pos, ve, window=window)
+            return x + y, k, v
+
+    class Stack(nn.Module):
+        def __init__(self, L=4, vocab=1024, dim=1024, H=8, D=128, window=4096, max_len=8192):
+            super().__init__()
+            self.embed = nn.Embedding(vocab, dim)
+            self.blocks = nn.ModuleList([Block(dim, H, D, max_len) for _ in range(L)])
+            self.skip_map, self.skip_weights, self.ve_module_map = {}, None, {}
+            self.lm_head_w = nn.Parameter(torch.randn(vocab, dim) * 0.02)
+            self.window_size = self.attn_window_size = window
+            self.eos_token_id = 0
+            self.attn_num_heads, self.attn_head_dim = H, D
+            self.bfloat16()
+
+    torch.manual_seed(0)
+    with torch.no_grad():
+        model = Stack().to(dev).eval()
+        Bs, T0, W, L = 16, 2048, 4096, 4
+        ids = torch.randint(1, 1024, (Bs, T0), device=dev)
+        cache = KVCache(L=L, B=Bs, H=8, W=W, D=128, device=dev, dtype=torch.bfloat16)
+
+        def prefill_direct():
+            cache.reset_history()
+            return core.prefill(model, ids, cache)
+
+        def prefill_stacked():   # the reference's route: stack [2, L, B, H, T, D], then one bulk write
+            cache.reset_history()
+            logits, kv = core.prefill(model, ids)
+            cache.bulk_write_packed(kv, T0)
+            return logits
+
+        ms_direct = time_gpu(prefill_direct, max(steps // 5, 3), 2)
+        ms_stacked = time_gpu(prefill_stacked, max(steps // 5, 3), 2)
+        prefill_direct()
+        tok = torch.randint(1, 1024, (Bs,), device=dev)
+        t_before = cache.t
+
+        def step_ring():
+            cache.t = t_before
+            return core.step(model, tok, cache)
+
+        def step_views():        # chronological copies, the reference's route (cache.view + write)
+            cache.t = t_before
+            x = x0 = F.rms_norm(model.embed(tok.view(-1, 1)), (1024,))
+            for i, blk in enumerate(model.blocks):
+                kc, vc = cache.view(i)
+                x, kn, vn = blk.step(x, None, x0, kc, vc, cache.t, W)
+                cache.write(i, kn, vn)
+            cache.advance()
+            return F.linear(F.rms_norm(x, (1024,)).flatten(end_dim=1), model.lm_head_w).float()
+
+        ms_ring = time_gpu(step_ring, 64, 8)
+        ms_views = time_gpu(step_views, 64, 8)
+    out["model_glue_L4_B16_T2048_W4096"] = {
+        "prefill_ms_ring_written_per_layer": ms_direct, "prefill_ms_stack_then_bulk_write": ms_stacked,
+        "step_ms_ring_in_place": ms_ring, "step_ms_chronological_views": ms_views,
+        "kv_bytes_per_step": 2 * L * Bs * 8 * min(t_before + 1, W) * 128 * 2}
+    del model, cache
+
+    # ---- training-time block masks as per-row lower bounds: one sequence of 32768, 3 documents ----
+    with torch.no_grad():
+        T, H, D, wblk = 32768, 8, 128, 8          # window of 8 blocks of 128 = 1024 keys
+        seq = torch.randint(1, 1000, (T,), device=dev)
+        seq[[9000, 20000]] = 0
+        masks = build_block_window_masks(seq, wblk, 4, eos_token_id=0)
+        g = torch.Generator(device=dev).manual_seed(0)
+        q, k, v = (torch.randn(1, T, H, D, generator=g, device=dev).bfloat16() for _ in range(3))
+        rows = {}
+        for name, m in (("long", masks[0]), ("short", masks[1])):
+            lo = m.doc_start.long()
+            pairs = int((torch.arange(T, device=dev) - lo + 1).sum())
+            o_buf = torch.empty_like(q)
+            ms = time_gpu(lambda: ops.prefill_attention(q, k, v, window=None, doc_start=m.doc_start, scale=SCALE, out=o_buf), max(steps // 2, 5), 3)
+            fl = 4.0 * D * H * pairs
+            rows[name] = {"ms": ms, "flops": fl, "tflops": fl / ms / 1e9, "frac_of_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS}
+    out["block_masks_B1_T32768_H8_D128_w8blocks"] = rows
+
+    # ---- the KDA layer: dim 2048, 16 heads of 128, B4 T8192; one decode step at batch 64 ------------
+    with torch.no_grad():
+        torch.manual_seed(0)
+        layer = KimiLinearSelfAttention(2048, 16, max_seq_len=8192, head_dim=128).to(dev).eval()
+        x = torch.randn(4, 8192, 2048, device=dev).bfloat16()
+        ms_layer = time_gpu(lambda: layer(x, None), max(steps // 10, 3), 2)
+        xs = torch.randn(64, 64, 2048, device=dev).bfloat16()
+        layer.prefill(xs, None)
+        x1 = torch.randn(64, 1, 2048, device=dev).bfloat16()
+        ms_step = time_gpu(lambda: layer.step(x1, None, None, 64, None, None), 32, 4)
+    out["kimi_layer_dim2048_H16"] = {"forward_ms_B4_T8192": ms_layer, "step_ms_B64": ms_step}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", default=None, help="prefill | ceiling | module | long | decode | kda | copy (default: all but copy)")
+    ap.add_argument("--only", default=None, help="prefill | ceiling | module | long | decode | kda | next | copy (default: all but copy)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -323,6 +437,8 @@ def main():
         extra["decode_c4"] = bench_decode_c4(256, 16, cpu)
         from daisy_amd import ops
         extra["hbm_read_ceiling"] = dict(ops.probe_read_rate(), what="read-only stream of 2 GiB, 8192 workgroups, 128 B in flight per lane")
+    if want("next"):
+        extra["next_rows"] = bench_next_rows(args.steps, args.warmup)
     if want("kda"):
         try:
             extra["kda_c5"] = bench_kda_c5(max(args.steps // 5, 4), max(args.warmup // 2, 2), cpu)

@@ -60,6 +60,12 @@ SIGNATURES = {
         c_float, c_float, c_void_p]),                           # softplus beta, threshold, stream
     "daisy_probe_matrix_rate": (c_int, [
         c_int, c_int, c_int, c_void_p, c_void_p, POINTER(ctypes.c_double), c_void_p]),
+    "daisy_short_conv_fwd": (c_int, [
+        c_void_p, _I64P, c_void_p, c_void_p, c_void_p,          # x (+ strides), weight, bias, cache_in
+        c_void_p, _I64P, c_void_p,                              # y (+ strides), cache_out
+        c_int, c_int, c_int, c_int, c_int, c_void_p]),          # B, T, C, K, apply_silu, stream
+    "daisy_gated_rmsnorm_fwd": (c_int, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_float, c_void_p]),
     "daisy_probe_read_rate": (c_int, [c_void_p, ctypes.c_size_t, c_int, c_void_p, c_void_p]),
     "daisy_qkv_prep_fwd": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q, k, v (+ strides)

@@ -14,8 +14,10 @@ Same parameters and names as the reference's ``KimiLinearSelfAttention`` (``q_pr
     y       = o_proj(rms_norm(o) * o_norm.weight * sigmoid(g_proj(x)))
 
 The delta-rule core runs on the HIP kernels (``chunk_kda`` for sequences, ``fused_recurrent_kda``
-with the state updated in place for single-token steps); projections, the four-tap convolution
-and the gated norm are PyTorch ops.  Three pieces of the reference come from the absent
+with the state updated in place for single-token steps), and so do the four-tap convolutions
+with their SiLU and the gated norm (one streaming kernel each, ``daisy_short_conv_fwd`` and
+``daisy_gated_rmsnorm_fwd``; on the CPU the same arithmetic runs as PyTorch ops); the projections
+are library GEMMs.  Three pieces of the reference come from the absent
 ``flash-linear-attention`` package and are restated from their documented behaviour, not pinned
 against it: ``ShortConvolution`` (depthwise causal conv + SiLU with a ``[B, C, K]`` state) and
 the gated RMS norm (``FusedRMSNormGated(activation="sigmoid", eps=1e-5)``, the module the
@@ -29,6 +31,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
+from . import ops
 from .kda import chunk_kda, fused_kda_gate, fused_recurrent_kda
 
 
@@ -68,6 +71,9 @@ class ShortConvolution(nn.Module):
             return torch.cat(ys, dim=1), (torch.cat(caches, dim=0) if output_final_state else None)
         B, T, C = x.shape
         K = self.kernel_size
+        if x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and 2 <= K <= 4 and C % 8 == 0:
+            # one streaming pass on the GPU (no transposes, no concatenation)
+            return ops.short_conv(x, self.weight, self.bias, cache, output_final_state, "silu")
         xt = x.transpose(1, 2)                                        # [B, C, T]
         prev = cache[..., 1:] if cache is not None else xt.new_zeros(B, C, K - 1)
         window = torch.cat([prev.to(xt.dtype), xt], dim=-1)           # [B, C, K - 1 + T]
@@ -88,6 +94,9 @@ class GatedRMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype))
 
     def forward(self, x: Tensor, gate: Tensor) -> Tensor:
+        if (x.is_cuda and x.dtype == gate.dtype == self.weight.dtype == torch.bfloat16
+                and self.hidden_size in (64, 128) and x.shape == gate.shape):
+            return ops.gated_rmsnorm(x, gate, self.weight, self.eps)
         xf = x.float()
         normed = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()
         return (normed * torch.sigmoid(gate.float())).to(x.dtype)

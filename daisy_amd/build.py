@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_NAME = "libdaisy_hip.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
-SOURCES = ["abi.hip", "decode.hip", "prefill.hip", "kda.hip", "kda_step.hip", "prep.hip", "probe.hip"]
+SOURCES = ["abi.hip", "decode.hip", "prefill.hip", "kda.hip", "kda_step.hip", "prep.hip", "kimi.hip", "probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

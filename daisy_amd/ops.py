@@ -366,3 +366,56 @@ def probe_read_rate(gib: int = 2, workgroups: int = 8192, repeats: int = 5, devi
         torch.cuda.synchronize(dev)
     ms = start.elapsed_time(end) / repeats
     return {"ms": ms, "bytes": nbytes, "gbs": nbytes / ms / 1e6}
+
+
+def short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               cache: Optional[torch.Tensor] = None, output_final_state: bool = False,
+               activation: Optional[str] = "silu") -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Depthwise causal convolution over time + SiLU for ``x [B, T, C]`` bf16 (``daisy_short_conv_fwd``).
+
+    ``weight [C, 1, K]`` or ``[C, K]``; ``cache [B, C, K]`` holds the last K inputs of the sequence
+    so far.  Returns ``(y [B, T, C], new cache or None)``.
+    """
+    dev = _lib.require_gpu(x, weight, bias, cache)
+    _check_bf16("x", x, 3)
+    B, T, C = x.shape
+    w = weight.reshape(C, -1)
+    K = w.shape[1]
+    if w.dtype != torch.bfloat16 or (bias is not None and bias.dtype != torch.bfloat16):
+        raise TypeError("short_conv: weight and bias must be bf16")
+    if activation not in (None, "silu"):
+        raise ValueError(f"short_conv: activation {activation!r} not supported")
+    if x.stride(2) != 1:
+        x = x.contiguous()
+    w = w.contiguous()
+    if cache is not None:
+        if cache.shape != (B, C, K):
+            raise ValueError(f"short_conv: cache must be [{B}, {C}, {K}], got {tuple(cache.shape)}")
+        cache = cache.to(torch.bfloat16).contiguous()
+    y = torch.empty(B, T, C, dtype=torch.bfloat16, device=dev)
+    new_cache = torch.empty(B, C, K, dtype=torch.bfloat16, device=dev) if output_final_state else None
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.daisy_short_conv_fwd(x.data_ptr(), _lib.strides(x, (0, 1)), w.data_ptr(), _lib.ptr(bias), _lib.ptr(cache),
+                                      y.data_ptr(), _lib.strides(y, (0, 1)), _lib.ptr(new_cache),
+                                      B, T, C, K, 1 if activation == "silu" else 0, _lib.current_stream(dev))
+    _lib.check(rc, "daisy_short_conv_fwd")
+    return y, new_cache
+
+
+def gated_rmsnorm(x: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
+    """``x * rsqrt(mean(x^2) + eps) * weight * sigmoid(gate)`` over the last dim (64 or 128), bf16."""
+    dev = _lib.require_gpu(x, gate, weight)
+    if x.dtype != torch.bfloat16 or gate.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError("gated_rmsnorm: x, gate and weight must be bf16")
+    if gate.shape != x.shape or weight.numel() != x.shape[-1]:
+        raise ValueError(f"gated_rmsnorm: shapes {tuple(x.shape)}, {tuple(gate.shape)}, {tuple(weight.shape)} do not match")
+    xc, gc, wc = x.contiguous(), gate.contiguous(), weight.contiguous()
+    out = torch.empty_like(xc)
+    D = x.shape[-1]
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        rc = lib.daisy_gated_rmsnorm_fwd(xc.data_ptr(), gc.data_ptr(), wc.data_ptr(), out.data_ptr(),
+                                         xc.numel() // D, D, float(eps), _lib.current_stream(dev))
+    _lib.check(rc, "daisy_gated_rmsnorm_fwd")
+    return out

@@ -209,6 +209,32 @@ int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
                        int B, int T, int H, int D, float eps, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * The KDA layer's elementwise neighbours (models/daisy/attention_kimi.py:155-158: three
+ * ShortConvolution modules in front of chunk_kda; :136-137: the gated RMS norm behind it; both
+ * modules come from a package absent from the reference checkout and are restated from their
+ * documented arithmetic).
+ *
+ * daisy_short_conv_fwd: depthwise causal convolution over time with K taps (2..4) per channel,
+ * optional bias and SiLU, bf16 in and out:
+ *     y[b, t, c] = act( bias[c] + sum_j weight[c, j] * x[b, t - (K-1) + j, c] )
+ * x, y       : [B, T, C] bf16, channel stride 1, strides = {batch, time} in elements (multiples of 8)
+ * weight     : [C, K] bf16 (the layout of a grouped Conv1d weight [C, 1, K]); bias: [C] bf16 or NULL
+ * cache_in   : [B, C, K] bf16 or NULL -- the last K inputs before t = 0 (zeros if NULL)
+ * cache_out  : [B, C, K] bf16 or NULL -- receives the last K inputs of (cache_in | x)
+ * C must be a multiple of 8.
+ */
+int daisy_short_conv_fwd(const void* x, const int64_t* x_strides, const void* weight, const void* bias,
+                         const void* cache_in, void* y, const int64_t* y_strides, void* cache_out,
+                         int B, int T, int C, int K, int apply_silu, void* stream);
+
+/* daisy_gated_rmsnorm_fwd: out = x * rsqrt(mean(x^2) + eps) * weight * sigmoid(gate) over the last
+ * dim, statistics in fp32, one rounding.  x, gate, out: [rows, D] bf16 contiguous; weight: [D] bf16;
+ * D = 64 or 128.
+ */
+int daisy_gated_rmsnorm_fwd(const void* x, const void* gate, const void* weight, void* out,
+                            int64_t rows, int D, float eps, void* stream);
+
+/* ---------------------------------------------------------------------------
  * Diagnostic (no counterpart in the reference): launches `workgroups` workgroups
  * of 8 wavefronts (two per SIMD) that each issue 8 * iters independent
  * v_mfma_f32_32x32x16_bf16 from registers -- alone (with_vector_mix = 0) or with

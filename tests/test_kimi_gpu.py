@@ -135,3 +135,55 @@ def test_padding_mask_packs_sequences():
             m.prefill(x[b:b + 1, S - n:], None)
             y1_b, _, _ = m.step(x1[b:b + 1], None, None, n, None, None)
             _close(y1[b], y1_b[0], f"step after padded prefill, row {b}", 2e-2)
+
+
+@pytest.mark.parametrize("B,T,C,K,bias,with_cache", [(2, 70, 256, 4, False, False), (1, 1, 64, 4, True, True),
+                                                     (3, 33, 128, 3, True, True), (1, 200, 2048, 4, False, True),
+                                                     (2, 2, 64, 2, False, True)])
+def test_short_convolution_kernel_matches_library_ops(B, T, C, K, bias, with_cache):
+    """The streaming kernel against the same module on the CPU (grouped conv1d + SiLU in bf16)."""
+    from daisy_amd.attention_kimi import ShortConvolution
+    torch.manual_seed(T + C)
+    m = ShortConvolution(C, K, bias=bias)
+    if bias:
+        with torch.no_grad():
+            m.bias.copy_((torch.randn(C) * 0.3).bfloat16())
+    x = torch.randn(B, T, C).bfloat16()
+    cache = torch.randn(B, C, K).bfloat16() if with_cache else None
+    with torch.no_grad():
+        y_ref, c_ref = m(x, cache, output_final_state=True)
+        md = ShortConvolution(C, K, bias=bias).to(DEV)
+        md.load_state_dict(m.state_dict())
+        y, c = md(x.to(DEV), None if cache is None else cache.to(DEV), output_final_state=True)
+    assert y.shape == (B, T, C) and c.shape == (B, C, K)
+    assert torch.equal(c.cpu(), c_ref), "carried window differs"
+    # identical up to one bf16 rounding of the pre-activation (the summation order may differ)
+    err = (y.float().cpu() - y_ref.float()).abs()
+    tol = 2.0 ** -7 * y_ref.float().abs().clamp_min(0.25)
+    say(f"short conv B{B} T{T} C{C} K{K}: max-abs {err.max().item():.3e}, mismatching {(err > 0).float().mean().item():.2%}")
+    assert bool((err <= tol).all())
+    # a sequence cut in two with the window carried equals the sequence in one go
+    if T >= 2:
+        with torch.no_grad():
+            h = T // 2
+            y1, c1 = md(x[:, :h].to(DEV), None if cache is None else cache.to(DEV), output_final_state=True)
+            y2, c2 = md(x[:, h:].to(DEV), c1, output_final_state=True)
+        assert torch.equal(torch.cat([y1, y2], dim=1), y) and torch.equal(c2, c)
+
+
+@pytest.mark.parametrize("rows,D", [(5, 128), (1000, 128), (77, 64)])
+def test_gated_rmsnorm_kernel_matches_formula(rows, D):
+    from daisy_amd.attention_kimi import GatedRMSNorm
+    torch.manual_seed(rows)
+    m = GatedRMSNorm(D)
+    with torch.no_grad():
+        m.weight.copy_((1 + 0.2 * torch.randn(D)).bfloat16())
+    x, g = torch.randn(rows, D).bfloat16() * 3, torch.randn(rows, D).bfloat16() * 2
+    with torch.no_grad():
+        ref = m(x, g)
+        md = GatedRMSNorm(D).to(DEV)
+        md.load_state_dict(m.state_dict())
+        out = md(x.to(DEV), g.to(DEV))
+    err = (out.float().cpu() - ref.float()).abs()
+    say(f"gated norm rows{rows} D{D}: max-abs {err.max().item():.3e}")
+    assert bool((err <= 2.0 ** -7 * ref.float().abs().clamp_min(1e-3)).all())

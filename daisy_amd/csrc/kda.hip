@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void kda_gate_kernel(const void* g, const floa
 // Numerics: the 16x16 blocks of A and P run on MFMA with both operands
 // referenced to the row before the block (every exponent <= 0 off the diagonal);
 // a diagonal block whose total decay exceeds exp(-80) is instead accumulated in
-// fp32 from running products of exp(g) (no exponent is ever positive, so strong
+// fp32 pair by pair with exp(G_i - G_j), j < i (no exponent is ever positive, so strong
 // decays cannot overflow).  The triangular solve works on 16-row blocks: fp32
 // inverses of the diagonal blocks, everything else as products of two-term bf16
 // splits (three MFMAs each, relative error ~2^-17).  The state update uses the
@@ -161,21 +161,29 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   {
     const int d = tid & 127, half = tid >> 7;
     float gv[32];
+    // Rows past the end re-read the last row (always valid) and are zeroed afterwards, so that
+    // the loads carry no branches and all go out together; the dtype is decided once, outside
+    // the loops, for the same reason.  bf16 g: the two channels of a pair read the same dword
+    // (no sub-dword loads) and take their half.
+    uint32_t graw[32];
+    if (p.g_bf16) {
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        const int64_t off = row_off(min(32 * half + i, p.T - 1 - t0)) + d;
+        graw[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p.g) + (off >> 1));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        const int64_t off = row_off(min(32 * half + i, p.T - 1 - t0)) + d;
+        graw[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p.g) + off);
+      }
+    }
+    const bool g16 = p.g_bf16 != 0, odd = (d & 1) != 0;
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
-      const int r = 32 * half + i;
-      // Rows past the end re-read the last row (always valid) and are zeroed afterwards, so
-      // that the loads carry no branches and all go out together.
-      const int64_t off = row_off(min(r, p.T - 1 - t0)) + d;
-      // bf16 g: the two channels of a pair read the same dword (no sub-dword loads) and take their half
-      float x;
-      if (p.g_bf16) {
-        const uint32_t w2 = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p.g) + (off >> 1));
-        x = (d & 1) ? bf16hi_to_f32(w2) : bf16lo_to_f32(w2);
-      } else {
-        x = __builtin_nontemporal_load(((const float*)p.g) + off);
-      }
-      gv[i] = (t0 + r < p.T) ? x : 0.f;
+      const float x = g16 ? (odd ? bf16hi_to_f32(graw[i]) : bf16lo_to_f32(graw[i])) : __uint_as_float(graw[i]);
+      gv[i] = (t0 + 32 * half + i < p.T) ? x : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -351,10 +359,10 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       }
     }
   };
-  // Blocks by wavefront: 0 -> (0,0), (3,3); 1 -> (1,0), (1,1); 2 -> (2,0), (2,1), (2,2);
+  // Blocks by wavefront, normally: 0 -> (0,0), (3,3); 1 -> (1,0), (1,1); 2 -> (2,0), (2,1), (2,2);
   // 3 -> (3,0), (3,1), (3,2).  A diagonal block whose decay is too steep for the MFMA path (some
   // channel beyond exp(-80) across the block: the column factors could overflow) is accumulated
-  // in fp32 from running products of exp(g), where no exponent is ever positive.
+  // in fp32 pair by pair with exp(G_i - G_j), j < i, where no exponent is ever positive.
   auto steep_diagonal = [&](int I) {
     const int il = lane >> 2, dq = lane & 3;
     const int ri = 16 * I + il;
@@ -364,33 +372,23 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
 #pragma unroll 1
     for (int dc = 0; dc < 4; ++dc) {
       const int d0 = 32 * dq + 8 * dc;
-      float ki[8], qi[8], E[8];
+      float ki[8], qi[8];
       unpack8(*reinterpret_cast<const u32x4*>(&Kr[ri][d0]), ki);
       unpack8(*reinterpret_cast<const u32x4*>(&Qr[ri][d0]), qi);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) E[e] = 1.f;
+      const f32x4 gi0 = lds_f4(&G[ri][d0]), gi1 = lds_f4(&G[ri][d0 + 4]);
 #pragma unroll
       for (int j = 15; j >= 0; --j) {
         const int rj = 16 * I + j;
         float kj[8];
         unpack8(*reinterpret_cast<const u32x4*>(&Kr[rj][d0]), kj);
-        if (j < 15) {
-          // E = exp(G_i - G_j) for j < i: multiply in exp(g) of row j+1; rows j >= i restart at 1.
-          const f32x4 ga0 = lds_f4(&G[rj + 1][d0]), ga1 = lds_f4(&G[rj + 1][d0 + 4]);
-          const f32x4 gb0 = lds_f4(&G[rj][d0]), gb1 = lds_f4(&G[rj][d0 + 4]);
-          f32x4 e0, e1;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { e0[e] = __builtin_amdgcn_exp2f(ga0[e] - gb0[e]); e1[e] = __builtin_amdgcn_exp2f(ga1[e] - gb1[e]); }
-          const bool live = j < il;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            E[e] = live ? E[e] * e0[e] : 1.f;
-            E[4 + e] = live ? E[4 + e] * e1[e] : 1.f;
-          }
-        }
+        // exp(G_i - G_j) for j < i: the exponent is a sum of log-decays, never positive; rows at or
+        // above the diagonal take the factor 1 (only j == i is used, by P).
+        const f32x4 gj0 = lds_f4(&G[rj][d0]), gj1 = lds_f4(&G[rj][d0 + 4]);
+        const bool below = j < il;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const float t = kj[e] * E[e];
+          const float diff = (e < 4) ? gi0[e & 3] - gj0[e & 3] : gi1[e & 3] - gj1[e & 3];
+          const float t = kj[e] * (below ? __builtin_amdgcn_exp2f(diff) : 1.f);
           a[j] = fmaf(ki[e], t, a[j]);
           pp[j] = fmaf(qi[e], t, pp[j]);
         }
@@ -411,10 +409,19 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
     }
   };
   {
-    const int nseg = (wave == 0) ? 2 : 1;
-    for (int sg = 0; sg < nseg; ++sg) {
-      const int I = (wave == 0) ? 3 * sg : wave;
-      const int jlo = (wave == 0) ? I : 0, jhi = (wave == 3) ? 2 : I;
+    // Segments (block row I, columns jlo..jhi) per wavefront, 4 bits each, two per wavefront
+    // (0xf.. = none).  A steep diagonal block costs about as much as five others, so when there
+    // is one the blocks are dealt differently: 0 -> (0,0), (3,0..1); 1 -> (1,1), (3,2);
+    // 2 -> (2,0..2); 3 -> (3,3), (1,0).
+    const bool any_steep = (steep[0] | steep[1] | steep[2] | steep[3]) != 0;
+    constexpr uint32_t kPlain[4] = {0x333000u, 0xfff101u, 0xfff202u, 0xfff203u};   // (jhi, jlo, I) second | first
+    constexpr uint32_t kSteep[4] = {0x103000u, 0x223111u, 0xfff202u, 0x001333u};
+    uint32_t plan = any_steep ? kSteep[0] : kPlain[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) if (wave == w) plan = any_steep ? kSteep[w] : kPlain[w];
+    for (int sg = 0; sg < 2; ++sg, plan >>= 12) {
+      const int I = plan & 15, jlo = (plan >> 4) & 15, jhi = (plan >> 8) & 15;
+      if (I == 15) break;
       row_operands(I);
       for (int J = jlo; J <= jhi; ++J) {
         if (J == I && steep[I]) steep_diagonal(I);

@@ -294,7 +294,7 @@ def bench_next_rows(steps, warmup):
     dev = "cuda:0"
     out = {}
 
-    # ---- glue: 4 attention layers, 16 sequences, prompt 2048, window 4096 ------------------------
+    # ---- glue: 4 attention layers, 16 sequences, prompt 4100, ring of 4096 (wrapped) ----------------
     class Block(nn.Module):
         def __init__(self, dim, H, D, max_len):
             super().__init__()
@@ -325,7 +325,7 @@ def bench_next_rows(steps, warmup):
     torch.manual_seed(0)
     with torch.no_grad():
         model = Stack().to(dev).eval()
-        Bs, T0, W, L = 16, 2048, 4096, 4
+        Bs, T0, W, L = 16, 4100, 4096, 4
         ids = torch.randint(1, 1024, (Bs, T0), device=dev)
         cache = KVCache(L=L, B=Bs, H=8, W=W, D=128, device=dev, dtype=torch.bfloat16)
 
@@ -361,7 +361,7 @@ def bench_next_rows(steps, warmup):
 
         ms_ring = time_gpu(step_ring, 64, 8)
         ms_views = time_gpu(step_views, 64, 8)
-    out["model_glue_L4_B16_T2048_W4096"] = {
+    out["model_glue_L4_B16_T4100_W4096"] = {
         "prefill_ms_ring_written_per_layer": ms_direct, "prefill_ms_stack_then_bulk_write": ms_stacked,
         "step_ms_ring_in_place": ms_ring, "step_ms_chronological_views": ms_views,
         "kv_bytes_per_step": 2 * L * Bs * 8 * min(t_before + 1, W) * 128 * 2}

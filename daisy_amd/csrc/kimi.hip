@@ -41,14 +41,36 @@ __global__ __launch_bounds__(256) void short_conv_kernel(ConvParams p) {
   {
     // channel c's taps are K consecutive values; 8 channels = 8K consecutive bf16
     const uint16_t* wp = p.w + (int64_t)c0 * K;
+    if (K == 4) {   // 64 contiguous bytes: four 16-byte loads, two channels each
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
+      for (int v = 0; v < 4; ++v) {
+        float f[8];
+        unpack8(*reinterpret_cast<const u32x4*>(wp + 8 * v), f);
 #pragma unroll
-      for (int j = 0; j < K; ++j) w[j][e] = bf16lo_to_f32(wp[e * K + j]);
+        for (int j = 0; j < K; ++j) { w[j][2 * v] = f[j % 8]; w[j][2 * v + 1] = f[(4 + j) % 8]; }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+#pragma unroll
+        for (int j = 0; j < K; ++j) w[j][e] = bf16lo_to_f32(wp[e * K + j]);
+    }
     if (p.bias != nullptr) unpack8(*reinterpret_cast<const u32x4*>(p.bias + c0), acc0);
     else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc0[e] = 0.f;
+    }
+  }
+  // The carried window of 8 channels is 8K contiguous values; for K = 4 it is read and written
+  // as four 16-byte pieces (two channels each).
+  float carried[K][8];
+  if (K == 4 && p.cache_in != nullptr && t0 < K - 1) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float f[8];
+      unpack8(*reinterpret_cast<const u32x4*>(p.cache_in + ((int64_t)b * p.C + c0) * K + 8 * v), f);
+#pragma unroll
+      for (int j = 0; j < K; ++j) { carried[j][2 * v] = f[j % 8]; carried[j][2 * v + 1] = f[(4 + j) % 8]; }
     }
   }
   // Input at time ti (may be negative: carried window or zero).
@@ -56,8 +78,17 @@ __global__ __launch_bounds__(256) void short_conv_kernel(ConvParams p) {
     if (ti >= 0) {
       unpack8(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.x + b * p.x_sb + (int64_t)ti * p.x_st + c0)), f);
     } else if (p.cache_in != nullptr) {
+      if (K == 4) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) f[e] = bf16lo_to_f32(p.cache_in[((int64_t)b * p.C + c0 + e) * K + K + ti]);
+        for (int j = 1; j < K; ++j)
+          if (K + ti == j) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = carried[j][e];
+          }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = bf16lo_to_f32(p.cache_in[((int64_t)b * p.C + c0 + e) * K + K + ti]);
+      }
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) f[e] = 0.f;
@@ -99,13 +130,23 @@ __global__ __launch_bounds__(256) void short_conv_kernel(ConvParams p) {
   }
   // The thread that reaches the end of the sequence leaves the window for the next call.
   if (p.cache_out != nullptr && t1 == p.T) {
+    float last[K][8];
 #pragma unroll
-    for (int j = 0; j < K; ++j) {
-      float f[8];
-      input_at(p.T - K + j, f);
+    for (int j = 0; j < K; ++j) input_at(p.T - K + j, last[j]);
+    if (K == 4) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        p.cache_out[((int64_t)b * p.C + c0 + e) * K + j] = (uint16_t)(pack_bf16x2(f[e], 0.f) & 0xffffu);
+      for (int v = 0; v < 4; ++v) {
+        float f[8];
+#pragma unroll
+        for (int j = 0; j < K; ++j) { f[j % 8] = last[j][2 * v]; f[(4 + j) % 8] = last[j][2 * v + 1]; }
+        *reinterpret_cast<u32x4*>(p.cache_out + ((int64_t)b * p.C + c0) * K + 8 * v) = pack8(f);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < K; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          p.cache_out[((int64_t)b * p.C + c0 + e) * K + j] = (uint16_t)(pack_bf16x2(last[j][e], 0.f) & 0xffffu);
     }
   }
 }
@@ -149,7 +190,8 @@ extern "C" int daisy_short_conv_fwd(const void* x, const int64_t* x_strides, con
   DAISY_CHECK_SUPPORTED(C % 8 == 0, "short_conv: channels (%d) must be a multiple of 8", C);
   DAISY_CHECK_ARG(B <= 65535, "short_conv: B must be <= 65535");
   auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
-  DAISY_CHECK_ARG(al16(x) && al16(y) && al16(bias), "short_conv: x, y and bias must be 16-byte aligned");
+  DAISY_CHECK_ARG(al16(x) && al16(y) && al16(bias) && al16(weight) && al16(cache_in) && al16(cache_out),
+                  "short_conv: x, y, weight, bias and the windows must be 16-byte aligned");
   for (int i = 0; i < 2; ++i)
     DAISY_CHECK_ARG(x_strides[i] % 8 == 0 && y_strides[i] % 8 == 0, "short_conv: strides must be multiples of 8 elements");
   ConvParams p;

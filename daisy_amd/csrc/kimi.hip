@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(ConvParams p) {
 #pragma unroll
         for (int j = 0; j < K - 1; ++j) a = fmaf(w[j][e], win[j][e], a);
         a = round_bf16(fmaf(w[K - 1][e], xin[e], a));
-        if (p.silu) a = a / (1.f + __expf(-a));
+        if (p.silu) a = a * __builtin_amdgcn_rcpf(1.f + __expf(-a));
         out[e] = a;
       }
       if (tb + u < t1) *reinterpret_cast<u32x4*>(p.y + b * p.y_sb + (int64_t)(tb + u) * p.y_st + c0) = pack8(out);
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(GatedNormParams p) {
   ss = group_sum<LPR>(ss);
   const float rstd = rsqrtf(ss / (float)D + p.eps);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = x[e] * rstd * w[e] * (1.f / (1.f + __expf(-g[e])));
+  for (int e = 0; e < 8; ++e) o[e] = x[e] * rstd * w[e] * __builtin_amdgcn_rcpf(1.f + __expf(-g[e]));
   if (row < p.rows) *reinterpret_cast<u32x4*>(p.out + r * D + 8 * c) = pack8(o);
 }
 

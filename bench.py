@@ -109,9 +109,24 @@ def bench_prefill_c2(steps, warmup, cpu_baseline=True):
         "frac_of_peak_kernel": flops / ms_kernel / 1e9 / PEAK_BF16_TFLOPS,
     }
     if cpu_baseline:
-        res["cpu_baseline"] = cpu_prefill_baseline(q[:1].cpu(), k[:1].cpu(), v[:1].cpu(), cos.cpu(), sin.cpu(), W,
-                                                   f"1 of {B} batch elements, all {H} heads, T={T}")
+        res["cpu_baseline"] = cpu_prefill_baseline(q[:2].cpu(), k[:2].cpu(), v[:2].cpu(), cos.cpu(), sin.cpu(), W,
+                                                   f"2 of {B} batch elements, all {H} heads, T={T}")
     return res
+
+
+CPU_SECONDS = 10.0   # how long each CPU baseline keeps repeating its sample
+
+
+def _repeat_for(fn, seconds):
+    """Runs fn at least twice and until `seconds` have passed; returns (mean seconds per run, runs)."""
+    fn()   # first run untimed: thread pools, allocator
+    runs, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        runs += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds:
+            return dt / runs, runs
 
 
 def cpu_prefill_baseline(q, k, v, cos, sin, W, sample):
@@ -120,13 +135,15 @@ def cpu_prefill_baseline(q, k, v, cos, sin, W, sample):
     torch.set_num_threads(os.cpu_count() or 1)
     B, T, H, D = q.shape
     mask = oracle.window_mask(T, W)
-    t0 = time.perf_counter()
-    qr, kr = oracle.apply_rope(q, cos[:T], sin[:T]), oracle.apply_rope(k, cos[:T], sin[:T])
-    torch.nn.functional.scaled_dot_product_attention(qr.transpose(1, 2), kr.transpose(1, 2), v.transpose(1, 2),
-                                                     attn_mask=mask, scale=SCALE)
-    dt = time.perf_counter() - t0
+
+    def one_pass():
+        qr, kr = oracle.apply_rope(q, cos[:T], sin[:T]), oracle.apply_rope(k, cos[:T], sin[:T])
+        torch.nn.functional.scaled_dot_product_attention(qr.transpose(1, 2), kr.transpose(1, 2), v.transpose(1, 2),
+                                                         attn_mask=mask, scale=SCALE)
+
+    dt, runs = _repeat_for(one_pass, CPU_SECONDS)
     return {"value": prefill_flops(B, T, H, D, W) / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
-            "kind": "port", "sample": sample, "seconds": dt}
+            "kind": "port", "sample": f"{sample}; {runs} passes in {dt * runs:.1f} s", "seconds": dt}
 
 
 # HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
@@ -223,7 +240,7 @@ def bench_decode_c4(steps=256, warmup=16, cpu_baseline=True):
     out = {"workload": "decode_c4_B64_H16_D128_W4096_256steps", "variants": results, **best}
     if cpu_baseline:
         out["cpu_baseline"] = cpu_decode_baseline(kc[:4].cpu(), vc[:4].cpu(), qs[0, :4].cpu(), ks[0, :4].cpu(), vs[0, :4].cpu(), W,
-                                                  f"4 of {B} batch elements, all {H} heads, 4 steps")
+                                                  f"4 of {B} batch elements, all {H} heads")
     return out
 
 
@@ -232,13 +249,13 @@ def cpu_decode_baseline(kc, vc, q, kn, vn, W, sample):
     torch.set_num_threads(os.cpu_count() or 1)
     B, H, _, D = kc.shape
     k_ctx, v_ctx = kc.transpose(1, 2), vc.transpose(1, 2)   # [B, n, H, D] views, n = W
-    reps = 4
-    t0 = time.perf_counter()
-    for _ in range(reps):
+    def one_step():
         k_ = torch.cat([k_ctx[:, 1:], kn[:, None]], 1).transpose(1, 2)
         v_ = torch.cat([v_ctx[:, 1:], vn[:, None]], 1).transpose(1, 2)
         torch.nn.functional.scaled_dot_product_attention(q[:, :, None], k_, v_, scale=SCALE, is_causal=False)
-    dt = (time.perf_counter() - t0) / reps
+
+    dt, runs = _repeat_for(one_step, CPU_SECONDS / 2)
+    sample = f"{sample}; {runs} steps in {dt * runs:.1f} s"
     return {"value": B * H * W * D * 4 / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
             "kind": "port", "sample": sample, "seconds_per_step": dt}
 
@@ -274,13 +291,12 @@ def bench_kda_c5(steps, warmup, cpu_baseline=True):
     if cpu_baseline:
         import oracle
         torch.set_num_threads(os.cpu_count() or 1)
-        Ts = 512
-        t0 = time.perf_counter()
-        oracle.kda_recurrent(q[:1, :Ts, :2].cpu(), k[:1, :Ts, :2].cpu(), v[:1, :Ts, :2].cpu(), gl[:1, :Ts, :2].cpu(), beta[:1, :Ts, :2].cpu())
-        dt = time.perf_counter() - t0
+        Ts = 2048
+        qc, kc, vc, gc, bc = (t[:1, :Ts, :2].cpu() for t in (q, k, v, gl, beta))
+        dt, runs = _repeat_for(lambda: oracle.kda_recurrent(qc, kc, vc, gc, bc), CPU_SECONDS / 2)
         tok_heads = Ts * 2
         out["cpu_baseline"] = {"value": tok_heads / dt, "unit": "token-heads/s", "cores": torch.get_num_threads(), "kind": "port",
-                               "sample": f"B=1, H=2 of 16, T={Ts} of {T} (naive recurrence)", "seconds": dt,
+                               "sample": f"B=1, H=2 of 16, T={Ts} of {T} (naive recurrence); {runs} passes in {dt * runs:.1f} s", "seconds": dt,
                                "gpu_token_heads_per_s": B * T * H / (ms / 1e3)}
     return out
 

@@ -79,10 +79,16 @@ def penalise_repeats(logits: Tensor, recent: Tensor, strength: Tensor, _one: Opt
                      half_life: float = 140.0, cap: float = 3.0) -> Tensor:
     """A token seen ``d`` positions ago (1 = the last one) counts ``0.5 ** (d / half_life)``; counts
     add up per token and saturate at ``cap``; the token's logit is divided by ``strength ** count``
-    when positive and multiplied by it otherwise.  ``_one`` is unused (kept for the call shape)."""
-    age = torch.arange(recent.numel(), 0, -1, device=logits.device, dtype=logits.dtype)
-    count = torch.zeros_like(logits).index_add_(0, recent, torch.pow(0.5, age / half_life)).clamp_(max=cap)
-    scale = torch.pow(strength, count)
+    when positive and multiplied by it otherwise.  ``_one`` is unused (kept for the call shape).
+    Works on one row (``logits [V]``, ``recent [n]``) or on a batch (``[B, V]``, ``[B, n]``)."""
+    n = recent.size(-1)
+    age = torch.arange(n, 0, -1, device=logits.device, dtype=logits.dtype)
+    weight = torch.pow(0.5, age / half_life)
+    if logits.dim() == 1:
+        count = torch.zeros_like(logits).index_add_(0, recent, weight)
+    else:                                   # a batch: logits [B, V], recent [B, n]
+        count = torch.zeros_like(logits).scatter_add_(1, recent, weight.expand_as(recent))
+    scale = torch.pow(strength, count.clamp_(max=cap))
     return logits * torch.where(logits > 0, scale.reciprocal(), scale)
 
 
@@ -229,3 +235,41 @@ class Generator:
         self._sync()
         t_end = time.perf_counter()
         return self.history.detach().clone(), t_prompt - t_start, t_end - t_prompt
+
+    @torch.inference_mode()
+    def generate_batch(self, prompt_ids: Tensor, max_new_tokens: int) -> Tensor:
+        """A batch of equally long prompts ``[B, T]`` -> ``[B, max_new_tokens]`` ids, with the same
+        sampling settings as ``generate``.  A row that produces the end-of-sequence token keeps
+        emitting it.  The reference's generator is built for one sequence (generate.py:76); this
+        path drives the model through ``daisy_amd.core`` (descriptor mask, keys and values of
+        every layer written straight into a bf16 ring of batch B, in-place decode steps), so the
+        model needs the attributes of the reference's ``DaisyCore`` and this package's attention.
+        """
+        from . import core
+        assert prompt_ids.ndim == 2 and prompt_ids.size(1) > 0 and max_new_tokens > 0
+        ids = prompt_ids.to(self.device)
+        B = ids.size(0)
+        cache = self._batch_caches.get(B) if hasattr(self, "_batch_caches") else None
+        if cache is None:
+            cache = KVCache(L=self.cache.L, B=B, H=self.cache.H, W=self.cache.W, D=self.cache.D,
+                            device=self.device, dtype=torch.bfloat16)
+            self._batch_caches = {**getattr(self, "_batch_caches", {}), B: cache}
+        cache.reset_history()
+        self.model.reset_history() if hasattr(self.model, "reset_history") else None
+        logits, _ = core.prefill(self.model, ids, cache)
+        seen = torch.empty(B, ids.size(1) + max_new_tokens, dtype=torch.long, device=self.device)
+        seen[:, :ids.size(1)] = ids
+        n_seen = ids.size(1)
+        eos = self.eos_token_id.to(torch.long)
+        done = torch.zeros(B, dtype=torch.bool, device=self.device)
+        for produced in range(1, max_new_tokens + 1):
+            scores = self._trim(logits)
+            scores = self.apply_repetition_penalty(scores, seen[:, max(n_seen - _PENALTY_LOOKBACK, 0):n_seen], self.rep_p_t, self._one)
+            token = self.sample(scores, self.temperature, self.top_k, self.top_p)
+            token = torch.where(done, eos, token)
+            done |= token == eos
+            seen[:, n_seen] = token
+            n_seen += 1
+            if produced < max_new_tokens:
+                logits = core.step(self.model, token, cache)
+        return seen[:, ids.size(1):n_seen].clone()

@@ -245,8 +245,9 @@ class CausalSelfAttention(nn.Module):
         # The one-pass norm + RoPE + ve-mix kernel works on bf16 rows of 64 or 128 channels.
         return self.fused_prep and self.qkvo_w.dtype == torch.bfloat16 and self.head_dim in (64, 128)
 
-    def _project_qkv_fused(self, x: Tensor, ve: Optional[Tensor], pos0: int):
-        """QKV projection, then norm + RoPE (rows ``pos0 + t``) + ve mix in one kernel; ``[B, T, H, D]``."""
+    def _project_qkv_fused(self, x: Tensor, ve: Optional[Tensor], pos0: int, k_out=None, v_out=None):
+        """QKV projection, then norm + RoPE (rows ``pos0 + t``) + ve mix in one kernel; ``[B, T, H, D]``.
+        ``k_out`` / ``v_out``: strided ``[B, T, H, D]`` views that receive k and v (e.g. slots of a ring cache)."""
         B, T = x.size(0), x.size(1)
         x = x.to(self.qkvo_w.dtype)
         qkv = F.linear(x, self.qkvo_w[:3].flatten(end_dim=1)).view(B, T, 3 * self.num_heads, self.head_dim)
@@ -259,13 +260,17 @@ class CausalSelfAttention(nn.Module):
         else:
             ve = None
         cos, sin = self.rotary._get_cos_sin(pos0 + T)
-        return ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, pos0=pos0, ve=ve, gate=gate)
+        return ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, pos0=pos0, ve=ve, gate=gate,
+                            k_out=k_out, v_out=v_out)
 
     def _attend(self, x: Tensor, ve: Optional[Tensor], attn_mask: MaskLike):
         B, T = x.size(0), x.size(1)
         mask = _as_window_mask(attn_mask)
+        # One-shot destination for k and v set by the caller of the enclosing block (the model glue
+        # points it at the ring cache's slots so that no copy into the cache follows).
+        dest = self.__dict__.pop("_kv_destination", None)
         if self._fused_prep_ok():
-            q, k_rot, v = self._project_qkv_fused(x, ve, 0)
+            q, k_rot, v = self._project_qkv_fused(x, ve, 0, *(dest or (None, None)))
             o, _ = ops.prefill_attention(q, k_rot, v, window=mask.window, scale=self.attn_scale, doc_start=mask.doc_start)
             y = F.linear(o.view(B, T, self.m_dim), self.qkvo_w[3])
             return y, k_rot, v

@@ -9,7 +9,8 @@ model attributes (``embed``, ``blocks``, ``skip_map``, ``skip_weights``, ``ve_mo
 
 * pass the window / document mask as a descriptor (no T x T tensor, no T <= 46340 cap),
 * write each layer's keys and values straight into the ring cache as the layer finishes
-  (nothing of size ``L * T`` is ever stacked), and
+  (nothing of size ``L * T`` is ever stacked; a prompt shorter than the ring is written into its
+  slots by the pre-attention kernel itself, with no copy at all), and
 * accept a batch of sequences (the cache has a batch dimension; the reference pins B = 1).
 
 They work on the reference's ``DaisyCore`` once its blocks hold this package's
@@ -23,7 +24,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor
 
-from .attention import WindowMask, build_window_mask
+from .attention import CausalSelfAttention, WindowMask, build_window_mask
 from .functional import norm
 from .kv_cache import KVCache
 
@@ -68,10 +69,22 @@ def prefill(model, input_seq: Tensor, cache: Optional[KVCache] = None, debug: bo
         if i in skip_map:
             gate = torch.sigmoid(skip_weights[skip_map[i]])
             x = x * gate + (1 - gate) * skip_connections[skip_map[i]]
-        x, k, v = model.blocks[i].prefill(x, ve_map.get(i), x0, attn_mask=attn_mask, debug=debug)
+        # A prompt that fits the ring without wrapping (T <= W - 1: position p goes to slot p) is
+        # written there by the pre-attention kernel itself; the attention kernel then reads its keys
+        # and values from the ring and nothing is copied afterwards.
+        attn = getattr(model.blocks[i], "attn", None)
+        direct = (cache is not None and cache.dtype == torch.bfloat16 and T <= cache.W - 1
+                  and isinstance(attn, CausalSelfAttention) and attn._fused_prep_ok())
+        if direct:
+            attn._kv_destination = (cache.k[i][:, :, :T].transpose(1, 2), cache.v[i][:, :, :T].transpose(1, 2))
+        try:
+            x, k, v = model.blocks[i].prefill(x, ve_map.get(i), x0, attn_mask=attn_mask, debug=debug)
+        finally:
+            if direct:
+                attn.__dict__.pop("_kv_destination", None)
         skip_connections.append(x)
         if cache is not None:
-            if k is not None:
+            if k is not None and not direct:
                 cache.bulk_write_layer(i, k, v, T)
         else:
             k_list.append(k)

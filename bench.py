@@ -382,12 +382,20 @@ def bench_next_rows(steps, warmup):
 
         ms_ring = time_gpu(step_ring, 64, 8)
         ms_views = time_gpu(step_views, 64, 8)
+        recorded = core.GraphedStep(model, cache)
+
+        def step_recorded():     # the same walk replayed as one HIP graph, position in device memory
+            cache.t = t_before
+            return recorded(tok)
+
+        ms_recorded = time_gpu(step_recorded, 64, 8)
     out["model_glue_L4_B16_T4100_W4096"] = {
         "prefill_ms_ring_written_per_layer": ms_direct, "prefill_ms_stack_then_bulk_write": ms_stacked,
         "prefill_ms_T2048_written_in_place": ms_direct_fit, "prefill_ms_T2048_stack_then_bulk_write": ms_stacked_fit,
-        "step_ms_ring_in_place": ms_ring, "step_ms_chronological_views": ms_views,
+        "step_ms_ring_in_place": ms_ring, "step_ms_ring_in_place_recorded_graph": ms_recorded,
+        "step_ms_chronological_views": ms_views,
         "kv_bytes_per_step": 2 * L * Bs * 8 * min(t_before + 1, W) * 128 * 2}
-    del model, cache
+    del model, cache, recorded
 
     # ---- training-time block masks as per-row lower bounds: one sequence of 32768, 3 documents ----
     with torch.no_grad():

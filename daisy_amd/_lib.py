@@ -41,6 +41,14 @@ SIGNATURES = {
         c_int, c_int, c_int,                                    # n_rows, new_idx, write_back
         c_float, c_int,                                         # scale, nsplit
         c_void_p, c_size_t, c_void_p]),                         # workspace, bytes, stream
+    "daisy_decode_fwd_at": (c_int, [
+        c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k_new, v_new (+strides)
+        c_void_p, _I64P, c_void_p, _I64P,                       # k_cache, v_cache (+strides)
+        c_void_p, _I64P,                                        # o (+strides)
+        c_int, c_int, c_int,                                    # B, H, D
+        c_int, c_void_p,                                        # ring_rows, pos (device int32)
+        c_float, c_int,                                         # scale, nsplit
+        c_void_p, c_size_t, c_void_p]),                         # workspace, bytes, stream
     "daisy_kda_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "daisy_kda_chunk_fwd": (c_int, [
         c_void_p, c_void_p, c_void_p,                           # q, k, v
@@ -71,6 +79,12 @@ SIGNATURES = {
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q, k, v (+ strides)
         c_void_p, _I64P, c_void_p,                               # ve, ve strides, gate
         c_void_p, c_void_p, c_int,                              # cos, sin, pos0
+        c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q_out, k_out, v_out (+ strides)
+        c_int, c_int, c_int, c_int, c_float, c_void_p]),        # B, T, H, D, eps, stream
+    "daisy_qkv_prep_fwd_at": (c_int, [
+        c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q, k, v (+ strides)
+        c_void_p, _I64P, c_void_p,                               # ve, ve strides, gate
+        c_void_p, c_void_p, c_void_p, c_int,                    # cos, sin, pos0 (device int32), table_rows
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q_out, k_out, v_out (+ strides)
         c_int, c_int, c_int, c_int, c_float, c_void_p]),        # B, T, H, D, eps, stream
 }

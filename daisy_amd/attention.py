@@ -259,7 +259,10 @@ class CausalSelfAttention(nn.Module):
             gate = torch.sigmoid(self.g_ve.detach()).to(torch.bfloat16).float().reshape(1)
         else:
             ve = None
-        cos, sin = self.rotary._get_cos_sin(pos0 + T)
+        if isinstance(pos0, Tensor):
+            cos, sin = self.rotary.cos, self.rotary.sin   # position known on the device only: whole tables
+        else:
+            cos, sin = self.rotary._get_cos_sin(pos0 + T)
         return ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, pos0=pos0, ve=ve, gate=gate,
                             k_out=k_out, v_out=v_out)
 
@@ -304,7 +307,7 @@ class CausalSelfAttention(nn.Module):
             self.last_k = k
         return y, k.transpose(1, 2), v.transpose(1, 2)
 
-    def step(self, x, k_ctx: Union[Tensor, RingContext], v_ctx: Union[Tensor, RingContext], pos: int,
+    def step(self, x, k_ctx: Union[Tensor, RingContext], v_ctx: Union[Tensor, RingContext], pos: Union[int, Tensor],
              ve: Optional[Tensor], window: Optional[int]):
         """One token: returns ``y [B, 1, dim]``, ``k [B, 1, H, D]``, ``v [B, 1, H, D]``.
 
@@ -312,10 +315,16 @@ class CausalSelfAttention(nn.Module):
         ``[B, n, H, D]`` (the reference's calling convention) or the
         ``RingContext`` of a ``KVCache`` layer, in which case the kernel streams
         the ring in place and appends the new row itself.
+
+        ``pos`` may be a one-element int32 device tensor (with a ``RingContext`` only): nothing on
+        the host then depends on the position, so the step can be recorded in a HIP graph and
+        replayed while the tensor counts up.
         """
         B = x.size(0)
         torch._assert(x.size(1) == 1, "step() requires single position only")
         fused = self._fused_prep_ok()
+        if isinstance(pos, Tensor):
+            return self._step_at(x, k_ctx, pos, ve, window, fused)
         if fused:
             # q and k come back rotated: the decode kernel is told not to rotate again.
             q, k, v = self._project_qkv_fused(x, ve, pos)
@@ -362,3 +371,15 @@ class CausalSelfAttention(nn.Module):
         y = o.reshape(B, 1, self.m_dim).to(dtype)
         y = F.linear(y, self.qkvo_w[3])
         return y, k_new, v_new
+
+    def _step_at(self, x, ring, pos: Tensor, ve: Optional[Tensor], window: Optional[int], fused: bool):
+        """``step`` at a position that only the device knows (see there)."""
+        if not (fused and isinstance(ring, RingContext) and ring.k.dtype == torch.bfloat16 and window == ring.W):
+            raise ValueError("a device-side position needs the fused pre-attention kernel (bf16 weights, head dim 64 "
+                             "or 128) and the RingContext of a bf16 KVCache whose size equals the window")
+        B = x.size(0)
+        q, k, v = self._project_qkv_fused(x, ve, pos)
+        o = ops.decode_attention_at(q[:, 0], k[:, 0], v[:, 0], ring.k, ring.v, pos, scale=self.attn_scale)
+        ring.mark_written()
+        y = F.linear(o.reshape(B, 1, self.m_dim), self.qkvo_w[3])
+        return y, k, v   # the rows as the kernel stored them in slot pos % W

@@ -117,10 +117,18 @@ def step(model, token_ids: Tensor, cache: KVCache) -> Tensor:
     this package's attention), or gets the chronological view and the row is written here.
     Advances the cache; returns ``logits [B, V]``.
     """
+    logits = _walk_step(model, token_ids, cache, cache.t)
+    cache.advance()
+    return logits
+
+
+def _walk_step(model, token_ids: Tensor, cache: KVCache, pos) -> Tensor:
+    """The layer walk of ``step`` at position ``pos`` (a host int, or a one-element int32 device
+    tensor when the walk is being recorded for replay); leaves ``cache.advance()`` to the caller."""
     token_ids = token_ids.reshape(-1, 1)
     B = token_ids.size(0)
     torch._assert(B == cache.B, "token batch does not match the cache")
-    pos = cache.t
+    on_device = isinstance(pos, Tensor)
     L = len(model.blocks)
     x = x0 = norm(model.embed(token_ids))
     skip_map, skip_weights = model.skip_map, model.skip_weights
@@ -138,14 +146,80 @@ def step(model, token_ids: Tensor, cache: KVCache) -> Tensor:
         elif in_place and getattr(blk.attn, "accepts_ring_context", False):
             k_ctx = v_ctx = cache.ring(i)
         else:
+            torch._assert(not on_device, "a recorded step needs attention layers that take the ring in place")
             k_ctx, v_ctx = cache.view(i)
         x, k_new, v_new = blk.step(x, ve_map.get(i), x0, k_ctx, v_ctx, pos, window)
         skip_connections.append(x)
         if k_new is not None and not cache._staged[i]:
+            torch._assert(not on_device, "a recorded step needs attention layers that write the ring themselves")
             cache.write(i, k_new.to(cache.dtype), v_new.to(cache.dtype))
-    cache.advance()
     x = norm(x)
     return F.linear(x.flatten(end_dim=1).bfloat16(), model.lm_head_w.bfloat16()).float()
+
+
+class GraphedStep:
+    """``step(model, tokens, cache)`` recorded once as a HIP graph and replayed for every later token.
+
+    A decode step of a small model is a few hundred short kernels, and launching them one by one
+    from Python costs more than running them.  Nothing in the recorded walk depends on the host's
+    idea of the position: the token ids sit in a fixed input buffer, and the position sits in a
+    device counter that the pre-attention and decode kernels read when they run and that the last
+    node of the graph increments.
+
+    Needs a bf16 cache whose ring size equals the model's attention window and attention layers
+    that take the ring in place with the fused pre-attention kernel (otherwise recording raises).
+    The returned logits are a buffer that the next call overwrites.  Rotary tables are fixed when
+    the step is recorded: positions up to their row count can be replayed.
+    """
+
+    def __init__(self, model, cache: KVCache):
+        torch._assert(cache.dtype == torch.bfloat16, "a recorded step needs a bf16 cache")
+        self.model, self.cache = model, cache
+        dev = cache.k.device
+        self.tokens = torch.zeros(cache.B, dtype=torch.long, device=dev)
+        self.pos = torch.zeros(1, dtype=torch.int32, device=dev)
+        self._pos_host: Optional[int] = None      # what self.pos holds, None = unknown
+        self._graph: Optional[torch.cuda.CUDAGraph] = None
+        self._logits: Optional[Tensor] = None
+        tables = [blk.attn.rotary.cos.shape[0] for blk in model.blocks
+                  if getattr(blk, "attn", None) is not None and hasattr(blk.attn, "rotary")]
+        self.max_positions = min(tables) if tables else None
+
+    def _body(self) -> Tensor:
+        logits = _walk_step(self.model, self.tokens, self.cache, self.pos)
+        self.pos.add_(1)
+        return logits
+
+    @torch.no_grad()
+    def _record(self):
+        dev = self.cache.k.device
+        # One eager pass on a side stream first (library handles, workspaces, the allocator's pools);
+        # it writes the same row the first replay writes again.
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            self._body()
+        torch.cuda.current_stream(dev).wait_stream(side)
+        self.pos.fill_(self.cache.t)
+        self._graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self._graph):
+            self._logits = self._body()
+        self.cache._staged = [False] * self.cache.L    # recording ran no kernel
+
+    @torch.no_grad()
+    def __call__(self, token_ids: Tensor) -> Tensor:
+        cache = self.cache
+        if self.max_positions is not None:
+            torch._assert(cache.t < self.max_positions, f"Rotary buffers too small {self.max_positions} < {cache.t + 1}")
+        self.tokens.copy_(token_ids.reshape(-1))
+        if self._pos_host != cache.t:
+            self.pos.fill_(cache.t)
+        if self._graph is None:
+            self._record()
+        self._graph.replay()
+        cache.advance()
+        self._pos_host = cache.t
+        return self._logits
 
 
 @torch.no_grad()

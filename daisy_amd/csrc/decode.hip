@@ -25,7 +25,24 @@ struct DecodeParams {
   float* partials;  // [B, H, nsplit, D + 2] when nsplit > 1
   int B, H, n_rows, new_idx, write_back, nsplit, rows_per_split;
   float scale_log2e;
+  // When set, the step's position t is read from device memory at run time (so that a recorded
+  // launch can be replayed for later positions): the cache is a ring of ring_rows slots,
+  // n_rows = min(t + 1, ring_rows) of them are live and the new row goes to slot t % ring_rows.
+  const int32_t* pos_dev; int ring_rows;
 };
+
+struct DecodeRange { int n_rows, new_idx, rows_per_split; };
+
+__device__ __forceinline__ DecodeRange decode_range(const DecodeParams& p) {
+  DecodeRange r{p.n_rows, p.new_idx, p.rows_per_split};
+  if (p.pos_dev != nullptr) {
+    const int t = max(p.pos_dev[0], 0);
+    r.n_rows = min(t + 1, p.ring_rows);
+    r.new_idx = t % p.ring_rows;
+    r.rows_per_split = (r.n_rows + p.nsplit - 1) / p.nsplit;
+  }
+  return r;
+}
 
 constexpr int kDecodeThreads = 256;
 constexpr int kDecodeWaves = kDecodeThreads / 64;
@@ -92,8 +109,10 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
 #pragma unroll
   for (int i = 0; i < 8; ++i) qf[i] *= p.scale_log2e;
 
-  const int r0 = split * p.rows_per_split;
-  const int r1 = min(r0 + p.rows_per_split, p.n_rows);
+  const DecodeRange rg = decode_range(p);
+  const int new_idx = rg.new_idx;
+  const int r0 = split * rg.rows_per_split;
+  const int r1 = min(r0 + rg.rows_per_split, rg.n_rows);
   uint16_t* kbase = p.kc + b * p.kc_sb + h * p.kc_sh + dl;
   uint16_t* vbase = p.vc + b * p.vc_sb + h * p.vc_sh + dl;
 
@@ -105,7 +124,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
 
   // Lanes whose row is past the range, or is the new token's slot, load a row
   // that is always readable instead (and are masked / overwritten below).
-  const int safe_row = (r0 != p.new_idx) ? r0 : r0 + 1;
+  const int safe_row = (r0 != new_idx) ? r0 : r0 + 1;
   const uint16_t* k_safe = (safe_row < r1) ? kbase + (int64_t)safe_row * p.kc_sr : p.k_new + b * p.kn_sb + h * p.kn_sh + dl;
   const uint16_t* v_safe = (safe_row < r1) ? vbase + (int64_t)safe_row * p.vc_sr : p.v_new + b * p.vn_sb + h * p.vn_sh + dl;
 
@@ -114,13 +133,13 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int row = base + u * RPW + sub;
-      const uint16_t* a = (row < r1 && row != p.new_idx) ? kbase + (int64_t)row * p.kc_sr : k_safe;
+      const uint16_t* a = (row < r1 && row != new_idx) ? kbase + (int64_t)row * p.kc_sr : k_safe;
       kr[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a));
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int row = base + u * RPW + sub;
-      const uint16_t* a = (row < r1 && row != p.new_idx) ? vbase + (int64_t)row * p.vc_sr : v_safe;
+      const uint16_t* a = (row < r1 && row != new_idx) ? vbase + (int64_t)row * p.vc_sr : v_safe;
       vr[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a));
     }
 
@@ -129,7 +148,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int row = base + u * RPW + sub;
-      if (row == p.new_idx && row < r1) {
+      if (row == new_idx && row < r1) {
         kr[u] = kn_packed;
         vr[u] = vn_packed;
         if (p.write_back) {
@@ -260,6 +279,7 @@ static int resolve_nsplit(int B, int H, int n_rows, int nsplit) {
 __global__ __launch_bounds__(64) void decode_scalar_kernel(DecodeParams p, int D) {
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const int half = D / 2;
+  const DecodeRange rg = decode_range(p);
   const uint16_t* qp = p.q + b * p.q_sb + h * p.q_sh;
   const uint16_t* knp = p.k_new + b * p.kn_sb + h * p.kn_sh;
   const uint16_t* vnp = p.v_new + b * p.vn_sb + h * p.vn_sh;
@@ -286,8 +306,8 @@ __global__ __launch_bounds__(64) void decode_scalar_kernel(DecodeParams p, int D
     }
   }
   float m = -INFINITY, l = 0.f;
-  for (int r = 0; r < p.n_rows; ++r) {
-    const bool is_new = r == p.new_idx;
+  for (int r = 0; r < rg.n_rows; ++r) {
+    const bool is_new = r == rg.new_idx;
     float kr[4], vr[4], part = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -316,8 +336,8 @@ __global__ __launch_bounds__(64) void decode_scalar_kernel(DecodeParams p, int D
     if (d < D) {
       op[d] = (uint16_t)(pack_bf16x2(acc[i] / l, 0.f) & 0xffffu);
       if (p.write_back) {
-        kc[(int64_t)p.new_idx * p.kc_sr + d] = (uint16_t)(pack_bf16x2(kn[i], 0.f) & 0xffffu);
-        vc[(int64_t)p.new_idx * p.vc_sr + d] = (uint16_t)(pack_bf16x2(vn[i], 0.f) & 0xffffu);
+        kc[(int64_t)rg.new_idx * p.kc_sr + d] = (uint16_t)(pack_bf16x2(kn[i], 0.f) & 0xffffu);
+        vc[(int64_t)rg.new_idx * p.vc_sr + d] = (uint16_t)(pack_bf16x2(vn[i], 0.f) & 0xffffu);
       }
     }
   }
@@ -335,17 +355,19 @@ extern "C" size_t daisy_decode_workspace_bytes(int B, int H, int D, int n_rows, 
   return (size_t)B * H * ns * (D + 2) * sizeof(float);
 }
 
-extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
-                                const void* k_new, const int64_t* k_new_strides,
-                                const void* v_new, const int64_t* v_new_strides,
-                                void* k_cache, const int64_t* k_cache_strides,
-                                void* v_cache, const int64_t* v_cache_strides,
-                                const float* cos_row, const float* sin_row,
-                                void* o, const int64_t* o_strides,
-                                int B, int H, int D,
-                                int n_rows, int new_idx, int write_back,
-                                float scale, int nsplit,
-                                void* workspace, size_t workspace_bytes, void* stream) {
+// Shared by the two entry points.  With pos_dev set, n_rows is the ring's slot count (it fixes the
+// split count and the grid) and the kernel derives the live rows and the new row's slot from *pos_dev.
+static int decode_launch(const void* q, const int64_t* q_strides,
+                         const void* k_new, const int64_t* k_new_strides,
+                         const void* v_new, const int64_t* v_new_strides,
+                         void* k_cache, const int64_t* k_cache_strides,
+                         void* v_cache, const int64_t* v_cache_strides,
+                         const float* cos_row, const float* sin_row,
+                         void* o, const int64_t* o_strides,
+                         int B, int H, int D,
+                         int n_rows, int new_idx, const int32_t* pos_dev, int write_back,
+                         float scale, int nsplit,
+                         void* workspace, size_t workspace_bytes, void* stream) {
   DAISY_CHECK_ARG(q && k_new && v_new && o, "decode: q, k_new, v_new and o must be non-NULL");
   DAISY_CHECK_ARG(q_strides && k_new_strides && v_new_strides && o_strides, "decode: stride arrays must be non-NULL");
   DAISY_CHECK_ARG(B > 0 && H > 0, "decode: B=%d and H=%d must be positive", B, H);
@@ -390,6 +412,7 @@ extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
   p.B = B; p.H = H; p.n_rows = n_rows; p.new_idx = new_idx; p.write_back = write_back;
   p.nsplit = fast ? resolve_nsplit(B, H, n_rows, nsplit) : 1;
   p.rows_per_split = (n_rows + p.nsplit - 1) / p.nsplit;
+  p.pos_dev = pos_dev; p.ring_rows = n_rows;
   p.scale_log2e = scale * kLog2e;
   p.partials = nullptr;
   if (p.nsplit > 1) {
@@ -424,4 +447,39 @@ extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
     }
   }
   return DAISY_OK;
+}
+
+extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
+                                const void* k_new, const int64_t* k_new_strides,
+                                const void* v_new, const int64_t* v_new_strides,
+                                void* k_cache, const int64_t* k_cache_strides,
+                                void* v_cache, const int64_t* v_cache_strides,
+                                const float* cos_row, const float* sin_row,
+                                void* o, const int64_t* o_strides,
+                                int B, int H, int D,
+                                int n_rows, int new_idx, int write_back,
+                                float scale, int nsplit,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  return decode_launch(q, q_strides, k_new, k_new_strides, v_new, v_new_strides, k_cache, k_cache_strides,
+                       v_cache, v_cache_strides, cos_row, sin_row, o, o_strides, B, H, D, n_rows, new_idx, nullptr,
+                       write_back, scale, nsplit, workspace, workspace_bytes, stream);
+}
+
+extern "C" int daisy_decode_fwd_at(const void* q, const int64_t* q_strides,
+                                   const void* k_new, const int64_t* k_new_strides,
+                                   const void* v_new, const int64_t* v_new_strides,
+                                   void* k_cache, const int64_t* k_cache_strides,
+                                   void* v_cache, const int64_t* v_cache_strides,
+                                   void* o, const int64_t* o_strides,
+                                   int B, int H, int D,
+                                   int ring_rows, const int32_t* pos,
+                                   float scale, int nsplit,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+  DAISY_CHECK_ARG(pos != nullptr, "decode_at: the device position pointer must be non-NULL");
+  DAISY_CHECK_ARG(k_cache && v_cache && k_cache_strides && v_cache_strides, "decode_at: the ring cache is required");
+  DAISY_CHECK_ARG(ring_rows >= 1, "decode_at: ring_rows=%d must be >= 1", ring_rows);
+  DAISY_CHECK_SUPPORTED(D == 64 || D == 128, "decode_at: head_dim %d not supported (64 or 128)", D);
+  return decode_launch(q, q_strides, k_new, k_new_strides, v_new, v_new_strides, k_cache, k_cache_strides,
+                       v_cache, v_cache_strides, nullptr, nullptr, o, o_strides, B, H, D, ring_rows, 0, pos,
+                       /*write_back=*/1, scale, nsplit, workspace, workspace_bytes, stream);
 }

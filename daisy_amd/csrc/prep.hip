@@ -24,6 +24,9 @@ struct PrepParams {
   uint16_t* ko; int64_t ko_sb, ko_st, ko_sh;
   uint16_t* vo; int64_t vo_sb, vo_st, vo_sh;
   int B, T, H, pos0;
+  // When set, the first position is read from device memory at run time (so that a recorded
+  // launch can be replayed for later positions) and held inside the table's rows.
+  const int32_t* pos0_dev; int table_rows;
   int64_t rows;
   float eps;
 };
@@ -79,7 +82,9 @@ __global__ __launch_bounds__(256) void qkv_prep_kernel(PrepParams p) {
   if (p.ve != nullptr) load_row(p.ve, p.e_sb, p.e_st, p.e_sh, el, eh);
   float cs[8], sn[8];
   if (p.cos != nullptr) {
-    const int64_t off = (int64_t)(p.pos0 + t) * HALF + 8 * c;
+    int pos0 = p.pos0;
+    if (p.pos0_dev != nullptr) pos0 = max(0, min(p.pos0_dev[0], p.table_rows - p.T));
+    const int64_t off = (int64_t)(pos0 + t) * HALF + 8 * c;
     const f32x4 c0 = *reinterpret_cast<const f32x4*>(p.cos + off), c1 = *reinterpret_cast<const f32x4*>(p.cos + off + 4);
     const f32x4 s0 = *reinterpret_cast<const f32x4*>(p.sin + off), s1 = *reinterpret_cast<const f32x4*>(p.sin + off + 4);
 #pragma unroll
@@ -122,15 +127,15 @@ __global__ __launch_bounds__(256) void qkv_prep_kernel(PrepParams p) {
 
 using namespace daisy;
 
-extern "C" int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
-                                  const void* k, const int64_t* k_strides,
-                                  const void* v, const int64_t* v_strides,
-                                  const void* ve, const int64_t* ve_strides, const float* gate,
-                                  const float* cos, const float* sin, int pos0,
-                                  void* q_out, const int64_t* q_out_strides,
-                                  void* k_out, const int64_t* k_out_strides,
-                                  void* v_out, const int64_t* v_out_strides,
-                                  int B, int T, int H, int D, float eps, void* stream) {
+static int prep_launch(const void* q, const int64_t* q_strides,
+                       const void* k, const int64_t* k_strides,
+                       const void* v, const int64_t* v_strides,
+                       const void* ve, const int64_t* ve_strides, const float* gate,
+                       const float* cos, const float* sin, int pos0, const int32_t* pos0_dev, int table_rows,
+                       void* q_out, const int64_t* q_out_strides,
+                       void* k_out, const int64_t* k_out_strides,
+                       void* v_out, const int64_t* v_out_strides,
+                       int B, int T, int H, int D, float eps, void* stream) {
   DAISY_CHECK_ARG(q && k && v && q_out && k_out && v_out, "qkv_prep: q, k, v and the three outputs must be non-NULL");
   DAISY_CHECK_ARG(q_strides && k_strides && v_strides && q_out_strides && k_out_strides && v_out_strides,
                   "qkv_prep: stride arrays must be non-NULL");
@@ -161,6 +166,7 @@ extern "C" int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
   p.ko = (uint16_t*)k_out; p.ko_sb = k_out_strides[0]; p.ko_st = k_out_strides[1]; p.ko_sh = k_out_strides[2];
   p.vo = (uint16_t*)v_out; p.vo_sb = v_out_strides[0]; p.vo_st = v_out_strides[1]; p.vo_sh = v_out_strides[2];
   p.B = B; p.T = T; p.H = H; p.pos0 = pos0; p.eps = eps;
+  p.pos0_dev = pos0_dev; p.table_rows = table_rows;
   p.rows = (int64_t)B * T * H;
   const int lpr = D / 16;
   const int64_t nwg = (p.rows * lpr + 255) / 256;
@@ -170,4 +176,33 @@ extern "C" int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
   else hipLaunchKernelGGL(qkv_prep_kernel<64>, dim3((unsigned)nwg), dim3(256), 0, s, p);
   DAISY_CHECK_LAUNCH("qkv_prep_kernel");
   return DAISY_OK;
+}
+
+extern "C" int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
+                                  const void* k, const int64_t* k_strides,
+                                  const void* v, const int64_t* v_strides,
+                                  const void* ve, const int64_t* ve_strides, const float* gate,
+                                  const float* cos, const float* sin, int pos0,
+                                  void* q_out, const int64_t* q_out_strides,
+                                  void* k_out, const int64_t* k_out_strides,
+                                  void* v_out, const int64_t* v_out_strides,
+                                  int B, int T, int H, int D, float eps, void* stream) {
+  return prep_launch(q, q_strides, k, k_strides, v, v_strides, ve, ve_strides, gate, cos, sin, pos0, nullptr, 0,
+                     q_out, q_out_strides, k_out, k_out_strides, v_out, v_out_strides, B, T, H, D, eps, stream);
+}
+
+extern "C" int daisy_qkv_prep_fwd_at(const void* q, const int64_t* q_strides,
+                                     const void* k, const int64_t* k_strides,
+                                     const void* v, const int64_t* v_strides,
+                                     const void* ve, const int64_t* ve_strides, const float* gate,
+                                     const float* cos, const float* sin, const int32_t* pos0, int table_rows,
+                                     void* q_out, const int64_t* q_out_strides,
+                                     void* k_out, const int64_t* k_out_strides,
+                                     void* v_out, const int64_t* v_out_strides,
+                                     int B, int T, int H, int D, float eps, void* stream) {
+  DAISY_CHECK_ARG(pos0 != nullptr, "qkv_prep_at: the device position pointer must be non-NULL");
+  DAISY_CHECK_ARG(cos && sin, "qkv_prep_at: the rotary tables are required");
+  DAISY_CHECK_ARG(table_rows >= T, "qkv_prep_at: table_rows=%d must cover the %d rows of the call", table_rows, T);
+  return prep_launch(q, q_strides, k, k_strides, v, v_strides, ve, ve_strides, gate, cos, sin, 0, pos0, table_rows,
+                     q_out, q_out_strides, k_out, k_out_strides, v_out, v_out_strides, B, T, H, D, eps, stream);
 }

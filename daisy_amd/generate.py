@@ -237,13 +237,17 @@ class Generator:
         return self.history.detach().clone(), t_prompt - t_start, t_end - t_prompt
 
     @torch.inference_mode()
-    def generate_batch(self, prompt_ids: Tensor, max_new_tokens: int) -> Tensor:
+    def generate_batch(self, prompt_ids: Tensor, max_new_tokens: int, record_steps: bool = False) -> Tensor:
         """A batch of equally long prompts ``[B, T]`` -> ``[B, max_new_tokens]`` ids, with the same
         sampling settings as ``generate``.  A row that produces the end-of-sequence token keeps
         emitting it.  The reference's generator is built for one sequence (generate.py:76); this
         path drives the model through ``daisy_amd.core`` (descriptor mask, keys and values of
         every layer written straight into a bf16 ring of batch B, in-place decode steps), so the
         model needs the attributes of the reference's ``DaisyCore`` and this package's attention.
+
+        ``record_steps``: record the decode step once per batch size as a HIP graph
+        (``core.GraphedStep``) and replay it for every token instead of launching its kernels
+        one by one; the model's parameters must stay where they are between calls.
         """
         from . import core
         assert prompt_ids.ndim == 2 and prompt_ids.size(1) > 0 and max_new_tokens > 0
@@ -256,6 +260,13 @@ class Generator:
             self._batch_caches = {**getattr(self, "_batch_caches", {}), B: cache}
         cache.reset_history()
         self.model.reset_history() if hasattr(self.model, "reset_history") else None
+        step = lambda tokens: core.step(self.model, tokens, cache)
+        if record_steps:
+            recorded = getattr(self, "_recorded_steps", {})
+            if B not in recorded:
+                recorded[B] = core.GraphedStep(self.model, cache)
+                self._recorded_steps = recorded
+            step = recorded[B]
         logits, _ = core.prefill(self.model, ids, cache)
         seen = torch.empty(B, ids.size(1) + max_new_tokens, dtype=torch.long, device=self.device)
         seen[:, :ids.size(1)] = ids
@@ -271,5 +282,5 @@ class Generator:
             seen[:, n_seen] = token
             n_seen += 1
             if produced < max_new_tokens:
-                logits = core.step(self.model, token, cache)
+                logits = step(token)
         return seen[:, ids.size(1):n_seen].clone()

@@ -5,7 +5,7 @@ validate, allocate outputs and pass raw pointers to ``libdaisy_hip.so``.
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import Optional, Tuple, Union
 
 import torch
 
@@ -130,6 +130,54 @@ def decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
             float(scale), int(nsplit),
             _lib.ptr(workspace), ws_bytes, _lib.current_stream(dev))
     _lib.check(rc, "daisy_decode_fwd")
+    return out
+
+
+def decode_attention_at(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
+                        k_ring: torch.Tensor, v_ring: torch.Tensor, pos: torch.Tensor, *,
+                        scale: float = ATTN_SCALE, out: Optional[torch.Tensor] = None,
+                        workspace: Optional[torch.Tensor] = None, nsplit: int = 0) -> torch.Tensor:
+    """``decode_attention`` over a ring cache with the position in device memory.
+
+    ``k_ring``/``v_ring``: bf16 ``[B, H, W, D]`` (slot order); ``pos``: one-element int32 device tensor
+    holding ``t``, the number of positions already in the ring.  The kernel reads ``t`` when it
+    runs, attends the ``min(t + 1, W)`` live rows and writes the new row (``k_new``, ``v_new``, already
+    rotated) to slot ``t % W``; the launch can therefore be recorded in a HIP graph and replayed
+    while the caller increments ``pos``.  Returns ``o`` bf16 ``[B, H, D]``.
+    """
+    dev = _lib.require_gpu(q, k_new, v_new, k_ring, v_ring, pos, out, workspace)
+    for name, t in (("q", q), ("k_new", k_new), ("v_new", v_new)):
+        _check_bf16(name, t, 3)
+    _check_bf16("k_ring", k_ring, 4)
+    _check_bf16("v_ring", v_ring, 4)
+    B, H, D = q.shape
+    if k_new.shape != q.shape or v_new.shape != q.shape:
+        raise ValueError("q, k_new, v_new must all be [B, H, D]")
+    W = k_ring.shape[2]
+    if k_ring.shape != (B, H, W, D) or v_ring.shape != k_ring.shape:
+        raise ValueError(f"k_ring, v_ring must be [B, H, W, D] = [{B}, {H}, W, {D}], got {tuple(k_ring.shape)}, {tuple(v_ring.shape)}")
+    if pos.dtype != torch.int32 or pos.numel() != 1:
+        raise ValueError("pos must be a one-element int32 tensor")
+    if out is None:
+        out = torch.empty((B, H, D), dtype=torch.bfloat16, device=dev)
+    else:
+        _check_bf16("out", out, 3)
+    lib = _lib.load()
+    need = int(lib.daisy_decode_workspace_bytes(B, H, D, W, nsplit))
+    if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(dev):
+        rc = lib.daisy_decode_fwd_at(
+            q.data_ptr(), _lib.strides(q, (0, 1)),
+            k_new.data_ptr(), _lib.strides(k_new, (0, 1)),
+            v_new.data_ptr(), _lib.strides(v_new, (0, 1)),
+            k_ring.data_ptr(), _lib.strides(k_ring, (0, 1, 2)),
+            v_ring.data_ptr(), _lib.strides(v_ring, (0, 1, 2)),
+            out.data_ptr(), _lib.strides(out, (0, 1)),
+            B, H, D, int(W), pos.data_ptr(), float(scale), int(nsplit),
+            _lib.ptr(workspace), ws_bytes, _lib.current_stream(dev))
+    _lib.check(rc, "daisy_decode_fwd_at")
     return out
 
 
@@ -262,7 +310,8 @@ def kda_gate_fwd(g: torch.Tensor, A_log: torch.Tensor, head_k_dim: int,
 
 
 def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
-             cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, pos0: int = 0,
+             cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+             pos0: Union[int, torch.Tensor] = 0,
              ve: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
              q_out: Optional[torch.Tensor] = None, k_out: Optional[torch.Tensor] = None,
              v_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
@@ -272,8 +321,19 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
     contiguous last dim; ``gate`` is a one-element fp32 tensor holding the (bf16-rounded)
     sigmoid of the gate logit.  Outputs default to new contiguous ``[B, T, H, D]`` tensors;
     any strided bf16 ``[B, T, H, D]`` view may be passed instead.
+
+    ``pos0`` may be a one-element int32 device tensor: the kernel then reads the position when
+    it runs (a launch recorded in a HIP graph follows the tensor's value from replay to replay);
+    the caller keeps ``pos0 + T`` within the tables, which cannot be checked here.
     """
-    dev = _lib.require_gpu(q, k, v, ve, gate, cos, sin, q_out, k_out, v_out)
+    pos_dev = pos0 if isinstance(pos0, torch.Tensor) else None
+    if pos_dev is not None:
+        if pos_dev.dtype != torch.int32 or pos_dev.numel() != 1:
+            raise ValueError("a device position must be a one-element int32 tensor")
+        if cos is None:
+            raise ValueError("a device position needs the rotary tables")
+        pos0 = 0
+    dev = _lib.require_gpu(q, k, v, ve, gate, cos, sin, q_out, k_out, v_out, pos_dev)
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_bf16(name, t, 4)
     B, T, H, D = q.shape
@@ -306,13 +366,15 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
     qo, ko, vo = outs
     d3 = (0, 1, 2)
     lib = _lib.load()
+    ins = (q.data_ptr(), _lib.strides(q, d3), k.data_ptr(), _lib.strides(k, d3), v.data_ptr(), _lib.strides(v, d3),
+           _lib.ptr(ve), None if ve is None else _lib.strides(ve, d3), _lib.ptr(gate), _lib.ptr(cos), _lib.ptr(sin))
+    outs = (qo.data_ptr(), _lib.strides(qo, d3), ko.data_ptr(), _lib.strides(ko, d3), vo.data_ptr(), _lib.strides(vo, d3),
+            B, T, H, D, float(eps))
     with torch.cuda.device(dev):
-        rc = lib.daisy_qkv_prep_fwd(
-            q.data_ptr(), _lib.strides(q, d3), k.data_ptr(), _lib.strides(k, d3), v.data_ptr(), _lib.strides(v, d3),
-            _lib.ptr(ve), None if ve is None else _lib.strides(ve, d3), _lib.ptr(gate),
-            _lib.ptr(cos), _lib.ptr(sin), int(pos0),
-            qo.data_ptr(), _lib.strides(qo, d3), ko.data_ptr(), _lib.strides(ko, d3), vo.data_ptr(), _lib.strides(vo, d3),
-            B, T, H, D, float(eps), _lib.current_stream(dev))
+        if pos_dev is None:
+            rc = lib.daisy_qkv_prep_fwd(*ins, int(pos0), *outs, _lib.current_stream(dev))
+        else:
+            rc = lib.daisy_qkv_prep_fwd_at(*ins, pos_dev.data_ptr(), int(cos.shape[0]), *outs, _lib.current_stream(dev))
     _lib.check(rc, "daisy_qkv_prep_fwd")
     return qo, ko, vo
 

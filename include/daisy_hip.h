@@ -124,6 +124,27 @@ int daisy_decode_fwd(const void* q, const int64_t* q_strides,
                      float scale, int nsplit,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same decode step with the position held in device memory: `pos` points at one
+ * int32 t (the number of tokens already in the ring, as DaisyCore.step's `pos`,
+ * models/daisy/daisy_core.py:294-323, and KVCache.t, inference/kv_cache.py:52-55).  The
+ * kernel reads t when it runs, attends min(t + 1, ring_rows) live rows and writes the new
+ * row to slot t % ring_rows, so that a launch recorded once (a HIP graph of the whole
+ * model step) can be replayed for every later position; the caller increments *pos
+ * between steps.  q and k_new arrive rotated (see daisy_qkv_prep_fwd_at); the new row is
+ * always written back.  The grid is fixed by ring_rows: size the workspace with
+ * daisy_decode_workspace_bytes(B, H, D, ring_rows, nsplit).  D is 64 or 128.
+ */
+int daisy_decode_fwd_at(const void* q, const int64_t* q_strides,
+                        const void* k_new, const int64_t* k_new_strides,
+                        const void* v_new, const int64_t* v_new_strides,
+                        void* k_cache, const int64_t* k_cache_strides,
+                        void* v_cache, const int64_t* v_cache_strides,
+                        void* o, const int64_t* o_strides,
+                        int B, int H, int D,
+                        int ring_rows, const int32_t* pos,
+                        float scale, int nsplit,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Kernel 3: chunked Kimi Delta Attention forward.
  *
@@ -207,6 +228,22 @@ int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
                        void* k_out, const int64_t* k_out_strides,
                        void* v_out, const int64_t* v_out_strides,
                        int B, int T, int H, int D, float eps, void* stream);
+
+/* The same pass with the first position read from device memory when the kernel runs
+ * (`pos0` points at one int32; the decode-step counterpart of Rotary.step's host `pos`,
+ * models/daisy/attention.py:64-70).  cos, sin are fp32 [table_rows, D/2] and required; a
+ * position whose rows would leave the table is held at the table's end (memory safety
+ * only: the caller keeps *pos0 + T <= table_rows).
+ */
+int daisy_qkv_prep_fwd_at(const void* q, const int64_t* q_strides,
+                          const void* k, const int64_t* k_strides,
+                          const void* v, const int64_t* v_strides,
+                          const void* ve, const int64_t* ve_strides, const float* gate,
+                          const float* cos, const float* sin, const int32_t* pos0, int table_rows,
+                          void* q_out, const int64_t* q_out_strides,
+                          void* k_out, const int64_t* k_out_strides,
+                          void* v_out, const int64_t* v_out_strides,
+                          int B, int T, int H, int D, float eps, void* stream);
 
 /* ---------------------------------------------------------------------------
  * The KDA layer's elementwise neighbours (models/daisy/attention_kimi.py:155-158: three

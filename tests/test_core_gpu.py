@@ -210,6 +210,46 @@ def test_batched_prefill_and_steps_match_single_sequences():
             core.prefill(model, bad, KVCache(4, B, 2, W, 128, DEV, torch.bfloat16))
 
 
+@pytest.mark.parametrize("window,T,n_steps", [(48, 20, 60), (1024, 1000, 40)])
+def test_recorded_step_replays_match_eager_steps(window, T, n_steps):
+    """core.GraphedStep: the step is recorded once and replayed with the position in device memory.
+    Every replay is checked against an eager step on a second cache, with eager work and a
+    synchronisation between replays; the ring is partly filled at first and wraps during the run
+    (the 1024-slot ring is read by several splits per head).  A cache that is reset and filled
+    again keeps working with the same recording."""
+    with torch.no_grad():
+        model = _Core(window=window, max_seq_len=2048).to(DEV)
+        B = 2
+        ids = torch.randint(2, 96, (B, T + n_steps), generator=torch.Generator().manual_seed(8)).to(DEV)
+        eager = KVCache(4, B, 2, window, 128, DEV, torch.bfloat16)
+        replayed = KVCache(4, B, 2, window, 128, DEV, torch.bfloat16)
+        core.prefill(model, ids[:, :T], eager)
+        core.prefill(model, ids[:, :T], replayed)
+        graphed = core.GraphedStep(model, replayed)
+        worst = 0.0
+        for s in range(n_steps):
+            say(f"recorded step W{window} replay {s}")
+            want = core.step(model, ids[:, T + s], eager)
+            got = graphed(ids[:, T + s]).clone()
+            torch.cuda.synchronize()
+            worst = max(worst, (got - want).abs().max().item())
+            _close(got, want, f"replay {s} logits", tol=1e-2)
+        say(f"recorded step W{window}: worst logit difference over {n_steps} replays {worst:.3e}")
+        assert replayed.t == eager.t == T + n_steps and int(graphed.pos) == replayed.t
+        _close(replayed.k, eager.k, "ring keys", tol=1e-2)
+        _close(replayed.v, eager.v, "ring values", tol=1e-2)
+        # a new prompt in the same cache: the recording follows the cache's position
+        for c in (eager, replayed):
+            c.reset_history()
+            core.prefill(model, ids[:, 3:T], c)
+        for s in range(3):
+            want = core.step(model, ids[:, T + s], eager)
+            _close(graphed(ids[:, T + s]), want, f"after reset, replay {s} logits", tol=1e-2)
+        # the walk cannot be recorded over chronological views
+        with pytest.raises(Exception):
+            core.GraphedStep(model, KVCache(4, B, 2, window, 128, DEV, torch.float16))
+
+
 def test_generator_generate_batch():
     """Generator.generate_batch: greedy equals core.generate_greedy; sampling settings apply per row and a
     seed reproduces the draw; the repetition penalty of a batch equals the penalty row by row."""
@@ -223,6 +263,8 @@ def test_generator_generate_batch():
         gen = Generator(model, window=model.window_size, seed=3, device=torch.device(DEV), dtype=torch.bfloat16, temperature=0.0)
         out = gen.generate_batch(ids, 6)
         assert out.shape == (B, 6) and torch.equal(out, core.generate_greedy(model, ids, 6))
+        for _ in range(2):   # recorded on the first call, replayed on the second
+            assert torch.equal(gen.generate_batch(ids, 6, record_steps=True), out), "recorded steps change the tokens"
         gen.set_temperature(0.8)
         gen.top_k, gen.top_p = 20, 0.9
         gen.set_repetition_penalty(1.3)

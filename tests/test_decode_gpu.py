@@ -91,6 +91,36 @@ def test_decode_consecutive_steps_append_in_place():
     assert torch.equal(dkc.cpu(), kc) and torch.equal(dvc.cpu(), vc)
 
 
+@pytest.mark.parametrize("B,H,D,W,nsplit", [(2, 3, 128, 64, 0), (1, 2, 128, 1024, 0), (1, 2, 128, 1024, 4), (3, 2, 64, 200, 3)])
+def test_decode_at_device_position_matches_oracle(B, H, D, W, nsplit):
+    """The position comes from device memory: one set of launch arguments serves an empty ring, a
+    partly filled one (most splits empty), the last free slot and wrapped positions."""
+    g = torch.Generator().manual_seed(W + D)
+    pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for t in (0, 1, 7, W // 2, W - 1, W, W + 1, 5 * W + 3):
+        say(f"decode_at case B{B} H{H} D{D} W{W} nsplit{nsplit} t{t}")
+        kc = torch.randn(B, H, W, D, generator=g).bfloat16()
+        vc = torch.randn(B, H, W, D, generator=g).bfloat16()
+        q, kn, vn = (torch.randn(B, H, D, generator=g).bfloat16() for _ in range(3))
+        n_rows, slot = min(t + 1, W), t % W
+        k_exp, v_exp = kc.clone(), vc.clone()
+        k_exp[:, :, slot] = kn
+        v_exp[:, :, slot] = vn
+        ref = _ref_decode(q, k_exp[:, :, :n_rows], v_exp[:, :, :n_rows])
+        dkc, dvc = kc.cuda(), vc.cuda()
+        pos.fill_(t)
+        o = ops.decode_attention_at(q.cuda(), kn.cuda(), vn.cuda(), dkc, dvc, pos, nsplit=nsplit)
+        torch.cuda.synchronize()
+        assert_close_bf16(o, ref, f"o at t={t}")
+        assert torch.equal(dkc.cpu(), k_exp), "cache K after the step (only the new slot may change)"
+        assert torch.equal(dvc.cpu(), v_exp), "cache V after the step"
+        if n_rows == W:
+            # full ring: same splits as the host-position entry point, so the same bits
+            o_host = ops.decode_attention(q.cuda(), kn.cuda(), vn.cuda(), kc.cuda(), vc.cuda(), n_rows=W, new_idx=slot,
+                                          write_back=True, nsplit=nsplit)
+            assert torch.equal(o, o_host), "device- and host-position entry points differ on a full ring"
+
+
 def test_decode_rejects_bad_arguments():
     z = torch.zeros(1, 1, 128, dtype=torch.bfloat16, device="cuda:0")
     rows = torch.zeros(1, 1, 4, 128, dtype=torch.bfloat16, device="cuda:0")

@@ -89,6 +89,29 @@ def test_prep_matches_library_ops_on_gpu():
         _check(got, ref.cpu(), what)
 
 
+def test_prep_at_device_position_equals_host_position():
+    """Position read from device memory: same bits as the host-position entry point, for a decode
+    row (T = 1) and a short run of rows, at several positions from one position tensor."""
+    B, H, D, rows = 2, 3, 128, 300
+    g = torch.Generator().manual_seed(11)
+    cos, sin = (t.cuda() for t in oracle.rope_tables(D, rows))
+    pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for T in (1, 5):
+        q, k, v, ve = (torch.randn(B, T, H, D, generator=g).bfloat16().cuda() for _ in range(4))
+        gate = torch.sigmoid(torch.tensor(0.3)).bfloat16().float().reshape(1).cuda()
+        for p0 in (0, 17, rows - T):
+            say(f"prep_at case T{T} pos0 {p0}")
+            pos.fill_(p0)
+            want = ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, pos0=p0, ve=ve, gate=gate)
+            got = ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, pos0=pos, ve=ve, gate=gate)
+            for a, b, name in zip(got, want, "qkv"):
+                assert torch.equal(a, b), f"{name} at pos0={p0}"
+    with pytest.raises(ValueError):
+        ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, pos0=pos)                      # no tables
+    with pytest.raises(ValueError):
+        ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, pos0=pos.long())
+
+
 def test_prep_rejects_bad_arguments():
     q = torch.zeros(1, 4, 2, 128, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError):

@@ -425,7 +425,14 @@ def bench_next_rows(steps, warmup):
         layer.prefill(xs, None)
         x1 = torch.randn(64, 1, 2048, device=dev).bfloat16()
         ms_step = time_gpu(lambda: layer.step(x1, None, None, 64, None, None), 32, 4)
-    out["kimi_layer_dim2048_H16"] = {"forward_ms_B4_T8192": ms_layer, "step_ms_B64": ms_step}
+        # the same step replayed as a HIP graph (state and windows are updated in place at fixed addresses)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            layer.step(x1, None, None, 64, None, None)
+        ms_step_graph = time_gpu(graph.replay, 32, 4)
+    out["kimi_layer_dim2048_H16"] = {"forward_ms_B4_T8192": ms_layer, "step_ms_B64": ms_step,
+                                     "step_ms_B64_recorded_graph": ms_step_graph}
+    del graph
     return out
 
 

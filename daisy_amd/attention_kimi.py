@@ -53,7 +53,9 @@ class ShortConvolution(nn.Module):
         self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=dtype)) if bias else None
 
     def forward(self, x: Tensor, cache: Optional[Tensor] = None, output_final_state: bool = False,
-                cu_seqlens: Optional[Tensor] = None) -> Tuple[Tensor, Optional[Tensor]]:
+                cu_seqlens: Optional[Tensor] = None, inplace_cache: bool = False) -> Tuple[Tensor, Optional[Tensor]]:
+        """``inplace_cache`` (GPU kernel path, a few steps at a time): the window is updated inside
+        ``cache`` and that tensor is returned, so that its address stays the same from step to step."""
         if cu_seqlens is not None:
             # Sequences packed along T of a batch of one: the window must not reach across a
             # boundary, so every sequence is convolved by itself; caches are [N, C, K].
@@ -73,7 +75,8 @@ class ShortConvolution(nn.Module):
         K = self.kernel_size
         if x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and 2 <= K <= 4 and C % 8 == 0:
             # one streaming pass on the GPU (no transposes, no concatenation)
-            return ops.short_conv(x, self.weight, self.bias, cache, output_final_state, "silu")
+            return ops.short_conv(x, self.weight, self.bias, cache, output_final_state, "silu", inplace_cache=inplace_cache)
+        torch._assert(not inplace_cache, "the window is updated in place by the GPU kernel only")
         xt = x.transpose(1, 2)                                        # [B, C, T]
         prev = cache[..., 1:] if cache is not None else xt.new_zeros(B, C, K - 1)
         window = torch.cat([prev.to(xt.dtype), xt], dim=-1)           # [B, C, K - 1 + T]
@@ -150,6 +153,10 @@ class KimiLinearSelfAttention(nn.Module):
         self._recurrent_state: Optional[Tensor] = None
         self._conv_state = None
         self._seen = 0
+        # Buffers that held the states before the last reset_history: the next prompt's states are
+        # stored into them when they fit, so that the addresses a recorded decode step reads and
+        # writes stay the same for the life of the module.
+        self._state_homes = (None, None, None, None)
 
     def _apply(self, fn, recurse=True):
         # The decay parameters stay fp32 under module-wide casts, as the reference creates them.
@@ -160,10 +167,30 @@ class KimiLinearSelfAttention(nn.Module):
                 prm.data = prm.data.float()
         return self
 
+    # step() keeps its own recurrent and convolution states; the k_ctx / v_ctx arguments are not read.
+    uses_kv_context = False
+
     def reset_history(self):
+        if self._recurrent_state is not None:
+            self._state_homes = (self._recurrent_state,) + tuple(self._conv_state or (None, None, None))
         self._recurrent_state = None
         self._conv_state = None
         self._seen = 0
+
+    def state_tensors(self):
+        """The tensors a decode step updates in place (recurrent state, convolution windows)."""
+        held = (self._recurrent_state,) + tuple(self._conv_state or ())
+        return [t for t in held if t is not None]
+
+    @staticmethod
+    def _store(home: Optional[Tensor], fresh: Optional[Tensor]) -> Optional[Tensor]:
+        """``fresh`` itself, or ``home`` holding its values when that buffer fits."""
+        if fresh is None or home is None or home is fresh:
+            return fresh
+        if home.shape == fresh.shape and home.dtype == fresh.dtype and home.device == fresh.device:
+            home.copy_(fresh)
+            return home
+        return fresh
 
     def _core(self, x: Tensor, ve: Optional[Tensor], use_cache: bool, attn_mask=None) -> Tensor:
         B0, S0, _ = x.shape
@@ -183,9 +210,12 @@ class KimiLinearSelfAttention(nn.Module):
         state = self._recurrent_state if use_cache else None
         convs = self._conv_state if (use_cache and self._conv_state is not None) else (None, None, None)
         if self.use_short_conv:
-            q, cq = self.q_conv1d(self.q_proj(x), convs[0], use_cache, cu_seqlens)
-            k, ck = self.k_conv1d(self.k_proj(x), convs[1], use_cache, cu_seqlens)
-            v, cv = self.v_conv1d(self.v_proj(x), convs[2], use_cache, cu_seqlens)
+            # a decode step shifts its windows in place (same tensors, same addresses, every step)
+            shift = (use_cache and T == 1 and cu_seqlens is None and x.is_cuda
+                     and all(c is not None and c.dtype == torch.bfloat16 and c.is_contiguous() for c in convs))
+            q, cq = self.q_conv1d(self.q_proj(x), convs[0], use_cache, cu_seqlens, shift)
+            k, ck = self.k_conv1d(self.k_proj(x), convs[1], use_cache, cu_seqlens, shift)
+            v, cv = self.v_conv1d(self.v_proj(x), convs[2], use_cache, cu_seqlens, shift)
         else:
             q, k, v = F.silu(self.q_proj(x)), F.silu(self.k_proj(x)), F.silu(self.v_proj(x))
             cq = ck = cv = None
@@ -203,8 +233,10 @@ class KimiLinearSelfAttention(nn.Module):
             o, state = chunk_kda(q, k, v, g, beta, initial_state=state, output_final_state=use_cache,
                                  use_qk_l2norm_in_kernel=True, cu_seqlens=cu_seqlens)
         if use_cache:
-            self._recurrent_state = state
-            self._conv_state = (cq, ck, cv)
+            homes = self._state_homes
+            self._recurrent_state = self._store(homes[0], state)
+            self._conv_state = tuple(self._store(h, c) for h, c in zip(homes[1:], (cq, ck, cv)))
+            self._state_homes = (self._recurrent_state,) + self._conv_state
             self._seen += T
         gate = self.g_proj(x).view(B, T, H, Dv)
         o = self.o_norm(o.to(gate.dtype), gate)

@@ -141,8 +141,8 @@ def _walk_step(model, token_ids: Tensor, cache: KVCache, pos) -> Tensor:
             gate = torch.sigmoid(skip_weights[skip_map[i]])
             x = x * gate + (1 - gate) * skip_connections[skip_map[i]]
         blk = model.blocks[i]
-        if getattr(blk, "attn", None) is None:
-            k_ctx = v_ctx = None
+        if getattr(blk, "attn", None) is None or not getattr(blk.attn, "uses_kv_context", True):
+            k_ctx = v_ctx = None        # no attention, or one that keeps its own state (KDA layers)
         elif in_place and getattr(blk.attn, "accepts_ring_context", False):
             k_ctx = v_ctx = cache.ring(i)
         else:
@@ -194,12 +194,18 @@ class GraphedStep:
     def _record(self):
         dev = self.cache.k.device
         # One eager pass on a side stream first (library handles, workspaces, the allocator's pools);
-        # it writes the same row the first replay writes again.
+        # in the ring it writes the same row the first replay writes again.
+        # Layers that keep their own state (KDA) would advance it twice: it is put back afterwards.
+        stateful = [t for blk in self.model.blocks if hasattr(getattr(blk, "attn", None), "state_tensors")
+                    for t in blk.attn.state_tensors()]
+        saved = [t.clone() for t in stateful]
         side = torch.cuda.Stream(device=dev)
         side.wait_stream(torch.cuda.current_stream(dev))
         with torch.cuda.stream(side):
             self._body()
         torch.cuda.current_stream(dev).wait_stream(side)
+        for t, old in zip(stateful, saved):
+            t.copy_(old)
         self.pos.fill_(self.cache.t)
         self._graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self._graph):

@@ -194,6 +194,9 @@ extern "C" int daisy_short_conv_fwd(const void* x, const int64_t* x_strides, con
                   "short_conv: x, y, weight, bias and the windows must be 16-byte aligned");
   for (int i = 0; i < 2; ++i)
     DAISY_CHECK_ARG(x_strides[i] % 8 == 0 && y_strides[i] % 8 == 0, "short_conv: strides must be multiples of 8 elements");
+  // Updating the window in place is safe only while the thread that writes it is the one that read it.
+  DAISY_CHECK_ARG(cache_out == nullptr || cache_out != cache_in || T <= kConvSeg,
+                  "short_conv: the window can be updated in place for T <= %d only (T=%d)", kConvSeg, T);
   ConvParams p;
   p.x = (const uint16_t*)x; p.x_sb = x_strides[0]; p.x_st = x_strides[1];
   p.w = (const uint16_t*)weight; p.bias = (const uint16_t*)bias; p.cache_in = (const uint16_t*)cache_in;

@@ -432,11 +432,13 @@ def probe_read_rate(gib: int = 2, workgroups: int = 8192, repeats: int = 5, devi
 
 def short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                cache: Optional[torch.Tensor] = None, output_final_state: bool = False,
-               activation: Optional[str] = "silu") -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+               activation: Optional[str] = "silu", inplace_cache: bool = False
+               ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """Depthwise causal convolution over time + SiLU for ``x [B, T, C]`` bf16 (``daisy_short_conv_fwd``).
 
     ``weight [C, 1, K]`` or ``[C, K]``; ``cache [B, C, K]`` holds the last K inputs of the sequence
-    so far.  Returns ``(y [B, T, C], new cache or None)``.
+    so far.  Returns ``(y [B, T, C], new cache or None)``.  ``inplace_cache``: the new window is
+    written into ``cache`` itself (bf16, contiguous, ``T <= 32``: decode steps) and ``cache`` is returned.
     """
     dev = _lib.require_gpu(x, weight, bias, cache)
     _check_bf16("x", x, 3)
@@ -453,9 +455,16 @@ def short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
     if cache is not None:
         if cache.shape != (B, C, K):
             raise ValueError(f"short_conv: cache must be [{B}, {C}, {K}], got {tuple(cache.shape)}")
+        if inplace_cache and (cache.dtype != torch.bfloat16 or not cache.is_contiguous()):
+            raise ValueError("short_conv: a window updated in place must be a contiguous bf16 tensor")
         cache = cache.to(torch.bfloat16).contiguous()
+    elif inplace_cache:
+        raise ValueError("short_conv: inplace_cache needs a cache")
     y = torch.empty(B, T, C, dtype=torch.bfloat16, device=dev)
-    new_cache = torch.empty(B, C, K, dtype=torch.bfloat16, device=dev) if output_final_state else None
+    if inplace_cache:
+        new_cache = cache
+    else:
+        new_cache = torch.empty(B, C, K, dtype=torch.bfloat16, device=dev) if output_final_state else None
     lib = _lib.load()
     with torch.cuda.device(dev):
         rc = lib.daisy_short_conv_fwd(x.data_ptr(), _lib.strides(x, (0, 1)), w.data_ptr(), _lib.ptr(bias), _lib.ptr(cache),

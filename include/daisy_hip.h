@@ -257,7 +257,8 @@ int daisy_qkv_prep_fwd_at(const void* q, const int64_t* q_strides,
  * x, y       : [B, T, C] bf16, channel stride 1, strides = {batch, time} in elements (multiples of 8)
  * weight     : [C, K] bf16 (the layout of a grouped Conv1d weight [C, 1, K]); bias: [C] bf16 or NULL
  * cache_in   : [B, C, K] bf16 or NULL -- the last K inputs before t = 0 (zeros if NULL)
- * cache_out  : [B, C, K] bf16 or NULL -- receives the last K inputs of (cache_in | x)
+ * cache_out  : [B, C, K] bf16 or NULL -- receives the last K inputs of (cache_in | x); may be the
+ *              same buffer as cache_in when T <= 32 (decode steps update their window in place)
  * C must be a multiple of 8.
  */
 int daisy_short_conv_fwd(const void* x, const int64_t* x_strides, const void* weight, const void* bias,

@@ -250,6 +250,41 @@ def test_recorded_step_replays_match_eager_steps(window, T, n_steps):
             core.GraphedStep(model, KVCache(4, B, 2, window, 128, DEV, torch.float16))
 
 
+def test_recorded_step_with_a_kda_layer():
+    """A hybrid stack (KDA layer first, attention layers after it): the KDA layer keeps its recurrent
+    state and convolution windows in buffers whose addresses survive reset_history, so the recording
+    made for the first prompt also serves the second one."""
+    import copy
+    from daisy_amd import KimiLinearSelfAttention
+    with torch.no_grad():
+        model = _Core(window=48, max_seq_len=512)
+        torch.manual_seed(1)
+        model.blocks[0].attn = KimiLinearSelfAttention(256, 2, 512, 128, receives_ve=True).bfloat16()
+        model = model.to(DEV)
+        twin = copy.deepcopy(model)
+        B, T, n_steps = 2, 30, 40
+        ids = torch.randint(2, 96, (B, T + n_steps), generator=torch.Generator().manual_seed(9)).to(DEV)
+        eager = KVCache(4, B, 2, 48, 128, DEV, torch.bfloat16)
+        replayed = KVCache(4, B, 2, 48, 128, DEV, torch.bfloat16)
+        graphed = None
+        for first in (0, 5):                                  # two prompts, one recording
+            for m, c in ((model, eager), (twin, replayed)):
+                for blk in m.blocks:
+                    if blk.attn is not None:
+                        blk.attn.reset_history()
+                c.reset_history()
+                core.prefill(m, ids[:, first:T], c)
+            if graphed is None:
+                graphed = core.GraphedStep(twin, replayed)
+            for s in range(n_steps):
+                say(f"recorded hybrid step, prompt from {first}, replay {s}")
+                want = core.step(model, ids[:, T + s], eager)
+                got = graphed(ids[:, T + s])
+                _close(got, want, f"prompt from {first}, replay {s} logits", tol=1e-2)
+            _close(twin.blocks[0].attn._recurrent_state, model.blocks[0].attn._recurrent_state, "KDA state", tol=1e-2)
+            _close(replayed.k, eager.k, "ring keys", tol=1e-2)
+
+
 def test_generator_generate_batch():
     """Generator.generate_batch: greedy equals core.generate_greedy; sampling settings apply per row and a
     seed reproduces the draw; the repetition penalty of a batch equals the penalty row by row."""

@@ -97,7 +97,8 @@ def penalise_repeats(logits: Tensor, recent: Tensor, strength: Tensor, _one: Opt
 # ----------------------------------------------------------------------------------------------
 class Generator:
     def __init__(self, model, window, seed, device=None, dtype=torch.float16, max_seq_len: int = 65536,
-                 temperature=1.0, top_k=None, top_p=None, repetition_penalty=1.0, eos_token_id=None):
+                 temperature=1.0, top_k=None, top_p=None, repetition_penalty=1.0, eos_token_id=None,
+                 record_steps: bool = False):
         eos = eos_token_id if eos_token_id is not None else getattr(model, "eos_token_id", None)
         if eos is None:
             raise AssertionError("eos_token_id must be given or be an attribute of the model")
@@ -121,6 +122,11 @@ class Generator:
         # In-place decode: every layer must understand ring handles and the ring must be bf16.
         self.use_ring_context = dtype == torch.bfloat16 and all(isinstance(a, CausalSelfAttention) for a in attn)
         self._rings = [self.cache.ring(i) for i in range(len(layers))] if self.use_ring_context else None
+        # record_steps: the decode step is recorded once as a HIP graph and replayed per token
+        # (daisy_amd.core.GraphedStep walks the model's layers itself, so the model needs the
+        # attributes of the reference's DaisyCore, a bf16 cache and this package's attention).
+        self.record_steps = bool(record_steps)
+        self._recorded_step = None
 
         torch.manual_seed(seed)
         self._tokens = torch.empty(256, dtype=torch.long, device=self.device)
@@ -192,6 +198,13 @@ class Generator:
         """One decode step: the model sees every layer's context as it was before this token,
         the new rows go into slot ``t % W`` (unless the decode kernel has already put them
         there), the cache moves on by one position."""
+        if self.record_steps:
+            if self._recorded_step is None:
+                from . import core
+                self._recorded_step = core.GraphedStep(self.model, self.cache)
+            logits = self._recorded_step(token)
+            self._remember(token)
+            return self._trim(logits)
         k_ctxs, v_ctxs = self._contexts()
         logits, k_rows, v_rows = self.model.step(token, k_ctxs, v_ctxs, self.cache.t)
         # A layer without attention returns None; its slot is filled with zeros shaped like the

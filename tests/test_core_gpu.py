@@ -87,6 +87,14 @@ class _Core(nn.Module):
     def compute_value_embeddings(self, ids):
         return {i: m(ids) for i, m in self.ve_module_map.items()}
 
+    def prefill(self, ids):        # the reference's signature: logits of the last position and kv [2, L, B, H, T, D]
+        return core.prefill(self, ids)
+
+    def reset_history(self):
+        for blk in self.blocks:
+            if blk.attn is not None:
+                blk.attn.reset_history()
+
     # the reference's own step signature (daisy_core.py:294-323), used as the comparison route
     def step(self, token_id, k_ctxs, v_ctxs, pos):
         token_id = token_id.view(1, 1)
@@ -285,6 +293,23 @@ def test_recorded_step_with_a_kda_layer():
             _close(replayed.k, eager.k, "ring keys", tol=1e-2)
 
 
+def test_generator_single_sequence_with_recorded_steps():
+    """Generator.generate (the reference's one-sequence loop) with record_steps: the same tokens as
+    with steps launched kernel by kernel, for two prompts in a row on one generator (one recording)."""
+    from daisy_amd import Generator
+    with torch.no_grad():
+        model = _Core().to(DEV)
+        kw = dict(window=model.window_size, seed=3, device=torch.device(DEV), dtype=torch.bfloat16, temperature=0.0)
+        plain, recorded = Generator(model, **kw), Generator(model, record_steps=True, **kw)
+        for seed, T in ((13, 30), (14, 55)):      # the second prompt is longer than the ring
+            ids = torch.randint(2, 96, (T,), generator=torch.Generator().manual_seed(seed)).to(DEV)
+            want = torch.cat(list(plain.generate(ids, 24)))
+            got = torch.cat(list(recorded.generate(ids, 24)))
+            say(f"prompt of {T}: {want.numel()} tokens, recorded equal: {torch.equal(want, got)}")
+            assert torch.equal(want, got)
+            assert torch.equal(plain.history, recorded.history)
+
+
 def test_generator_generate_batch():
     """Generator.generate_batch: greedy equals core.generate_greedy; sampling settings apply per row and a
     seed reproduces the draw; the repetition penalty of a batch equals the penalty row by row."""
@@ -292,7 +317,6 @@ def test_generator_generate_batch():
     from daisy_amd.generate import penalise_repeats
     with torch.no_grad():
         model = _Core().to(DEV)
-        model.reset_history = lambda: None
         B, T = 3, 40
         ids = torch.randint(2, 96, (B, T), generator=torch.Generator().manual_seed(7)).to(DEV)
         gen = Generator(model, window=model.window_size, seed=3, device=torch.device(DEV), dtype=torch.bfloat16, temperature=0.0)

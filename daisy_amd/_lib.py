@@ -49,6 +49,16 @@ SIGNATURES = {
         c_int, c_void_p,                                        # ring_rows, pos (device int32)
         c_float, c_int,                                         # scale, nsplit
         c_void_p, c_size_t, c_void_p]),                         # workspace, bytes, stream
+    "daisy_attn_step_fwd": (c_int, [
+        c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k, v rows of the projection (+strides)
+        c_void_p, _I64P, c_void_p,                              # ve, ve strides, gate
+        c_void_p, c_void_p, c_int,                              # cos, sin, table_rows
+        c_int, c_void_p, c_float,                               # pos, pos_dev, eps
+        c_void_p, _I64P, c_void_p, _I64P,                       # k_cache, v_cache (+strides)
+        c_void_p, _I64P,                                        # o (+strides)
+        c_int, c_int, c_int, c_int,                             # B, H, D, ring_rows
+        c_float, c_int,                                         # scale, nsplit
+        c_void_p, c_size_t, c_void_p]),                         # workspace, bytes, stream
     "daisy_kda_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "daisy_kda_chunk_fwd": (c_int, [
         c_void_p, c_void_p, c_void_p,                           # q, k, v

@@ -323,8 +323,15 @@ class CausalSelfAttention(nn.Module):
         B = x.size(0)
         torch._assert(x.size(1) == 1, "step() requires single position only")
         fused = self._fused_prep_ok()
+        ring = k_ctx if isinstance(k_ctx, RingContext) else None
+        in_ring = fused and ring is not None and ring.k.dtype == torch.bfloat16 and window == ring.W
         if isinstance(pos, Tensor):
-            return self._step_at(x, k_ctx, pos, ve, window, fused)
+            if not in_ring:
+                raise ValueError("a device-side position needs the fused kernels (bf16 weights, head dim 64 or 128) "
+                                 "and the RingContext of a bf16 KVCache whose size equals the window")
+            return self._step_in_ring(x, ring, pos, ve)
+        if in_ring and pos == ring.t:
+            return self._step_in_ring(x, ring, pos, ve)
         if fused:
             # q and k come back rotated: the decode kernel is told not to rotate again.
             q, k, v = self._project_qkv_fused(x, ve, pos)
@@ -338,7 +345,6 @@ class CausalSelfAttention(nn.Module):
             cos_row, sin_row = cos[pos], sin[pos]
         qk, kk, vk = (self._kernel_dtype(t)[:, 0] for t in (q, k, v))  # [B, H, D]
 
-        ring = k_ctx if isinstance(k_ctx, RingContext) else None
         if ring is not None and (window != ring.W or ring.k.dtype != torch.bfloat16 or pos != ring.t):
             # Not the layout the in-place path streams; use the chronological rows.
             k_ctx, v_ctx = ring.cache.view(ring.layer)
@@ -372,14 +378,24 @@ class CausalSelfAttention(nn.Module):
         y = F.linear(y, self.qkvo_w[3])
         return y, k_new, v_new
 
-    def _step_at(self, x, ring, pos: Tensor, ve: Optional[Tensor], window: Optional[int], fused: bool):
-        """``step`` at a position that only the device knows (see there)."""
-        if not (fused and isinstance(ring, RingContext) and ring.k.dtype == torch.bfloat16 and window == ring.W):
-            raise ValueError("a device-side position needs the fused pre-attention kernel (bf16 weights, head dim 64 "
-                             "or 128) and the RingContext of a bf16 KVCache whose size equals the window")
-        B = x.size(0)
-        q, k, v = self._project_qkv_fused(x, ve, pos)
-        o = ops.decode_attention_at(q[:, 0], k[:, 0], v[:, 0], ring.k, ring.v, pos, scale=self.attn_scale)
+    def _step_in_ring(self, x, ring: RingContext, pos: Union[int, Tensor], ve: Optional[Tensor]):
+        """The step as two projections around one kernel: norm, RoPE, value-embedding mix, the new
+        rows' way into slot ``pos % W`` and the attention over the ring all happen in
+        ``ops.attn_step``.  Returns the new rows as views of the ring, or ``None, None`` when only
+        the device knows the position."""
+        B, H, D = x.size(0), self.num_heads, self.head_dim
+        qkv = F.linear(x.to(self.qkvo_w.dtype), self.qkvo_w[:3].flatten(end_dim=1)).view(B, 3 * H, D)
+        ve_rows = gate = None
+        if self.receives_ve:
+            torch._assert(ve is not None, "ve must be provided when receives_ve=True")
+            ve_rows = ve.to(torch.bfloat16).view(B, H, D)
+            gate = torch.sigmoid(self.g_ve.detach()).to(torch.bfloat16).float().reshape(1)
+        o = ops.attn_step(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], ring.k, ring.v, pos,
+                          cos=self.rotary.cos, sin=self.rotary.sin, eps=NORM_EPS_BF16, ve=ve_rows, gate=gate,
+                          scale=self.attn_scale)
         ring.mark_written()
         y = F.linear(o.reshape(B, 1, self.m_dim), self.qkvo_w[3])
-        return y, k, v   # the rows as the kernel stored them in slot pos % W
+        if isinstance(pos, Tensor):
+            return y, None, None
+        slot = pos % ring.W
+        return y, ring.k[:, :, slot, :].unsqueeze(1), ring.v[:, :, slot, :].unsqueeze(1)

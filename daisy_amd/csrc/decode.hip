@@ -29,6 +29,11 @@ struct DecodeParams {
   // launch can be replayed for later positions): the cache is a ring of ring_rows slots,
   // n_rows = min(t + 1, ring_rows) of them are live and the new row goes to slot t % ring_rows.
   const int32_t* pos_dev; int ring_rows;
+  // For the kernel variant that prepares the rows itself (RMS norm of q, k_new, v_new, RoPE of q
+  // and k_new at the step's position, value-embedding mix): the position when it is a launch
+  // argument, the rotation tables, and the optional second value row with its gate.
+  int pos_host; const float* cos_tab; const float* sin_tab; int table_rows; float eps;
+  const uint16_t* ve; int64_t ve_sb, ve_sh; const float* gate;
 };
 
 struct DecodeRange { int n_rows, new_idx, rows_per_split; };
@@ -73,6 +78,57 @@ __device__ __forceinline__ void load_vec_rot(const uint16_t* vec, int dl, const 
   }
 }
 
+// RMS norm of this lane's 8 channels of a [D] bf16 row (statistics over the row's D/8 lanes),
+// rounded to bf16 like the norm's output tensor, then the rotation, rounded again: the arithmetic
+// and the roundings of qkv_prep_kernel for one row.
+template <int D>
+__device__ __forceinline__ void norm_rot(const uint16_t* vec, int dl, const float* cos_row, const float* sin_row,
+                                         float eps, float* out) {
+  constexpr int LPR = D / 8, HALF = D / 2;
+  const bool lower = dl < HALF;
+  const int pl = lower ? dl + HALF : dl - HALF;
+  const int tl = lower ? dl : dl - HALF;
+  float own[8], par[8];
+  unpack8(*reinterpret_cast<const u32x4*>(vec + dl), own);
+  unpack8(*reinterpret_cast<const u32x4*>(vec + pl), par);
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ss += own[i] * own[i];
+  ss = group_sum<LPR>(ss);
+  const float rstd = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float a = round_bf16(own[i] * rstd), b = round_bf16(par[i] * rstd);
+    const float c = cos_row[tl + i], sn = sin_row[tl + i];
+    out[i] = round_bf16(lower ? rope_lo(a, b, c, sn) : rope_hi(b, a, c, sn));
+  }
+}
+
+// RMS norm of a value row and, when a second row is given, gate * v + (1 - gate) * ve with every
+// product and the sum rounded to bf16 (the roundings of a bf16 tensor library).
+template <int D>
+__device__ __forceinline__ void norm_mix(const uint16_t* vec, const uint16_t* ve, const float* gate, int dl,
+                                         float eps, float* out) {
+  constexpr int LPR = D / 8;
+  float own[8];
+  unpack8(*reinterpret_cast<const u32x4*>(vec + dl), own);
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ss += own[i] * own[i];
+  ss = group_sum<LPR>(ss);
+  const float rstd = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) out[i] = round_bf16(own[i] * rstd);
+  if (ve != nullptr) {
+    float e[8];
+    unpack8(*reinterpret_cast<const u32x4*>(ve + dl), e);
+    const float g = gate[0];
+    const float og = round_bf16(1.0f - g);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = round_bf16(round_bf16(g * out[i]) + round_bf16(og * e[i]));
+  }
+}
+
 struct SoftmaxState {
   float m, l;
   float acc[8];
@@ -89,7 +145,9 @@ __device__ __forceinline__ void merge_state(SoftmaxState& a, const SoftmaxState&
   a.m = m;
 }
 
-template <int D>
+// PREP: q, k_new and v_new are rows of the QKV projection output; the kernel normalises, rotates
+// and mixes them itself (every workgroup of a (batch, head) redoes these few hundred flops).
+template <int D, bool PREP>
 __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) {
   constexpr int LPR = D / 8;        // lanes per cache row
   constexpr int RPW = 64 / LPR;     // rows per wavefront load
@@ -102,9 +160,20 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
   const int dl = (lane % LPR) * 8;
 
   float qf[8], knf[8];
-  load_vec_rot<D>(p.q + b * p.q_sb + h * p.q_sh, dl, p.cos_row, p.sin_row, qf);
-  load_vec_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_row, p.sin_row, knf);
-  const u32x4 vn_packed = *reinterpret_cast<const u32x4*>(p.v_new + b * p.vn_sb + h * p.vn_sh + dl);
+  u32x4 vn_packed;
+  if constexpr (PREP) {
+    const int t = p.pos_dev != nullptr ? max(p.pos_dev[0], 0) : p.pos_host;
+    const int64_t trow = (int64_t)min(t, p.table_rows - 1) * (D / 2);
+    norm_rot<D>(p.q + b * p.q_sb + h * p.q_sh, dl, p.cos_tab + trow, p.sin_tab + trow, p.eps, qf);
+    norm_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_tab + trow, p.sin_tab + trow, p.eps, knf);
+    float vnf[8];
+    norm_mix<D>(p.v_new + b * p.vn_sb + h * p.vn_sh, p.ve ? p.ve + b * p.ve_sb + h * p.ve_sh : nullptr, p.gate, dl, p.eps, vnf);
+    vn_packed = pack8(vnf);
+  } else {
+    load_vec_rot<D>(p.q + b * p.q_sb + h * p.q_sh, dl, p.cos_row, p.sin_row, qf);
+    load_vec_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_row, p.sin_row, knf);
+    vn_packed = *reinterpret_cast<const u32x4*>(p.v_new + b * p.vn_sb + h * p.vn_sh + dl);
+  }
   const u32x4 kn_packed = pack8(knf);
 #pragma unroll
   for (int i = 0; i < 8; ++i) qf[i] *= p.scale_log2e;
@@ -377,7 +446,13 @@ extern "C" size_t daisy_decode_workspace_bytes(int B, int H, int D, int n_rows, 
   return (size_t)B * H * ns * (D + 2) * sizeof(float);
 }
 
-// Shared by the two entry points.  With pos_dev set, n_rows is the ring's slot count (it fixes the
+// What daisy_attn_step_fwd adds to a decode launch: the kernel prepares the rows itself.
+struct StepPrep {
+  int pos_host; const float* cos; const float* sin; int table_rows; float eps;
+  const void* ve; const int64_t* ve_strides; const float* gate;
+};
+
+// Shared by the entry points.  With pos_dev set, n_rows is the ring's slot count (it fixes the
 // split count and the grid) and the kernel derives the live rows and the new row's slot from *pos_dev.
 static int decode_launch(const void* q, const int64_t* q_strides,
                          const void* k_new, const int64_t* k_new_strides,
@@ -389,7 +464,7 @@ static int decode_launch(const void* q, const int64_t* q_strides,
                          int B, int H, int D,
                          int n_rows, int new_idx, const int32_t* pos_dev, int write_back,
                          float scale, int nsplit,
-                         void* workspace, size_t workspace_bytes, void* stream) {
+                         void* workspace, size_t workspace_bytes, void* stream, const StepPrep* prep = nullptr) {
   DAISY_CHECK_ARG(q && k_new && v_new && o, "decode: q, k_new, v_new and o must be non-NULL");
   DAISY_CHECK_ARG(q_strides && k_new_strides && v_new_strides && o_strides, "decode: stride arrays must be non-NULL");
   DAISY_CHECK_ARG(B > 0 && H > 0, "decode: B=%d and H=%d must be positive", B, H);
@@ -435,6 +510,13 @@ static int decode_launch(const void* q, const int64_t* q_strides,
   p.nsplit = fast ? resolve_nsplit(B, H, n_rows, nsplit) : 1;
   p.rows_per_split = (n_rows + p.nsplit - 1) / p.nsplit;
   p.pos_dev = pos_dev; p.ring_rows = n_rows;
+  p.pos_host = 0; p.cos_tab = p.sin_tab = nullptr; p.table_rows = 0; p.eps = 0.f;
+  p.ve = nullptr; p.ve_sb = p.ve_sh = 0; p.gate = nullptr;
+  if (prep != nullptr) {
+    p.pos_host = prep->pos_host; p.cos_tab = prep->cos; p.sin_tab = prep->sin; p.table_rows = prep->table_rows;
+    p.eps = prep->eps; p.ve = (const uint16_t*)prep->ve; p.gate = prep->gate;
+    if (prep->ve) { p.ve_sb = prep->ve_strides[0]; p.ve_sh = prep->ve_strides[1]; }
+  }
   p.scale_log2e = scale * kLog2e;
   p.partials = nullptr;
   if (p.nsplit > 1) {
@@ -454,14 +536,16 @@ static int decode_launch(const void* q, const int64_t* q_strides,
   }
   dim3 grid(p.nsplit, H, B);
   if (D == 128) {
-    hipLaunchKernelGGL(decode_kernel<128>, grid, dim3(kDecodeThreads), 0, s, p);
+    if (prep) hipLaunchKernelGGL((decode_kernel<128, true>), grid, dim3(kDecodeThreads), 0, s, p);
+    else hipLaunchKernelGGL((decode_kernel<128, false>), grid, dim3(kDecodeThreads), 0, s, p);
     DAISY_CHECK_LAUNCH("decode_kernel");
     if (p.nsplit > 1) {
       hipLaunchKernelGGL(decode_combine_kernel<128>, dim3(H, B), dim3(128), 0, s, p);
       DAISY_CHECK_LAUNCH("decode_combine_kernel");
     }
   } else {
-    hipLaunchKernelGGL(decode_kernel<64>, grid, dim3(kDecodeThreads), 0, s, p);
+    if (prep) hipLaunchKernelGGL((decode_kernel<64, true>), grid, dim3(kDecodeThreads), 0, s, p);
+    else hipLaunchKernelGGL((decode_kernel<64, false>), grid, dim3(kDecodeThreads), 0, s, p);
     DAISY_CHECK_LAUNCH("decode_kernel");
     if (p.nsplit > 1) {
       hipLaunchKernelGGL(decode_combine_kernel<64>, dim3(H, B), dim3(64), 0, s, p);
@@ -504,4 +588,37 @@ extern "C" int daisy_decode_fwd_at(const void* q, const int64_t* q_strides,
   return decode_launch(q, q_strides, k_new, k_new_strides, v_new, v_new_strides, k_cache, k_cache_strides,
                        v_cache, v_cache_strides, nullptr, nullptr, o, o_strides, B, H, D, ring_rows, 0, pos,
                        /*write_back=*/1, scale, nsplit, workspace, workspace_bytes, stream);
+}
+
+extern "C" int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
+                                   const void* k, const int64_t* k_strides,
+                                   const void* v, const int64_t* v_strides,
+                                   const void* ve, const int64_t* ve_strides, const float* gate,
+                                   const float* cos, const float* sin, int table_rows,
+                                   int pos, const int32_t* pos_dev, float eps,
+                                   void* k_cache, const int64_t* k_cache_strides,
+                                   void* v_cache, const int64_t* v_cache_strides,
+                                   void* o, const int64_t* o_strides,
+                                   int B, int H, int D, int ring_rows,
+                                   float scale, int nsplit,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+  DAISY_CHECK_SUPPORTED(D == 64 || D == 128, "attn_step: head_dim %d not supported (64 or 128)", D);
+  DAISY_CHECK_ARG(k_cache && v_cache && k_cache_strides && v_cache_strides, "attn_step: the ring cache is required");
+  DAISY_CHECK_ARG(ring_rows >= 1, "attn_step: ring_rows=%d must be >= 1", ring_rows);
+  DAISY_CHECK_ARG(cos && sin && table_rows >= 1, "attn_step: the rotary tables are required");
+  DAISY_CHECK_ARG((ve == nullptr) == (gate == nullptr), "attn_step: ve and gate must both be given or both NULL");
+  DAISY_CHECK_ARG(ve == nullptr || ve_strides != nullptr, "attn_step: ve needs ve_strides");
+  DAISY_CHECK_ARG(pos_dev != nullptr || (pos >= 0 && pos < table_rows),
+                  "attn_step: position %d outside the rotary tables (%d rows)", pos, table_rows);
+  auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+  DAISY_CHECK_ARG(al16(ve) && (!ve || (ve_strides[0] % 8 == 0 && ve_strides[1] % 8 == 0)),
+                  "attn_step: ve must be 16-byte aligned with strides that are multiples of 8 elements");
+  StepPrep prep{pos, cos, sin, table_rows, eps, ve, ve_strides, gate};
+  // With the position on the host the live rows and the slot are launch arguments (and the split
+  // count follows the live rows); with the position on the device the kernel derives them.
+  const int n_rows = pos_dev ? ring_rows : (pos + 1 < ring_rows ? pos + 1 : ring_rows);
+  const int new_idx = pos_dev ? 0 : pos % ring_rows;
+  return decode_launch(q, q_strides, k, k_strides, v, v_strides, k_cache, k_cache_strides, v_cache, v_cache_strides,
+                       nullptr, nullptr, o, o_strides, B, H, D, n_rows, new_idx, pos_dev, /*write_back=*/1, scale, nsplit,
+                       workspace, workspace_bytes, stream, &prep);
 }

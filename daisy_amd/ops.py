@@ -181,6 +181,70 @@ def decode_attention_at(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tenso
     return out
 
 
+def attn_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_ring: torch.Tensor, v_ring: torch.Tensor,
+              pos: Union[int, torch.Tensor], *, cos: torch.Tensor, sin: torch.Tensor, eps: float,
+              ve: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+              scale: float = ATTN_SCALE, out: Optional[torch.Tensor] = None,
+              workspace: Optional[torch.Tensor] = None, nsplit: int = 0) -> torch.Tensor:
+    """The attention part of one decode step in one launch (``daisy_attn_step_fwd``).
+
+    ``q``, ``k``, ``v``: the new token's rows of the QKV projection output, bf16 ``[B, H, D]`` views;
+    the kernel normalises them, rotates q and k with row ``pos`` of ``cos``/``sin`` (fp32
+    ``[rows, D/2]``), mixes ``v`` with ``ve [B, H, D]`` through ``gate`` (one fp32), writes the new rows
+    into slot ``pos % W`` of ``k_ring``/``v_ring [B, H, W, D]`` and attends the live rows.  ``pos`` is an
+    int or a one-element int32 device tensor (read when the kernel runs).  Returns ``o [B, H, D]``.
+    """
+    pos_dev = pos if isinstance(pos, torch.Tensor) else None
+    dev = _lib.require_gpu(q, k, v, k_ring, v_ring, cos, sin, ve, gate, pos_dev, out, workspace)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_bf16(name, t, 3)
+    _check_bf16("k_ring", k_ring, 4)
+    _check_bf16("v_ring", v_ring, 4)
+    B, H, D = q.shape
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("q, k, v must all be [B, H, D]")
+    W = k_ring.shape[2]
+    if k_ring.shape != (B, H, W, D) or v_ring.shape != k_ring.shape:
+        raise ValueError(f"k_ring, v_ring must be [{B}, {H}, W, {D}], got {tuple(k_ring.shape)}, {tuple(v_ring.shape)}")
+    for name, t in (("cos", cos), ("sin", sin)):
+        if t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != D // 2 or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous fp32 [rows, {D // 2}] table, got {tuple(t.shape)} {t.dtype}")
+    if pos_dev is not None:
+        if pos_dev.dtype != torch.int32 or pos_dev.numel() != 1:
+            raise ValueError("a device position must be a one-element int32 tensor")
+        live = W
+    else:
+        torch._assert(0 <= pos < cos.shape[0], f"Rotary buffers too small {cos.shape[0]} < {pos + 1}")
+        live = min(int(pos) + 1, W)
+    if (ve is None) != (gate is None):
+        raise ValueError("ve and gate must be given together")
+    if ve is not None:
+        _check_bf16("ve", ve, 3)
+        if ve.shape != q.shape or gate.dtype != torch.float32 or gate.numel() != 1:
+            raise ValueError("ve must be [B, H, D] and gate a one-element fp32 tensor")
+    if out is None:
+        out = torch.empty((B, H, D), dtype=torch.bfloat16, device=dev)
+    else:
+        _check_bf16("out", out, 3)
+    lib = _lib.load()
+    need = int(lib.daisy_decode_workspace_bytes(B, H, D, live, nsplit))
+    if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    d2 = (0, 1)
+    with torch.cuda.device(dev):
+        rc = lib.daisy_attn_step_fwd(
+            q.data_ptr(), _lib.strides(q, d2), k.data_ptr(), _lib.strides(k, d2), v.data_ptr(), _lib.strides(v, d2),
+            _lib.ptr(ve), None if ve is None else _lib.strides(ve, d2), _lib.ptr(gate),
+            cos.data_ptr(), sin.data_ptr(), int(cos.shape[0]),
+            0 if pos_dev is not None else int(pos), _lib.ptr(pos_dev), float(eps),
+            k_ring.data_ptr(), _lib.strides(k_ring, (0, 1, 2)), v_ring.data_ptr(), _lib.strides(v_ring, (0, 1, 2)),
+            out.data_ptr(), _lib.strides(out, d2), B, H, D, int(W), float(scale), int(nsplit),
+            _lib.ptr(workspace), ws_bytes, _lib.current_stream(dev))
+    _lib.check(rc, "daisy_attn_step_fwd")
+    return out
+
+
 def kda_workspace_bytes(B: int, T: int, H: int, Dk: int, Dv: int, chunk: int = 64) -> int:
     return int(_lib.load().daisy_kda_workspace_bytes(B, T, H, Dk, Dv, chunk))
 

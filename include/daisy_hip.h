@@ -145,6 +145,32 @@ int daisy_decode_fwd_at(const void* q, const int64_t* q_strides,
                         float scale, int nsplit,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* The attention part of one decode step in a single launch: what CausalSelfAttention.step
+ * (models/daisy/attention.py:181-202) does between its two projections.  q, k, v are the rows
+ * of the QKV projection output for the new token, bf16 [B, H, D] with {batch, head} strides
+ * (three views of one [B, 3H, D] tensor).  The kernel applies the weightless RMS norm to all
+ * three (eps as in daisy_qkv_prep_fwd), rotates q and k with row `pos` of the tables
+ * (cos, sin: fp32 [table_rows, D/2]), mixes v with ve through *gate when both are given, writes
+ * the new K and V rows into slot pos % ring_rows of the ring cache [B, H, ring_rows, D] and
+ * attends the min(pos + 1, ring_rows) live rows.  The position is `pos` when pos_dev is NULL,
+ * else the int32 that pos_dev points at, read when the kernel runs (see daisy_decode_fwd_at;
+ * the workspace is then sized for ring_rows, otherwise for the live rows).
+ * Same results as daisy_qkv_prep_fwd followed by daisy_decode_fwd up to the order of the
+ * fp32 sums inside the norm.  D is 64 or 128.
+ */
+int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
+                        const void* k, const int64_t* k_strides,
+                        const void* v, const int64_t* v_strides,
+                        const void* ve, const int64_t* ve_strides, const float* gate,
+                        const float* cos, const float* sin, int table_rows,
+                        int pos, const int32_t* pos_dev, float eps,
+                        void* k_cache, const int64_t* k_cache_strides,
+                        void* v_cache, const int64_t* v_cache_strides,
+                        void* o, const int64_t* o_strides,
+                        int B, int H, int D, int ring_rows,
+                        float scale, int nsplit,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Kernel 3: chunked Kimi Delta Attention forward.
  *

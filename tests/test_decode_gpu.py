@@ -121,6 +121,57 @@ def test_decode_at_device_position_matches_oracle(B, H, D, W, nsplit):
             assert torch.equal(o, o_host), "device- and host-position entry points differ on a full ring"
 
 
+@pytest.mark.parametrize("B,H,D,W,mix,nsplit", [(2, 3, 128, 64, True, 0), (1, 2, 128, 1024, False, 4), (3, 2, 64, 200, True, 3),
+                                                (16, 8, 128, 4096, True, 0)])
+def test_attn_step_prepares_rows_and_attends_in_one_launch(B, H, D, W, mix, nsplit):
+    """daisy_attn_step_fwd against the oracle's chain (norm, RoPE, value-embedding mix on bf16
+    tensors, then fp32 attention over the ring with the new rows in slot t % W), with the position
+    as a launch argument and in device memory; and against the two-kernel path."""
+    from daisy_amd.functional import NORM_EPS_BF16
+    g = torch.Generator().manual_seed(W + D + B)
+    cos, sin = oracle.rope_tables(D, 6 * W + 8)
+    g_logit = -0.4
+    gate = torch.sigmoid(torch.tensor(g_logit)).bfloat16().float().reshape(1).cuda() if mix else None
+    pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for t in (0, 3, W - 1, W, 5 * W + 3):
+        say(f"attn_step case B{B} H{H} D{D} W{W} mix{mix} nsplit{nsplit} t{t}")
+        kc, vc = (torch.randn(B, H, W, D, generator=g).bfloat16() for _ in range(2))
+        qkv = (torch.randn(B, 3 * H, D, generator=g) * 1.7).bfloat16()
+        q, k, v = qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:]
+        ve = torch.randn(B, H, D, generator=g).bfloat16() if mix else None
+        qn = oracle.apply_rope(oracle.rms_norm(q)[:, None], cos[t:t + 1], sin[t:t + 1])[:, 0]
+        kn = oracle.apply_rope(oracle.rms_norm(k)[:, None], cos[t:t + 1], sin[t:t + 1])[:, 0]
+        vn = oracle.rms_norm(v)
+        if mix:
+            vn = oracle.attention._mix_ve(vn, ve, g_logit)
+        n_rows, slot = min(t + 1, W), t % W
+        k_exp, v_exp = kc.clone(), vc.clone()
+        k_exp[:, :, slot], v_exp[:, :, slot] = kn, vn
+        ref = _ref_decode(qn, k_exp[:, :, :n_rows], v_exp[:, :, :n_rows])
+        qkv_d = qkv.cuda()
+        rows = (qkv_d[:, :H], qkv_d[:, H:2 * H], qkv_d[:, 2 * H:])
+        kw = dict(cos=cos.cuda(), sin=sin.cuda(), eps=NORM_EPS_BF16, ve=None if ve is None else ve.cuda(), gate=gate, nsplit=nsplit)
+        outs = []
+        for where in ("host", "device"):
+            dk, dv = kc.cuda(), vc.cuda()
+            pos.fill_(t)
+            o = ops.attn_step(*rows, dk, dv, t if where == "host" else pos, **kw)
+            assert_close_bf16(o, ref, f"o, position on the {where}, t={t}")
+            # the stored rows: the bf16 chain's, except where an fp32 sum sits on a rounding boundary
+            for got, want, name in ((dk, k_exp, "K"), (dv, v_exp, "V")):
+                assert torch.equal(got.cpu()[:, :, :slot], want[:, :, :slot]) and torch.equal(got.cpu()[:, :, slot + 1:], want[:, :, slot + 1:])
+                row, row_ref = got.cpu()[:, :, slot].float(), want[:, :, slot].float()
+                assert (row - row_ref).abs().max() <= 4e-2 and (row != row_ref).float().mean() <= 5e-3, f"new {name} row, t={t}"
+            outs.append((o, dk, dv))
+        assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2]), "host and device position store different rows"
+        # the two-kernel path: same rows up to the order of the sums in the norm, same attention
+        q2, k2, v2 = ops.qkv_prep(*(r.unsqueeze(1) for r in rows), eps=NORM_EPS_BF16, cos=kw["cos"], sin=kw["sin"], pos0=t,
+                                  ve=None if ve is None else kw["ve"].unsqueeze(1), gate=gate)
+        dk, dv = kc.cuda(), vc.cuda()
+        o2 = ops.decode_attention(q2[:, 0], k2[:, 0], v2[:, 0], dk, dv, n_rows=n_rows, new_idx=slot, write_back=True, nsplit=nsplit)
+        assert_close_bf16(outs[0][0], o2.float(), f"one launch vs two, t={t}", max_abs=8e-3, mean_abs=3e-4)
+
+
 def test_decode_rejects_bad_arguments():
     z = torch.zeros(1, 1, 128, dtype=torch.bfloat16, device="cuda:0")
     rows = torch.zeros(1, 1, 4, 128, dtype=torch.bfloat16, device="cuda:0")

@@ -131,9 +131,20 @@ def check(rc: int, what: str) -> None:
         raise RuntimeError(f"{what} failed (code {rc}): {msg}")
 
 
+_STRIDE_ARRAYS: dict = {}
+
+
 def strides(t: torch.Tensor, dims) -> ctypes.Array:
-    """Element strides of the given dims as an int64 C array."""
-    return (c_int64 * len(dims))(*[t.stride(d) for d in dims])
+    """Element strides of the given dims as an int64 C array (read-only for the callee, so equal
+    stride tuples share one array: decode loops ask for the same few over and over)."""
+    st = t.stride()
+    key = tuple(st[d] for d in dims)
+    arr = _STRIDE_ARRAYS.get(key)
+    if arr is None:
+        if len(_STRIDE_ARRAYS) > 4096:
+            _STRIDE_ARRAYS.clear()
+        arr = _STRIDE_ARRAYS[key] = (c_int64 * len(key))(*key)
+    return arr
 
 
 def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -159,5 +170,29 @@ def require_gpu(*tensors: Optional[torch.Tensor]) -> torch.device:
     return dev
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream(dev: torch.device) -> int:
+    """The ``hipStream_t`` of torch's current stream on ``dev`` as an integer."""
+    if _raw_stream is not None and dev.index is not None:
+        return _raw_stream(dev.index)
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def on_device(dev: torch.device):
+    """Context that makes ``dev`` the current device for the launch; free when it already is."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(dev)

@@ -66,7 +66,7 @@ def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *,
     w = 0 if window is None else int(window)
     flags = _lib.PREFILL_ROTATE_K_IN_KERNEL if rotate_k_in_kernel else 0
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = lib.daisy_prefill_fwd(
             q.data_ptr(), _lib.strides(q, (0, 1, 2)),
             k.data_ptr(), _lib.strides(k, (0, 1, 2)),
@@ -117,7 +117,7 @@ def decode_attention(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
     if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = lib.daisy_decode_fwd(
             q.data_ptr(), _lib.strides(q, (0, 1)),
             k_new.data_ptr(), _lib.strides(k_new, (0, 1)),
@@ -167,7 +167,7 @@ def decode_attention_at(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tenso
     if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = lib.daisy_decode_fwd_at(
             q.data_ptr(), _lib.strides(q, (0, 1)),
             k_new.data_ptr(), _lib.strides(k_new, (0, 1)),
@@ -232,7 +232,7 @@ def attn_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_ring: torch.T
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     d2 = (0, 1)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = lib.daisy_attn_step_fwd(
             q.data_ptr(), _lib.strides(q, d2), k.data_ptr(), _lib.strides(k, d2), v.data_ptr(), _lib.strides(v, d2),
             _lib.ptr(ve), None if ve is None else _lib.strides(ve, d2), _lib.ptr(gate),
@@ -279,7 +279,7 @@ def kda_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
     if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = lib.daisy_kda_chunk_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(),
             g.data_ptr(), 1 if g.dtype == torch.bfloat16 else 0, beta.data_ptr(),
@@ -328,7 +328,7 @@ def kda_recurrent_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torc
     else:
         final = torch.empty((B, H, Dk, Dv), dtype=torch.float32, device=dev) if output_final_state else None
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = lib.daisy_kda_recurrent_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(),
             g.data_ptr(), 1 if g.dtype == torch.bfloat16 else 0, beta.data_ptr(),
@@ -365,7 +365,7 @@ def kda_gate_fwd(g: torch.Tensor, A_log: torch.Tensor, head_k_dim: int,
     out = torch.empty((*g.shape[:-1], H, head_k_dim), dtype=g.dtype, device=dev)
     rows = gc.numel() // last
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = lib.daisy_kda_gate_fwd(gc.data_ptr(), a.data_ptr(), _lib.ptr(bias), out.data_ptr(),
                                     rows, H, head_k_dim, 1 if g.dtype == torch.bfloat16 else 0,
                                     float(beta), float(threshold), _lib.current_stream(dev))
@@ -434,7 +434,7 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
            _lib.ptr(ve), None if ve is None else _lib.strides(ve, d3), _lib.ptr(gate), _lib.ptr(cos), _lib.ptr(sin))
     outs = (qo.data_ptr(), _lib.strides(qo, d3), ko.data_ptr(), _lib.strides(ko, d3), vo.data_ptr(), _lib.strides(vo, d3),
             B, T, H, D, float(eps))
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         if pos_dev is None:
             rc = lib.daisy_qkv_prep_fwd(*ins, int(pos0), *outs, _lib.current_stream(dev))
         else:
@@ -455,7 +455,7 @@ def probe_matrix_rate(with_vector_mix: bool, iters: int = 50000, workgroups: int
     lib = _lib.load()
     flop = ctypes.c_double(0.0)
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         stream = _lib.current_stream(dev)
         rc = lib.daisy_probe_matrix_rate(int(with_vector_mix), workgroups, max(iters // 10, 1), sink.data_ptr(),
                                          ticks.data_ptr(), ctypes.byref(flop), stream)   # warm-up
@@ -482,7 +482,7 @@ def probe_read_rate(gib: int = 2, workgroups: int = 8192, repeats: int = 5, devi
     sink = torch.empty(4096, dtype=torch.int32, device=dev)
     lib = _lib.load()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         stream = _lib.current_stream(dev)
         _lib.check(lib.daisy_probe_read_rate(buf.data_ptr(), nbytes, workgroups, sink.data_ptr(), stream), "daisy_probe_read_rate")
         start.record()
@@ -530,7 +530,7 @@ def short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
     else:
         new_cache = torch.empty(B, C, K, dtype=torch.bfloat16, device=dev) if output_final_state else None
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = lib.daisy_short_conv_fwd(x.data_ptr(), _lib.strides(x, (0, 1)), w.data_ptr(), _lib.ptr(bias), _lib.ptr(cache),
                                       y.data_ptr(), _lib.strides(y, (0, 1)), _lib.ptr(new_cache),
                                       B, T, C, K, 1 if activation == "silu" else 0, _lib.current_stream(dev))
@@ -549,7 +549,7 @@ def gated_rmsnorm(x: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps
     out = torch.empty_like(xc)
     D = x.shape[-1]
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         rc = lib.daisy_gated_rmsnorm_fwd(xc.data_ptr(), gc.data_ptr(), wc.data_ptr(), out.data_ptr(),
                                          xc.numel() // D, D, float(eps), _lib.current_stream(dev))
     _lib.check(rc, "daisy_gated_rmsnorm_fwd")

@@ -54,7 +54,7 @@ SIGNATURES = {
         c_void_p, _I64P, c_void_p,                              # ve, ve strides, gate
         c_void_p, c_void_p, c_int,                              # cos, sin, table_rows
         c_int, c_void_p, c_float,                               # pos, pos_dev, eps
-        c_void_p, _I64P, c_void_p, _I64P,                       # k_cache, v_cache (+strides)
+        c_void_p, _I64P, c_void_p, _I64P, c_int,                # k_cache, v_cache (+strides), cache_is_f16
         c_void_p, _I64P,                                        # o (+strides)
         c_int, c_int, c_int, c_int,                             # B, H, D, ring_rows
         c_float, c_int,                                         # scale, nsplit

@@ -324,11 +324,12 @@ class CausalSelfAttention(nn.Module):
         torch._assert(x.size(1) == 1, "step() requires single position only")
         fused = self._fused_prep_ok()
         ring = k_ctx if isinstance(k_ctx, RingContext) else None
-        in_ring = fused and ring is not None and ring.k.dtype == torch.bfloat16 and window == ring.W
+        # the one-launch step streams a bf16 ring, or an fp16 one (the reference generator's default)
+        in_ring = fused and ring is not None and ring.k.dtype in (torch.bfloat16, torch.float16) and window == ring.W
         if isinstance(pos, Tensor):
             if not in_ring:
                 raise ValueError("a device-side position needs the fused kernels (bf16 weights, head dim 64 or 128) "
-                                 "and the RingContext of a bf16 KVCache whose size equals the window")
+                                 "and the RingContext of a bf16 or fp16 KVCache whose size equals the window")
             return self._step_in_ring(x, ring, pos, ve)
         if in_ring and pos == ring.t:
             return self._step_in_ring(x, ring, pos, ve)
@@ -398,4 +399,7 @@ class CausalSelfAttention(nn.Module):
         if isinstance(pos, Tensor):
             return y, None, None
         slot = pos % ring.W
-        return y, ring.k[:, :, slot, :].unsqueeze(1), ring.v[:, :, slot, :].unsqueeze(1)
+        k_new, v_new = ring.k[:, :, slot, :].unsqueeze(1), ring.v[:, :, slot, :].unsqueeze(1)
+        if k_new.dtype != y.dtype:      # an fp16 ring: the rows go back in the model's dtype, as the reference's do
+            k_new, v_new = k_new.to(y.dtype), v_new.to(y.dtype)
+        return y, k_new, v_new

@@ -134,7 +134,7 @@ def _walk_step(model, token_ids: Tensor, cache: KVCache, pos) -> Tensor:
     skip_map, skip_weights = model.skip_map, model.skip_weights
     ve_map = _value_embeddings(model, token_ids)
     window = getattr(model, "attn_window_size", cache.W)
-    in_place = cache.dtype == torch.bfloat16
+    in_place = cache.dtype in (torch.bfloat16, torch.float16)
     skip_connections = []
     for i in range(L):
         if i in skip_map:
@@ -166,14 +166,14 @@ class GraphedStep:
     device counter that the pre-attention and decode kernels read when they run and that the last
     node of the graph increments.
 
-    Needs a bf16 cache whose ring size equals the model's attention window and attention layers
+    Needs a bf16 or fp16 cache whose ring size equals the model's attention window and attention layers
     that take the ring in place with the fused pre-attention kernel (otherwise recording raises).
     The returned logits are a buffer that the next call overwrites.  Rotary tables are fixed when
     the step is recorded: positions up to their row count can be replayed.
     """
 
     def __init__(self, model, cache: KVCache):
-        torch._assert(cache.dtype == torch.bfloat16, "a recorded step needs a bf16 cache")
+        torch._assert(cache.dtype in (torch.bfloat16, torch.float16), "a recorded step needs a bf16 or fp16 cache")
         self.model, self.cache = model, cache
         dev = cache.k.device
         self.tokens = torch.zeros(cache.B, dtype=torch.long, device=dev)

@@ -129,6 +129,33 @@ __device__ __forceinline__ void norm_mix(const uint16_t* vec, const uint16_t* ve
   }
 }
 
+// Cache rows in fp16 (the reference's default cache dtype, inference/generate.py:62): eight
+// values of a 16-byte piece to floats and back.  bf16 rows convert to fp16 without loss as long as
+// they are in fp16's normal range, which normalised keys and values are.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void unpack8_f16(const u32x4& r, float* f) {
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const f16x2 h = __builtin_bit_cast(f16x2, w[i]);
+    f[2 * i] = (float)h[0];
+    f[2 * i + 1] = (float)h[1];
+  }
+}
+__device__ __forceinline__ u32x4 pack8_f16(const float* f) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const f16x2 h = {(_Float16)f[2 * i], (_Float16)f[2 * i + 1]};
+    w[i] = __builtin_bit_cast(uint32_t, h);
+  }
+  return u32x4{w[0], w[1], w[2], w[3]};
+}
+template <bool F16>
+__device__ __forceinline__ void unpack8_cache(const u32x4& r, float* f) {
+  if constexpr (F16) unpack8_f16(r, f); else unpack8(r, f);
+}
+
 struct SoftmaxState {
   float m, l;
   float acc[8];
@@ -147,7 +174,8 @@ __device__ __forceinline__ void merge_state(SoftmaxState& a, const SoftmaxState&
 
 // PREP: q, k_new and v_new are rows of the QKV projection output; the kernel normalises, rotates
 // and mixes them itself (every workgroup of a (batch, head) redoes these few hundred flops).
-template <int D, bool PREP>
+// F16C: the cache rows are fp16 (the new rows are converted on their way in).
+template <int D, bool PREP, bool F16C = false>
 __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) {
   constexpr int LPR = D / 8;        // lanes per cache row
   constexpr int RPW = 64 / LPR;     // rows per wavefront load
@@ -168,13 +196,14 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
     norm_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_tab + trow, p.sin_tab + trow, p.eps, knf);
     float vnf[8];
     norm_mix<D>(p.v_new + b * p.vn_sb + h * p.vn_sh, p.ve ? p.ve + b * p.ve_sb + h * p.ve_sh : nullptr, p.gate, dl, p.eps, vnf);
-    vn_packed = pack8(vnf);
+    vn_packed = F16C ? pack8_f16(vnf) : pack8(vnf);
   } else {
+    static_assert(!F16C, "fp16 cache rows come with the kernel-side preparation only");
     load_vec_rot<D>(p.q + b * p.q_sb + h * p.q_sh, dl, p.cos_row, p.sin_row, qf);
     load_vec_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_row, p.sin_row, knf);
     vn_packed = *reinterpret_cast<const u32x4*>(p.v_new + b * p.vn_sb + h * p.vn_sh + dl);
   }
-  const u32x4 kn_packed = pack8(knf);
+  const u32x4 kn_packed = F16C ? pack8_f16(knf) : pack8(knf);
 #pragma unroll
   for (int i = 0; i < 8; ++i) qf[i] *= p.scale_log2e;
 
@@ -226,7 +255,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
         }
       }
       float kf[8];
-      unpack8(kr[u], kf);
+      unpack8_cache<F16C>(kr[u], kf);
       float d = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) d = fmaf(qf[i], kf[i], d);
@@ -247,7 +276,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
       const float pu = fast_exp2(s[u] - mu);
       st.l += pu;
       float vf[8];
-      unpack8(vr[u], vf);
+      unpack8_cache<F16C>(vr[u], vf);
 #pragma unroll
       for (int i = 0; i < 8; ++i) st.acc[i] = fmaf(pu, vf[i], st.acc[i]);
     }
@@ -450,6 +479,7 @@ extern "C" size_t daisy_decode_workspace_bytes(int B, int H, int D, int n_rows, 
 struct StepPrep {
   int pos_host; const float* cos; const float* sin; int table_rows; float eps;
   const void* ve; const int64_t* ve_strides; const float* gate;
+  int cache_f16;
 };
 
 // Shared by the entry points.  With pos_dev set, n_rows is the ring's slot count (it fixes the
@@ -536,7 +566,8 @@ static int decode_launch(const void* q, const int64_t* q_strides,
   }
   dim3 grid(p.nsplit, H, B);
   if (D == 128) {
-    if (prep) hipLaunchKernelGGL((decode_kernel<128, true>), grid, dim3(kDecodeThreads), 0, s, p);
+    if (prep && prep->cache_f16) hipLaunchKernelGGL((decode_kernel<128, true, true>), grid, dim3(kDecodeThreads), 0, s, p);
+    else if (prep) hipLaunchKernelGGL((decode_kernel<128, true>), grid, dim3(kDecodeThreads), 0, s, p);
     else hipLaunchKernelGGL((decode_kernel<128, false>), grid, dim3(kDecodeThreads), 0, s, p);
     DAISY_CHECK_LAUNCH("decode_kernel");
     if (p.nsplit > 1) {
@@ -544,7 +575,8 @@ static int decode_launch(const void* q, const int64_t* q_strides,
       DAISY_CHECK_LAUNCH("decode_combine_kernel");
     }
   } else {
-    if (prep) hipLaunchKernelGGL((decode_kernel<64, true>), grid, dim3(kDecodeThreads), 0, s, p);
+    if (prep && prep->cache_f16) hipLaunchKernelGGL((decode_kernel<64, true, true>), grid, dim3(kDecodeThreads), 0, s, p);
+    else if (prep) hipLaunchKernelGGL((decode_kernel<64, true>), grid, dim3(kDecodeThreads), 0, s, p);
     else hipLaunchKernelGGL((decode_kernel<64, false>), grid, dim3(kDecodeThreads), 0, s, p);
     DAISY_CHECK_LAUNCH("decode_kernel");
     if (p.nsplit > 1) {
@@ -597,7 +629,7 @@ extern "C" int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
                                    const float* cos, const float* sin, int table_rows,
                                    int pos, const int32_t* pos_dev, float eps,
                                    void* k_cache, const int64_t* k_cache_strides,
-                                   void* v_cache, const int64_t* v_cache_strides,
+                                   void* v_cache, const int64_t* v_cache_strides, int cache_is_f16,
                                    void* o, const int64_t* o_strides,
                                    int B, int H, int D, int ring_rows,
                                    float scale, int nsplit,
@@ -613,7 +645,7 @@ extern "C" int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
   auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
   DAISY_CHECK_ARG(al16(ve) && (!ve || (ve_strides[0] % 8 == 0 && ve_strides[1] % 8 == 0)),
                   "attn_step: ve must be 16-byte aligned with strides that are multiples of 8 elements");
-  StepPrep prep{pos, cos, sin, table_rows, eps, ve, ve_strides, gate};
+  StepPrep prep{pos, cos, sin, table_rows, eps, ve, ve_strides, gate, cache_is_f16 != 0};
   // With the position on the host the live rows and the slot are launch arguments (and the split
   // count follows the live rows); with the position on the device the kernel derives them.
   const int n_rows = pos_dev ? ring_rows : (pos + 1 < ring_rows ? pos + 1 : ring_rows);

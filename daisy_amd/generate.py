@@ -119,8 +119,10 @@ class Generator:
         first = next(a for a in attn if a is not None)
         self.cache = KVCache(L=len(layers), B=1, H=first.num_heads, W=window, D=first.head_dim,
                              device=self.device, dtype=dtype)
-        # In-place decode: every layer must understand ring handles and the ring must be bf16.
-        self.use_ring_context = dtype == torch.bfloat16 and all(isinstance(a, CausalSelfAttention) for a in attn)
+        # In-place decode: every attention layer must understand ring handles; the ring is bf16, or
+        # fp16 (the reference's default, which the decode kernel reads and appends to as it is).
+        self.use_ring_context = (dtype in (torch.bfloat16, torch.float16)
+                                 and all(a is None or isinstance(a, CausalSelfAttention) for a in attn))
         self._rings = [self.cache.ring(i) for i in range(len(layers))] if self.use_ring_context else None
         # record_steps: the decode step is recorded once as a HIP graph and replayed per token
         # (daisy_amd.core.GraphedStep walks the model's layers itself, so the model needs the

@@ -191,15 +191,20 @@ def attn_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_ring: torch.T
     ``q``, ``k``, ``v``: the new token's rows of the QKV projection output, bf16 ``[B, H, D]`` views;
     the kernel normalises them, rotates q and k with row ``pos`` of ``cos``/``sin`` (fp32
     ``[rows, D/2]``), mixes ``v`` with ``ve [B, H, D]`` through ``gate`` (one fp32), writes the new rows
-    into slot ``pos % W`` of ``k_ring``/``v_ring [B, H, W, D]`` and attends the live rows.  ``pos`` is an
+    into slot ``pos % W`` of ``k_ring``/``v_ring [B, H, W, D]`` (bf16 or fp16) and attends the live rows.  ``pos`` is an
     int or a one-element int32 device tensor (read when the kernel runs).  Returns ``o [B, H, D]``.
     """
     pos_dev = pos if isinstance(pos, torch.Tensor) else None
     dev = _lib.require_gpu(q, k, v, k_ring, v_ring, cos, sin, ve, gate, pos_dev, out, workspace)
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_bf16(name, t, 3)
-    _check_bf16("k_ring", k_ring, 4)
-    _check_bf16("v_ring", v_ring, 4)
+    if k_ring.dtype == torch.float16 and v_ring.dtype == torch.float16 and k_ring.dim() == 4 and k_ring.stride(-1) == 1 \
+            and v_ring.stride(-1) == 1:
+        ring_f16 = True       # the reference generator's default cache dtype
+    else:
+        ring_f16 = False
+        _check_bf16("k_ring", k_ring, 4)
+        _check_bf16("v_ring", v_ring, 4)
     B, H, D = q.shape
     if k.shape != q.shape or v.shape != q.shape:
         raise ValueError("q, k, v must all be [B, H, D]")
@@ -239,6 +244,7 @@ def attn_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_ring: torch.T
             cos.data_ptr(), sin.data_ptr(), int(cos.shape[0]),
             0 if pos_dev is not None else int(pos), _lib.ptr(pos_dev), float(eps),
             k_ring.data_ptr(), _lib.strides(k_ring, (0, 1, 2)), v_ring.data_ptr(), _lib.strides(v_ring, (0, 1, 2)),
+            1 if ring_f16 else 0,
             out.data_ptr(), _lib.strides(out, d2), B, H, D, int(W), float(scale), int(nsplit),
             _lib.ptr(workspace), ws_bytes, _lib.current_stream(dev))
     _lib.check(rc, "daisy_attn_step_fwd")

@@ -156,7 +156,9 @@ int daisy_decode_fwd_at(const void* q, const int64_t* q_strides,
  * else the int32 that pos_dev points at, read when the kernel runs (see daisy_decode_fwd_at;
  * the workspace is then sized for ring_rows, otherwise for the live rows).
  * Same results as daisy_qkv_prep_fwd followed by daisy_decode_fwd up to the order of the
- * fp32 sums inside the norm.  D is 64 or 128.
+ * fp32 sums inside the norm.  D is 64 or 128.  cache_is_f16: the ring holds fp16 rows (the
+ * default cache dtype of the reference's Generator, inference/generate.py:62) instead of bf16;
+ * the new rows are converted on their way in, which loses nothing for normalised rows.
  */
 int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
                         const void* k, const int64_t* k_strides,
@@ -165,7 +167,7 @@ int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
                         const float* cos, const float* sin, int table_rows,
                         int pos, const int32_t* pos_dev, float eps,
                         void* k_cache, const int64_t* k_cache_strides,
-                        void* v_cache, const int64_t* v_cache_strides,
+                        void* v_cache, const int64_t* v_cache_strides, int cache_is_f16,
                         void* o, const int64_t* o_strides,
                         int B, int H, int D, int ring_rows,
                         float scale, int nsplit,

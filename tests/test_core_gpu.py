@@ -255,7 +255,7 @@ def test_recorded_step_replays_match_eager_steps(window, T, n_steps):
             _close(graphed(ids[:, T + s]), want, f"after reset, replay {s} logits", tol=1e-2)
         # the walk cannot be recorded over chronological views
         with pytest.raises(Exception):
-            core.GraphedStep(model, KVCache(4, B, 2, window, 128, DEV, torch.float16))
+            core.GraphedStep(model, KVCache(4, B, 2, window, 128, DEV, torch.float32))
 
 
 def test_recorded_step_with_a_kda_layer():
@@ -308,6 +308,13 @@ def test_generator_single_sequence_with_recorded_steps():
             say(f"prompt of {T}: {want.numel()} tokens, recorded equal: {torch.equal(want, got)}")
             assert torch.equal(want, got)
             assert torch.equal(plain.history, recorded.history)
+        # the reference's default cache dtype (fp16): the ring is streamed and appended to in place
+        # all the same, and holds the same values (bf16 rows convert to fp16 without loss)
+        kw.pop("dtype")
+        default = Generator(model, **kw)
+        assert default.cache.dtype == torch.float16 and default.use_ring_context
+        assert torch.equal(torch.cat(list(default.generate(ids, 24))), want)
+        assert torch.equal(default.cache.k.float(), plain.cache.k.float()) and torch.equal(default.cache.v.float(), plain.cache.v.float())
 
 
 def test_generator_generate_batch():

@@ -121,12 +121,14 @@ def test_decode_at_device_position_matches_oracle(B, H, D, W, nsplit):
             assert torch.equal(o, o_host), "device- and host-position entry points differ on a full ring"
 
 
+@pytest.mark.parametrize("ring_dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,H,D,W,mix,nsplit", [(2, 3, 128, 64, True, 0), (1, 2, 128, 1024, False, 4), (3, 2, 64, 200, True, 3),
                                                 (16, 8, 128, 4096, True, 0)])
-def test_attn_step_prepares_rows_and_attends_in_one_launch(B, H, D, W, mix, nsplit):
+def test_attn_step_prepares_rows_and_attends_in_one_launch(B, H, D, W, mix, nsplit, ring_dtype):
     """daisy_attn_step_fwd against the oracle's chain (norm, RoPE, value-embedding mix on bf16
     tensors, then fp32 attention over the ring with the new rows in slot t % W), with the position
-    as a launch argument and in device memory; and against the two-kernel path."""
+    as a launch argument and in device memory; and against the two-kernel path.  The ring is bf16
+    or fp16 (the reference generator's default cache dtype; bf16 rows convert to it without loss)."""
     from daisy_amd.functional import NORM_EPS_BF16
     g = torch.Generator().manual_seed(W + D + B)
     cos, sin = oracle.rope_tables(D, 6 * W + 8)
@@ -135,7 +137,8 @@ def test_attn_step_prepares_rows_and_attends_in_one_launch(B, H, D, W, mix, nspl
     pos = torch.zeros(1, dtype=torch.int32, device="cuda")
     for t in (0, 3, W - 1, W, 5 * W + 3):
         say(f"attn_step case B{B} H{H} D{D} W{W} mix{mix} nsplit{nsplit} t{t}")
-        kc, vc = (torch.randn(B, H, W, D, generator=g).bfloat16() for _ in range(2))
+        # (values below fp16's normal range would not survive the conversion of the random fill)
+        kc, vc = (torch.randn(B, H, W, D, generator=g).bfloat16().to(ring_dtype).bfloat16() for _ in range(2))
         qkv = (torch.randn(B, 3 * H, D, generator=g) * 1.7).bfloat16()
         q, k, v = qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:]
         ve = torch.randn(B, H, D, generator=g).bfloat16() if mix else None
@@ -153,14 +156,17 @@ def test_attn_step_prepares_rows_and_attends_in_one_launch(B, H, D, W, mix, nspl
         kw = dict(cos=cos.cuda(), sin=sin.cuda(), eps=NORM_EPS_BF16, ve=None if ve is None else ve.cuda(), gate=gate, nsplit=nsplit)
         outs = []
         for where in ("host", "device"):
-            dk, dv = kc.cuda(), vc.cuda()
+            dk, dv = kc.cuda().to(ring_dtype), vc.cuda().to(ring_dtype)
             pos.fill_(t)
             o = ops.attn_step(*rows, dk, dv, t if where == "host" else pos, **kw)
             assert_close_bf16(o, ref, f"o, position on the {where}, t={t}")
             # the stored rows: the bf16 chain's, except where an fp32 sum sits on a rounding boundary
             for got, want, name in ((dk, k_exp, "K"), (dv, v_exp, "V")):
-                assert torch.equal(got.cpu()[:, :, :slot], want[:, :, :slot]) and torch.equal(got.cpu()[:, :, slot + 1:], want[:, :, slot + 1:])
-                row, row_ref = got.cpu()[:, :, slot].float(), want[:, :, slot].float()
+                assert got.dtype == ring_dtype
+                got = got.float().cpu()
+                want = want.float()
+                assert torch.equal(got[:, :, :slot], want[:, :, :slot]) and torch.equal(got[:, :, slot + 1:], want[:, :, slot + 1:])
+                row, row_ref = got[:, :, slot], want[:, :, slot]
                 assert (row - row_ref).abs().max() <= 4e-2 and (row != row_ref).float().mean() <= 5e-3, f"new {name} row, t={t}"
             outs.append((o, dk, dv))
         assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][2], outs[1][2]), "host and device position store different rows"

@@ -98,7 +98,7 @@ def penalise_repeats(logits: Tensor, recent: Tensor, strength: Tensor, _one: Opt
 class Generator:
     def __init__(self, model, window, seed, device=None, dtype=torch.float16, max_seq_len: int = 65536,
                  temperature=1.0, top_k=None, top_p=None, repetition_penalty=1.0, eos_token_id=None,
-                 record_steps: bool = False):
+                 record_steps: bool = False, direct_prefill: bool = False):
         eos = eos_token_id if eos_token_id is not None else getattr(model, "eos_token_id", None)
         if eos is None:
             raise AssertionError("eos_token_id must be given or be an attribute of the model")
@@ -129,6 +129,10 @@ class Generator:
         # attributes of the reference's DaisyCore, a bf16 cache and this package's attention).
         self.record_steps = bool(record_steps)
         self._recorded_step = None
+        # direct_prefill: the prompt runs through daisy_amd.core.prefill instead of model.prefill: no
+        # T x T mask, no [2, L, B, H, T, D] stack, every layer's keys and values go straight into
+        # the cache (same requirements on the model as record_steps).
+        self.direct_prefill = bool(direct_prefill)
 
         torch.manual_seed(seed)
         self._tokens = torch.empty(256, dtype=torch.long, device=self.device)
@@ -181,8 +185,12 @@ class Generator:
         returns the logits of its last position, ``[1, vocab]``."""
         n = prompt_ids.numel()
         assert n > 0
-        logits, kv = self.model.prefill(prompt_ids.view(1, n))
-        self.cache.bulk_write_packed(kv, n)
+        if self.direct_prefill:
+            from . import core
+            logits, _ = core.prefill(self.model, prompt_ids.view(1, n), self.cache)
+        else:
+            logits, kv = self.model.prefill(prompt_ids.view(1, n))
+            self.cache.bulk_write_packed(kv, n)
         self._remember(prompt_ids)
         return self._trim(logits)
 

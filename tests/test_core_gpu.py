@@ -294,13 +294,14 @@ def test_recorded_step_with_a_kda_layer():
 
 
 def test_generator_single_sequence_with_recorded_steps():
-    """Generator.generate (the reference's one-sequence loop) with record_steps: the same tokens as
-    with steps launched kernel by kernel, for two prompts in a row on one generator (one recording)."""
+    """Generator.generate (the reference's one-sequence loop) with record_steps and direct_prefill: the
+    same tokens as through model.prefill + bulk_write_packed and steps launched kernel by kernel, for
+    two prompts in a row on one generator (one recording)."""
     from daisy_amd import Generator
     with torch.no_grad():
         model = _Core().to(DEV)
         kw = dict(window=model.window_size, seed=3, device=torch.device(DEV), dtype=torch.bfloat16, temperature=0.0)
-        plain, recorded = Generator(model, **kw), Generator(model, record_steps=True, **kw)
+        plain, recorded = Generator(model, **kw), Generator(model, record_steps=True, direct_prefill=True, **kw)
         for seed, T in ((13, 30), (14, 55)):      # the second prompt is longer than the ring
             ids = torch.randint(2, 96, (T,), generator=torch.Generator().manual_seed(seed)).to(DEV)
             want = torch.cat(list(plain.generate(ids, 24)))

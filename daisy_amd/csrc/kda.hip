@@ -132,7 +132,7 @@ __host__ __device__ constexpr int off_block(int I, int J) { return I * (I - 1) /
 __device__ __forceinline__ void split_bf16(float x, float& hi, float& lo) { hi = round_bf16(x); lo = x - hi; }
 
 __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
-  __shared__ __attribute__((aligned(16))) float G[KC][KD];           // inclusive running log-decay; later staging for Wn
+  __shared__ __attribute__((aligned(16))) float G[KC][KD + 4];       // inclusive running log-decay (rows 4 banks apart: 16 rows read side by side do not collide); later staging for Wn
   __shared__ __attribute__((aligned(16))) uint16_t Kr[KC][KD + 8];   // k as given (bf16)
   __shared__ __attribute__((aligned(16))) uint16_t QV[KC][KD + 8];   // q as given; v as given once A and P are done
   __shared__ __attribute__((aligned(16))) float Ad[4][16][16];       // diagonal blocks of A, [block][column j][row i]; later T = (I + A_II)^-1 as bf16 hi | lo

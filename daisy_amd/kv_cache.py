@@ -11,7 +11,7 @@ writes the new row itself, and no chronological copy is ever made.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional, Tuple
+from typing import Tuple
 
 import torch
 from torch import Tensor
@@ -99,27 +99,31 @@ class KVCache:
         self.t += 1
         self._staged = [False] * self.L
 
-    def _prompt_slots(self, pos) -> Tuple[slice, Optional[Tensor]]:
+    def _prompt_runs(self, pos):
         """A prompt of ``pos`` tokens leaves room for the token that follows: only its last
-        ``min(pos, W - 1)`` positions are kept.  Returns their source range and target slots."""
+        ``min(pos, W - 1)`` positions are kept.  Position p goes to slot ``p % W``, so the kept
+        positions land in at most two runs of consecutive slots; returns ``(source, slots)``
+        slice pairs (plain slice copies run several times faster than an indexed scatter)."""
         kept = min(pos, max(self.W - 1, 0))
-        if kept == 0:
-            return slice(0, 0), None
-        positions = torch.arange(pos - kept, pos, device=self.k.device)
-        return slice(pos - kept, pos), positions.remainder_(self.W)
+        runs = []
+        first = pos - kept
+        while kept > 0:
+            slot = first % self.W
+            n = min(kept, self.W - slot)
+            runs.append((slice(first, first + n), slice(slot, slot + n)))
+            first, kept = first + n, kept - n
+        return runs
 
     def bulk_write_packed(self, kv, pos):
         """Stores a prompt's keys and values from ``kv [2, L, B, H, T, D]`` and sets ``t = pos``."""
-        src, slots = self._prompt_slots(pos)
-        if slots is not None:
-            self.k.index_copy_(3, slots, kv[0][:, :, :, src].to(self.dtype))
-            self.v.index_copy_(3, slots, kv[1][:, :, :, src].to(self.dtype))
+        for src, slots in self._prompt_runs(pos):
+            self.k[:, :, :, slots].copy_(kv[0][:, :, :, src])
+            self.v[:, :, :, slots].copy_(kv[1][:, :, :, src])
         self.t = pos
         self._staged = [False] * self.L
 
     def bulk_write_layer(self, layer, k, v, pos):
         """Per-layer form of ``bulk_write_packed`` for ``k, v [B, H, T, D]``; does not move ``t``."""
-        src, slots = self._prompt_slots(pos)
-        if slots is not None:
-            self.k[layer].index_copy_(2, slots, k[:, :, src].to(self.dtype))
-            self.v[layer].index_copy_(2, slots, v[:, :, src].to(self.dtype))
+        for src, slots in self._prompt_runs(pos):
+            self.k[layer][:, :, slots].copy_(k[:, :, src])
+            self.v[layer][:, :, slots].copy_(v[:, :, src])

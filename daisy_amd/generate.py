@@ -121,8 +121,10 @@ class Generator:
                              device=self.device, dtype=dtype)
         # In-place decode: every attention layer must understand ring handles; the ring is bf16, or
         # fp16 (the reference's default, which the decode kernel reads and appends to as it is).
+        # (layers that keep their own state, like the KDA layer, never look at their context)
         self.use_ring_context = (dtype in (torch.bfloat16, torch.float16)
-                                 and all(a is None or isinstance(a, CausalSelfAttention) for a in attn))
+                                 and all(a is None or isinstance(a, CausalSelfAttention)
+                                         or not getattr(a, "uses_kv_context", True) for a in attn))
         self._rings = [self.cache.ring(i) for i in range(len(layers))] if self.use_ring_context else None
         # record_steps: the decode step is recorded once as a HIP graph and replayed per token
         # (daisy_amd.core.GraphedStep walks the model's layers itself, so the model needs the
@@ -225,7 +227,9 @@ class Generator:
                 continue
             if k_row is None or v_row is None:
                 if blank is None:
-                    blank = torch.zeros_like(k_rows[0], dtype=self.dtype)
+                    # (the reference shapes it like the first layer's row, generate.py:240-241, and so
+                    # needs attention in the first layer; the cache's own geometry serves every stack)
+                    blank = torch.zeros(self.cache.B, 1, self.cache.H, self.cache.D, device=self.device, dtype=self.dtype)
                 k_row = v_row = blank
             self.cache.write(layer, k_row.to(self.dtype), v_row.to(self.dtype))
         self.cache.advance()

@@ -291,6 +291,15 @@ def test_recorded_step_with_a_kda_layer():
                 _close(got, want, f"prompt from {first}, replay {s} logits", tol=1e-2)
             _close(twin.blocks[0].attn._recurrent_state, model.blocks[0].attn._recurrent_state, "KDA state", tol=1e-2)
             _close(replayed.k, eager.k, "ring keys", tol=1e-2)
+        # the one-sequence generator on the hybrid stack: rings for the attention layers, recorded steps
+        from daisy_amd import Generator
+        kw = dict(window=48, seed=5, device=torch.device(DEV), dtype=torch.bfloat16, temperature=0.0)
+        plain, recorded = Generator(model, **kw), Generator(twin, record_steps=True, direct_prefill=True, **kw)
+        assert plain.use_ring_context
+        want = torch.cat(list(plain.generate(ids[0, :T], 20)))
+        got = torch.cat(list(recorded.generate(ids[0, :T], 20)))
+        say(f"hybrid generator: {want.tolist()} vs {got.tolist()}")
+        assert torch.equal(want, got)
 
 
 def test_generator_single_sequence_with_recorded_steps():

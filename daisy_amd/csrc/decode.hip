@@ -193,9 +193,16 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
     const int t = p.pos_dev != nullptr ? max(p.pos_dev[0], 0) : p.pos_host;
     const int64_t trow = (int64_t)min(t, p.table_rows - 1) * (D / 2);
     norm_rot<D>(p.q + b * p.q_sb + h * p.q_sh, dl, p.cos_tab + trow, p.sin_tab + trow, p.eps, qf);
-    norm_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_tab + trow, p.sin_tab + trow, p.eps, knf);
+    // Only the split that holds the new token's slot needs the new key and value rows.
+    const DecodeRange own = decode_range(p);
+    const int own0 = split * own.rows_per_split;
     float vnf[8];
-    norm_mix<D>(p.v_new + b * p.vn_sb + h * p.vn_sh, p.ve ? p.ve + b * p.ve_sb + h * p.ve_sh : nullptr, p.gate, dl, p.eps, vnf);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { knf[i] = 0.f; vnf[i] = 0.f; }
+    if (own.new_idx >= own0 && own.new_idx < own0 + own.rows_per_split) {
+      norm_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_tab + trow, p.sin_tab + trow, p.eps, knf);
+      norm_mix<D>(p.v_new + b * p.vn_sb + h * p.vn_sh, p.ve ? p.ve + b * p.ve_sb + h * p.ve_sh : nullptr, p.gate, dl, p.eps, vnf);
+    }
     vn_packed = F16C ? pack8_f16(vnf) : pack8(vnf);
   } else {
     static_assert(!F16C, "fp16 cache rows come with the kernel-side preparation only");

@@ -139,3 +139,32 @@ def test_ring_context_is_a_view():
     assert ring.k.data_ptr() == cache.k[1].data_ptr() and ring.W == 4 and ring.t == 0
     ring.mark_written()
     assert cache._staged == [False, True]
+
+
+def test_bf16_rows_survive_an_fp16_cache():
+    """The reference's generator keeps its cache in fp16 by default (inference/generate.py:62) while the
+    model's keys and values are bf16.  bf16 has fewer mantissa bits than fp16, so the conversion loses
+    nothing inside fp16's normal range (|x| >= 2^-14; normalised rows never exceed sqrt(D)); below it
+    the absolute error stays under 2^-25.  The decode kernel relies on this when it appends to and
+    reads from an fp16 ring."""
+    import torch
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(4096, 128, generator=g)
+    rows = (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+    back = rows.half().bfloat16()
+    normal = rows.float().abs() >= 2.0 ** -14
+    assert torch.equal(back[normal], rows[normal])
+    assert (back.float() - rows.float()).abs().max().item() <= 2.0 ** -25
+    assert rows.float().abs().max().item() <= 128 ** 0.5 + 0.1
+    # and a ring written through fp16 reads back what a bf16 ring holds
+    from daisy_amd import KVCache
+    a = KVCache(1, 2, 2, 8, 16, "cpu", torch.bfloat16)
+    b = KVCache(1, 2, 2, 8, 16, "cpu", torch.float16)
+    for t in range(11):
+        k, v = (torch.randn(2, 1, 2, 16, generator=g).bfloat16() for _ in range(2))
+        for c in (a, b):
+            c.write(0, k.to(c.dtype), v.to(c.dtype))
+            c.advance()
+    ka, va = a.view(0)
+    kb, vb = b.view(0)
+    assert torch.equal(ka.float(), kb.float()) and torch.equal(va.float(), vb.float())

@@ -176,18 +176,19 @@ def test_short_convolution_window_updated_in_place():
     out-of-place call, for one step and for a few steps at once; long inputs are refused."""
     from daisy_amd import ops
     g = torch.Generator().manual_seed(12)
-    B, C, K = 3, 256, 4
-    w = (torch.randn(C, 1, K, generator=g) * 0.3).bfloat16().to(DEV)
-    bias = (torch.randn(C, generator=g) * 0.1).bfloat16().to(DEV)
-    window = torch.randn(B, C, K, generator=g).bfloat16().to(DEV)
-    for T in (1, 5, 32):
-        x = torch.randn(B, T, C, generator=g).bfloat16().to(DEV)
-        y_ref, w_ref = ops.short_conv(x, w, bias, window, True)
-        mine = window.clone()
-        y, w_new = ops.short_conv(x, w, bias, mine, True, inplace_cache=True)
-        assert w_new.data_ptr() == mine.data_ptr()
-        assert torch.equal(y, y_ref) and torch.equal(mine, w_ref), f"T={T}"
-        window = w_ref
+    B, C = 3, 256
+    for K in (4, 3, 2):
+        w = (torch.randn(C, 1, K, generator=g) * 0.3).bfloat16().to(DEV)
+        bias = (torch.randn(C, generator=g) * 0.1).bfloat16().to(DEV)
+        window = torch.randn(B, C, K, generator=g).bfloat16().to(DEV)
+        for T in (1, 1, 2, 5, 32):
+            x = torch.randn(B, T, C, generator=g).bfloat16().to(DEV)
+            y_ref, w_ref = ops.short_conv(x, w, bias, window, True)
+            mine = window.clone()
+            y, w_new = ops.short_conv(x, w, bias, mine, True, inplace_cache=True)
+            assert w_new.data_ptr() == mine.data_ptr()
+            assert torch.equal(y, y_ref) and torch.equal(mine, w_ref), f"K={K} T={T}"
+            window = w_ref
     with pytest.raises(RuntimeError, match="in place"):
         ops.short_conv(torch.zeros(B, 40, C, device=DEV, dtype=torch.bfloat16), w, bias, window.clone(), True, inplace_cache=True)
 

@@ -10,6 +10,13 @@
 // kernel over fp32 partials in the caller's workspace.
 //
 // HBM traffic per step is the K and V rows once: B*H*n_rows*D*2*2 bytes.
+//
+// Variants of the same kernel (template flags): PREP takes the new token's rows straight from the
+// QKV projection and does the RMS norm, the rotation and the value-embedding mix itself, so that a
+// decode step is one launch between the two projections; F16C reads and appends to a cache kept in
+// fp16.  The step's position comes as a launch argument or from one int32 in device memory that
+// the kernel reads when it runs: launch arguments then do not change from step to step and a
+// recorded launch (HIP graph) can be replayed for every later token.
 #include "common.h"
 
 namespace daisy {

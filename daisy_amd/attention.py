@@ -16,6 +16,7 @@ one from token ids.  A dense reference mask is still accepted and converted
 from __future__ import annotations
 
 import os
+import weakref
 from dataclasses import dataclass
 from typing import Optional, Union
 
@@ -113,8 +114,19 @@ def _as_window_mask(attn_mask: MaskLike) -> WindowMask:
     if isinstance(attn_mask, WindowMask):
         return attn_mask
     if isinstance(attn_mask, Tensor):
-        return dense_mask_to_window(attn_mask)
+        # The reference hands one dense mask to every layer of a prefill (daisy_core.py:338-345):
+        # it is converted once (the conversion reads all T x T entries and synchronises twice).
+        global _last_dense_mask
+        ref, version, converted = _last_dense_mask
+        if ref is not None and ref() is attn_mask and attn_mask._version == version:
+            return converted
+        converted = dense_mask_to_window(attn_mask)
+        _last_dense_mask = (weakref.ref(attn_mask), attn_mask._version, converted)
+        return converted
     raise TypeError(f"unsupported attn_mask type {type(attn_mask).__name__}")
+
+
+_last_dense_mask = (None, -1, None)
 
 
 def _apply_rope(x_BTHD: Tensor, cos: Tensor, sin: Tensor) -> Tensor:

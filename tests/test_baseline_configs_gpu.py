@@ -97,6 +97,48 @@ def test_config4_decode_full_size_256_steps():
     assert torch.equal(kc[bi.to(DEV), hi.to(DEV)].cpu(), k_cpu) and torch.equal(vc[bi.to(DEV), hi.to(DEV)].cpu(), v_cpu)
 
 
+@pytest.mark.parametrize("ring_dtype", [torch.bfloat16, torch.float16])
+def test_config4_decode_steps_in_one_launch(ring_dtype):
+    """The configuration-4 ring (B64 H16 D128, 4096 slots, positions from 8192) through the one-launch step:
+    rows straight from a QKV projection, norm + RoPE + append + attention in the kernel, position in
+    device memory and counted up on the device, ring in bf16 and in the reference generator's fp16.
+    32 consecutive steps, each checked on sampled (batch, head) pairs against the CPU oracle's chain."""
+    from daisy_amd.functional import NORM_EPS_BF16
+    B, H, D, W, t0, steps = 64, 16, 128, 4096, 8192, 32
+    gd = torch.Generator(device=DEV).manual_seed(1)
+    kc = torch.randn(B, H, W, D, generator=gd, device=DEV).bfloat16().to(ring_dtype)
+    vc = torch.randn(B, H, W, D, generator=gd, device=DEV).bfloat16().to(ring_dtype)
+    pairs = [(0, 0), (17, 5), (63, 15), (31, 8)]
+    bi = torch.tensor([p[0] for p in pairs]).to(DEV)
+    hi = torch.tensor([p[1] for p in pairs]).to(DEV)
+    k_cpu, v_cpu = kc[bi, hi].float().cpu(), vc[bi, hi].float().cpu()      # [P, W, D]
+    cos, sin = oracle.rope_tables(D, t0 + steps)
+    cos_d, sin_d = cos.to(DEV), sin.to(DEV)
+    pos = torch.full((1,), t0, dtype=torch.int32, device=DEV)
+    ws = torch.empty(max(ops.decode_workspace_bytes(B, H, D, W), 1), dtype=torch.uint8, device=DEV)
+    o = torch.empty(B, H, D, dtype=torch.bfloat16, device=DEV)
+    worst = 0.0
+    for s in range(steps):
+        t = t0 + s
+        slot = t % W
+        qkv = (torch.randn(B, 3 * H, D, generator=gd, device=DEV) * 1.3).bfloat16()
+        ops.attn_step(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], kc, vc, pos, cos=cos_d, sin=sin_d, eps=NORM_EPS_BF16,
+                      scale=SCALE, out=o, workspace=ws)
+        pos.add_(1)
+        rows = [oracle.rms_norm(qkv[:, i * H:(i + 1) * H][bi, hi].cpu()) for i in range(3)]          # [P, D] each
+        q_ref = oracle.apply_rope(rows[0][:, None, None], cos[t:t + 1], sin[t:t + 1])[:, 0, 0]
+        k_ref = oracle.apply_rope(rows[1][:, None, None], cos[t:t + 1], sin[t:t + 1])[:, 0, 0]
+        k_cpu[:, slot], v_cpu[:, slot] = k_ref.float(), rows[2].float()
+        ref = oracle.sdpa(q_ref[:, None, None, :], k_cpu[:, None], v_cpu[:, None], None, SCALE)[:, 0, 0]
+        mx, _ = assert_close_bf16(o[bi, hi], ref, f"config 4 one-launch step {s} ({ring_dtype})")
+        worst = max(worst, mx)
+    say(f"config 4, one launch per step, {ring_dtype}: worst max-abs over {steps} steps {worst:.2e}")
+    assert int(pos) == t0 + steps and kc.dtype == ring_dtype
+    got_k, got_v = kc[bi, hi].float().cpu(), vc[bi, hi].float().cpu()
+    assert (got_k != k_cpu).float().mean() <= 1e-4 and (got_k - k_cpu).abs().max() <= 4e-2, "ring keys"
+    assert (got_v != v_cpu).float().mean() <= 1e-4 and (got_v - v_cpu).abs().max() <= 4e-2, "ring values"
+
+
 def test_config5_kda_full_size():
     """B4 T8192 H16 Dk=Dv=128 chunk 64: q, k L2-normalised, g = logsigmoid(N(0,1)), beta = sigmoid(N(0,1)), S0 = 0."""
     B, T, H, Dk = 4, 8192, 16, 128

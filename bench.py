@@ -237,7 +237,31 @@ def bench_decode_c4(steps=256, warmup=16, cpu_baseline=True):
         results[f"nsplit{nsplit}"] = {"ms_per_step": ms, "bytes": nbytes, "gbs": nbytes / ms / 1e6,
                                       "frac_of_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
     best = max(results.values(), key=lambda r: r["gbs"])
-    out = {"workload": "decode_c4_B64_H16_D128_W4096_256steps", "variants": results, **best}
+    # The same ring through the one-launch step (rows of a QKV projection; norm, RoPE, append and attention in the
+    # kernel; position in device memory), on a bf16 ring and on the reference generator's default, fp16.
+    from daisy_amd.functional import NORM_EPS_BF16
+    cos, sin = rope_table(D, t0 + n + 1, device=dev)
+    raw = torch.cat([qs, ks, vs], dim=2)                      # [n, B, 3H, D]
+    pos = torch.zeros(1, dtype=torch.int32, device=dev)
+    ws = torch.empty(max(ops.decode_workspace_bytes(B, H, D, W, 0), 1), dtype=torch.uint8, device=dev)
+    one_launch = {}
+    for name, ring_dtype in (("bf16_ring", torch.bfloat16), ("fp16_ring", torch.float16)):
+        kr, vr = kc.to(ring_dtype), vc.to(ring_dtype)
+        pos.fill_(t0)
+        step = [0]
+
+        def fused():
+            r = raw[step[0] % n]
+            ops.attn_step(r[:, :H], r[:, H:2 * H], r[:, 2 * H:], kr, vr, pos, cos=cos, sin=sin, eps=NORM_EPS_BF16,
+                          scale=SCALE, out=o, workspace=ws)
+            pos.add_(1)
+            step[0] += 1
+
+        ms = time_gpu(fused, steps, warmup)
+        one_launch[name] = {"ms_per_step": ms, "gbs": nbytes / ms / 1e6, "frac_of_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+        del kr, vr
+    out = {"workload": "decode_c4_B64_H16_D128_W4096_256steps", "variants": results, **best,
+           "one_launch_step_device_position": one_launch}
     if cpu_baseline:
         out["cpu_baseline"] = cpu_decode_baseline(kc[:4].cpu(), vc[:4].cpu(), qs[0, :4].cpu(), ks[0, :4].cpu(), vs[0, :4].cpu(), W,
                                                   f"4 of {B} batch elements, all {H} heads")

@@ -139,7 +139,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   __shared__ __attribute__((aligned(16))) uint16_t AoH[6][16][16];   // -A, off-diagonal blocks (off_block), [row][column], bf16 high term
   __shared__ __attribute__((aligned(16))) uint16_t AoL[6][16][16];   //   ... low term
   __shared__ float rk[KC], rq[KC], bt[KC];                           // 1/|k|, 1/|q|, beta (0 for padded rows)
-  __shared__ int steep[4];                                           // per 16-row block: total decay beyond exp(-80)
+  __shared__ int steep[4];                                           // per 16-row block: total decay beyond exp(-80); 2 when some 4 rows of it alone go beyond
   auto& Qr = QV;
   auto& Vr = QV;
 
@@ -209,7 +209,14 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       float tot = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) tot += gv[16 * blk + i];
-      if (tot < -80.f) steep[2 * half + blk] = 1;   // same value from every writer
+      if (tot < -80.f) atomicMax(&steep[2 * half + blk], 1);
+      // ... and whether four consecutive rows alone decay that far (then no reference row per
+      // group of four keeps the exponents of the matrix-core path in range)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const float t4 = gv[16 * blk + 4 * g4] + gv[16 * blk + 4 * g4 + 1] + gv[16 * blk + 4 * g4 + 2] + gv[16 * blk + 4 * g4 + 3];
+        if (t4 < -80.f) atomicMax(&steep[2 * half + blk], 2);
+      }
     }
     __syncthreads();
     if (half == 1) {
@@ -408,6 +415,82 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       }
     }
   };
+  // A steep diagonal block on the matrix cores after all: with one reference row per group of four
+  // rows (the row before the group) every row factor exp(G_i - G_ref(i)) is <= 1, and the column
+  // factors exp(G_ref - G_j) are <= 1 for columns of earlier groups and at most the decay of four
+  // rows inside the group.  Pass r multiplies all rows by the columns scaled for the reference of
+  // group r; the accumulator layout gives rows 4r..4r+3 to the lanes with q4 == r, which keep
+  // that pass's result.  Four passes, a fifth of the exponentials of the pairwise path.
+  auto steep_diagonal_mfma = [&](int I) {
+    const int li = lane & 15, q4 = lane >> 4;
+    const int ri = 16 * I + li;
+    // The diagonal block is the last of its segment: the row operands of the block row are not needed
+    // again and their registers take the ones made here.
+    bf16x8 (&sa)[4] = va;
+    bf16x8 (&sq)[4] = vq;
+    {
+      const int ref = 16 * I + (li & ~3) - 1;   // -1: the chunk's first rows, G_ref = 0
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int d0 = 32 * m + 8 * q4;
+        float ki[8], qi[8], ak[8], aq[8];
+        unpack8(*reinterpret_cast<const u32x4*>(&Kr[ri][d0]), ki);
+        unpack8(*reinterpret_cast<const u32x4*>(&Qr[ri][d0]), qi);
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+          const f32x4 gi = lds_f4(&G[ri][d0 + 4 * hf]);
+          const f32x4 gr = (ref >= 0) ? lds_f4(&G[max(ref, 0)][d0 + 4 * hf]) : zero;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float fi = __builtin_amdgcn_exp2f(gi[e] - gr[e]);
+            ak[4 * hf + e] = ki[4 * hf + e] * fi;
+            aq[4 * hf + e] = qi[4 * hf + e] * fi;
+          }
+        }
+        sa[m] = __builtin_bit_cast(bf16x8, pack8(ak));
+        sq[m] = __builtin_bit_cast(bf16x8, pack8(aq));
+      }
+    }
+    f32x4 accA = {0.f, 0.f, 0.f, 0.f}, accP = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+    for (int r = 0; r < 4; ++r) {
+      const int ref = 16 * I + 4 * r - 1;
+      const bool live = (li >> 2) <= r;     // later columns are above the diagonal for every row of the group
+      f32x4 pa = {0.f, 0.f, 0.f, 0.f}, pp = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int d0 = 32 * m + 8 * q4;
+        float kj[8], bk[8];
+        unpack8(*reinterpret_cast<const u32x4*>(&Kr[ri][d0]), kj);
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+          const f32x4 gj = lds_f4(&G[ri][d0 + 4 * hf]);
+          const f32x4 gr = (ref >= 0) ? lds_f4(&G[max(ref, 0)][d0 + 4 * hf]) : zero;
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            bk[4 * hf + e] = live ? kj[4 * hf + e] * __builtin_amdgcn_exp2f(fminf(gr[e] - gj[e], 120.f)) : 0.f;
+        }
+        const bf16x8 vb = __builtin_bit_cast(bf16x8, pack8(bk));
+        pa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sa[m], vb, pa, 0, 0, 0);
+        pp = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sq[m], vb, pp, 0, 0, 0);
+      }
+      if (q4 == r) { accA = pa; accP = pp; }
+    }
+    // accumulator: lane holds column j = 16I + li, rows i = 16I + 4*q4 + r
+    const int j = 16 * I + li;
+    const float rkj = rk[j];
+    f32x4 av;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = 16 * I + 4 * q4 + r;
+      av[r] = bt[i] * rk[i] * rkj * accA[r];
+      const float pv = (j <= i) ? p.scale * rq[i] * rkj * accP[r] : 0.f;
+      p.Pm[(ci * KC + i) * KC + perm32(j)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
+    }
+    *reinterpret_cast<f32x4*>(&Ad[I][li][4 * q4]) = av;   // entries with i <= j are never read
+  };
   {
     // Segments (block row I, columns jlo..jhi) per wavefront, 4 bits each, two per wavefront
     // (0xf.. = none).  A steep diagonal block costs about as much as five others, so when there
@@ -424,7 +507,8 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       if (I == 15) break;
       row_operands(I);
       for (int J = jlo; J <= jhi; ++J) {
-        if (J == I && steep[I]) steep_diagonal(I);
+        if (J == I && steep[I] == 2) steep_diagonal(I);
+        else if (J == I && steep[I] == 1) steep_diagonal_mfma(I);
         else mfma_block(I, J);
       }
     }

@@ -39,7 +39,10 @@ def _check(o, S, o_ref, S_ref, what):
     (2, 200, 2, 1.0),     # ragged last chunk
     (1, 17, 1, 1.0),      # shorter than a chunk
     (1, 512, 2, 0.05),    # slow decay: long memory, the S0 terms matter
-    (1, 256, 2, 8.0),     # very fast decay (|g| up to ~50 per step): nothing may overflow
+    (1, 256, 2, 8.0),     # very fast decay (|g| up to ~50 per step): nothing may overflow; diagonal blocks decay
+                          # beyond e^-80 over 16 rows and take the four-reference path on the matrix cores
+    (1, 192, 2, 15.0),    # some groups of four rows decay beyond e^-80 by themselves, others do not
+    (1, 256, 2, 30.0),    # most groups of four rows do: the pairwise fp32 path
     (2, 1024, 4, 1.0),
 ])
 def test_kda_matches_recurrence(B, T, H, g_scale):

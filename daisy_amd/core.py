@@ -230,11 +230,12 @@ class GraphedStep:
 
 @torch.no_grad()
 def generate_greedy(model, prompt_ids: Tensor, max_new_tokens: int, window: Optional[int] = None,
-                    cache: Optional[KVCache] = None) -> Tensor:
+                    cache: Optional[KVCache] = None, record_steps: bool = False) -> Tensor:
     """Greedy continuation of a batch of equally long prompts ``[B, T]`` -> ``[B, max_new_tokens]``.
 
     Rows that produce the end-of-sequence token keep emitting it.  The cache (bf16 ring of
-    ``window`` slots, default the model's window) is created unless given.
+    ``window`` slots, default the model's window) is created unless given.  ``record_steps``: the
+    decode step is recorded once (``GraphedStep``) and replayed for every token.
     """
     assert prompt_ids.ndim == 2 and prompt_ids.size(1) > 0 and max_new_tokens > 0
     B = prompt_ids.size(0)
@@ -245,6 +246,7 @@ def generate_greedy(model, prompt_ids: Tensor, max_new_tokens: int, window: Opti
                         device=dev, dtype=torch.bfloat16)
     vocab = model.embed.num_embeddings
     logits, _ = prefill(model, prompt_ids, cache)
+    one_step = GraphedStep(model, cache) if record_steps else (lambda tokens: step(model, tokens, cache))
     done = torch.zeros(B, dtype=torch.bool, device=dev)
     eos = torch.tensor(model.eos_token_id, device=dev)
     out = []
@@ -254,5 +256,5 @@ def generate_greedy(model, prompt_ids: Tensor, max_new_tokens: int, window: Opti
         done = done | (tok == eos)
         out.append(tok)
         if i < max_new_tokens - 1:
-            logits = step(model, tok, cache)
+            logits = one_step(tok)
     return torch.stack(out, dim=1)

@@ -212,6 +212,7 @@ def test_batched_prefill_and_steps_match_single_sequences():
             _close(cache.k[:, b:b + 1], c1.k, f"row {b} ring keys", tol=2e-2)
         out = core.generate_greedy(model, ids[:, :T], 6)
         assert out.shape == (B, 6) and out.dtype == torch.long
+        assert torch.equal(core.generate_greedy(model, ids[:, :T], 6, record_steps=True), out)
         with pytest.raises(Exception, match="end-of-sequence"):
             bad = ids[:, :T].clone()
             bad[1, 5] = model.eos_token_id

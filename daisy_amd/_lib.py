@@ -16,8 +16,10 @@ import torch
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libdaisy_hip.so")
 _lib: Optional[ctypes.CDLL] = None
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 PREFILL_ROTATE_K_IN_KERNEL = 1
+STATUS_POSITION_PAST_TABLES = 1
+DECODE_STATIC_SCRATCH_BYTES = 4 << 20
 
 _I64P = POINTER(c_int64)
 
@@ -31,6 +33,12 @@ SIGNATURES = {
         c_void_p, _I64P, c_void_p, _I64P,                       # o, k_out (+strides)
         c_int, c_int, c_int, c_int,                             # B, T, H, D
         c_int, c_float, c_int, c_void_p]),                      # window, scale, flags, stream
+    "daisy_prefill_fwd_f32": (c_int, [
+        c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k, v (+strides), fp32
+        c_void_p, c_void_p, c_void_p,                           # cos, sin, doc_start
+        c_void_p, _I64P, c_void_p, _I64P,                       # o, k_out (+strides), fp32
+        c_int, c_int, c_int, c_int,                             # B, T, H, D
+        c_int, c_float, c_void_p]),                             # window, scale, stream
     "daisy_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "daisy_decode_fwd": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k_new, v_new (+strides)
@@ -41,6 +49,14 @@ SIGNATURES = {
         c_int, c_int, c_int,                                    # n_rows, new_idx, write_back
         c_float, c_int,                                         # scale, nsplit
         c_void_p, c_size_t, c_void_p]),                         # workspace, bytes, stream
+    "daisy_decode_fwd_f32": (c_int, [
+        c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k_new, v_new (+strides), fp32
+        c_void_p, _I64P, c_void_p, _I64P,                       # k_cache, v_cache (+strides), fp32
+        c_void_p, c_void_p,                                     # cos_row, sin_row
+        c_void_p, _I64P,                                        # o (+strides)
+        c_int, c_int, c_int,                                    # B, H, D
+        c_int, c_int, c_int,                                    # n_rows, new_idx, write_back
+        c_float, c_void_p]),                                    # scale, stream
     "daisy_decode_fwd_at": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k_new, v_new (+strides)
         c_void_p, _I64P, c_void_p, _I64P,                       # k_cache, v_cache (+strides)
@@ -53,7 +69,7 @@ SIGNATURES = {
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k, v rows of the projection (+strides)
         c_void_p, _I64P, c_void_p,                              # ve, ve strides, gate
         c_void_p, c_void_p, c_int,                              # cos, sin, table_rows
-        c_int, c_void_p, c_float,                               # pos, pos_dev, eps
+        c_int, c_void_p, c_void_p, c_float,                     # pos, pos_dev, status, eps
         c_void_p, _I64P, c_void_p, _I64P, c_int,                # k_cache, v_cache (+strides), cache_is_f16
         c_void_p, _I64P,                                        # o (+strides)
         c_int, c_int, c_int, c_int,                             # B, H, D, ring_rows
@@ -67,6 +83,21 @@ SIGNATURES = {
         c_int, c_int, c_int, c_int, c_int, c_int,               # B, T, H, Dk, Dv, chunk
         c_float, c_int, c_float,                                # scale, l2norm_qk, l2_eps
         c_void_p, c_size_t, c_void_p]),                         # workspace, bytes, stream
+    "daisy_kda_varlen_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "daisy_kda_chunk_varlen_fwd": (c_int, [
+        c_void_p, c_void_p, c_void_p,                           # q, k, v
+        c_void_p, c_int, c_void_p,                              # g, g_is_bf16, beta
+        c_void_p, c_int,                                        # cu_seqlens (device int32), n_seq
+        c_void_p, c_void_p, c_void_p,                           # initial_state, o, final_state
+        c_int, c_int, c_int, c_int, c_int,                      # T, H, Dk, Dv, chunk
+        c_float, c_int, c_float,                                # scale, l2norm_qk, l2_eps
+        c_void_p, c_size_t, c_void_p]),                         # workspace, bytes, stream
+    "daisy_kda_recurrent_varlen_fwd": (c_int, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,  # q, k, v, g, g_is_bf16, beta
+        c_void_p, c_int,                                        # cu_seqlens (device int32), n_seq
+        c_void_p, c_void_p, c_void_p,                           # initial_state, o, final_state
+        c_int, c_int, c_int, c_int,                             # T, H, Dk, Dv
+        c_float, c_int, c_float, c_void_p]),                    # scale, l2norm_qk, l2_eps, stream
     "daisy_kda_recurrent_fwd": (c_int, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,  # q, k, v, g, g_is_bf16, beta
         c_void_p, c_void_p, c_void_p,                           # initial_state, o, final_state
@@ -76,15 +107,17 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p, c_void_p,                 # g, A_log, bias, out
         c_int64, c_int, c_int, c_int,                           # rows, H, Dk, io_is_bf16
         c_float, c_float, c_void_p]),                           # softplus beta, threshold, stream
-    "daisy_probe_matrix_rate": (c_int, [
-        c_int, c_int, c_int, c_void_p, c_void_p, POINTER(ctypes.c_double), c_void_p]),
     "daisy_short_conv_fwd": (c_int, [
         c_void_p, _I64P, c_void_p, c_void_p, c_void_p,          # x (+ strides), weight, bias, cache_in
         c_void_p, _I64P, c_void_p,                              # y (+ strides), cache_out
         c_int, c_int, c_int, c_int, c_int, c_void_p]),          # B, T, C, K, apply_silu, stream
     "daisy_gated_rmsnorm_fwd": (c_int, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_float, c_void_p]),
-    "daisy_probe_read_rate": (c_int, [c_void_p, ctypes.c_size_t, c_int, c_void_p, c_void_p]),
+    "daisy_short_conv_varlen_fwd": (c_int, [
+        c_void_p, c_int64, c_void_p, c_void_p,                  # x, x row stride, weight, bias
+        c_void_p, c_int, c_void_p,                              # cu_seqlens (device int32), n_seq, cache_in
+        c_void_p, c_int64, c_void_p,                            # y, y row stride, cache_out
+        c_int, c_int, c_int, c_int, c_void_p]),                 # T, C, K, apply_silu, stream
     "daisy_qkv_prep_fwd": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q, k, v (+ strides)
         c_void_p, _I64P, c_void_p,                               # ve, ve strides, gate
@@ -94,7 +127,7 @@ SIGNATURES = {
     "daisy_qkv_prep_fwd_at": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q, k, v (+ strides)
         c_void_p, _I64P, c_void_p,                               # ve, ve strides, gate
-        c_void_p, c_void_p, c_void_p, c_int,                    # cos, sin, pos0 (device int32), table_rows
+        c_void_p, c_void_p, c_void_p, c_int, c_void_p,          # cos, sin, pos0 (device int32), table_rows, status
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q_out, k_out, v_out (+ strides)
         c_int, c_int, c_int, c_int, c_float, c_void_p]),        # B, T, H, D, eps, stream
 }

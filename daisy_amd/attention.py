@@ -18,7 +18,7 @@ from __future__ import annotations
 import os
 import weakref
 from dataclasses import dataclass
-from typing import Optional, Union
+from typing import Optional, Tuple, Union
 
 import torch
 import torch.nn.functional as F
@@ -35,10 +35,16 @@ class WindowMask:
 
     ``window``: keys visible per query including itself (``None`` = unlimited).
     ``doc_start``: int32 ``[T]`` on the GPU, first position of each query's
-    document, or ``None`` for a single document.
+    document, or ``None`` for a single document; ``0 <= doc_start[q] <= q`` and
+    non-decreasing (the attention kernel skips key tiles by it).
+    ``kv_out``: optional ``(k, v)`` pair of bf16 ``[B, T, H, D]`` views that receive the keys
+    (normalised, rotated) and values (normalised, mixed) of the call the mask is passed to, e.g.
+    slots of a ring cache, so that no copy into the cache follows.  The model glue sets it per
+    layer; a reference-style ``Block`` passes the descriptor through untouched.
     """
     window: Optional[int]
     doc_start: Optional[Tensor] = None
+    kv_out: Optional[Tuple[Tensor, Tensor]] = None
 
 
 def doc_start_from_ids(input_seq: Tensor, eos_token_id: int) -> Tensor:
@@ -90,7 +96,9 @@ def build_block_window_masks(input_seq: Tensor, sliding_window_num_blocks, num_l
 def dense_mask_to_window(attn_mask: Tensor) -> WindowMask:
     """Converts a reference-style additive mask ``[..., T, T]`` to a ``WindowMask``.
 
-    Raises if some row is not a single run of allowed keys ending at the query.
+    Raises if some row is not a single run of allowed keys ending at the query, or if the first
+    allowed key moves backwards from one row to the next (the kernel chooses the key tiles of a
+    block of queries from the block's first row).
     """
     m = attn_mask.reshape(-1, attn_mask.shape[-2], attn_mask.shape[-1])
     torch._assert(m.shape[0] == 1, "a dense attn_mask must broadcast over batch and heads")
@@ -102,31 +110,137 @@ def dense_mask_to_window(attn_mask: Tensor) -> WindowMask:
     band = (pos[None, :] >= first[:, None]) & (pos[None, :] <= pos[:, None])
     if not bool((count == pos - first + 1).all()) or not bool((allowed == band).all()):
         raise ValueError("attn_mask is not a causal band per row; only window/document masks are supported")
+    if not bool((first[1:] >= first[:-1]).all()):
+        raise ValueError("attn_mask's first allowed key decreases along the sequence; not supported")
     return WindowMask(None, first.to(torch.int32).contiguous())
 
 
-MaskLike = Union[None, WindowMask, Tensor]
+def _marked_blocks(num: Tensor, indices: Tensor) -> Tensor:
+    """Boolean ``[rows, cols]``: entry (i, j) set when j is among the first ``num[i]`` of ``indices[i]``."""
+    rows, cols = indices.shape
+    keep = torch.arange(cols, device=indices.device)[None, :] < num[:, None].long()
+    dense = torch.zeros(rows, cols + 1, dtype=torch.bool, device=indices.device)
+    dense[torch.arange(rows, device=indices.device)[:, None].expand(rows, cols),
+          torch.where(keep, indices.long(), torch.full_like(indices, cols, dtype=torch.long))] = True
+    return dense[:, :cols]
 
 
-def _as_window_mask(attn_mask: MaskLike) -> WindowMask:
+def block_mask_to_window(block_mask, pairs_per_pass: int = 256) -> WindowMask:
+    """Converts a ``torch.nn.attention.flex_attention.BlockMask`` to a ``WindowMask``.
+
+    The reference's training forward hands such an object to ``forward(block_mask=...)``
+    (models/daisy/attention.py:156-171, built at models/daisy/daisy_core.py:209-221): per query
+    block a list of *full* key blocks (every pair visible) and a list of *partial* ones (pairs
+    filtered by ``mask_mod``).  The attention kernel takes one lower bound per query instead, so
+    the set of visible keys of every row must be one run ``[lo(q), q]`` with ``lo`` non-decreasing
+    -- which is what causal / sliding-window / document masks give.  The conversion evaluates
+    ``mask_mod`` once on the partial blocks (as ``flex_attention`` itself does), derives ``lo``
+    and verifies both conditions; anything else raises ``ValueError``.
+    """
+    qb_size, kb_size = block_mask.BLOCK_SIZE
+    num_p, idx_p = block_mask.kv_num_blocks, block_mask.kv_indices
+    torch._assert(num_p.dim() == 3 and num_p.shape[0] == 1 and num_p.shape[1] == 1,
+                  "a BlockMask must have batch and head dimensions of 1 (one mask shared by all)")
+    num_p, idx_p = num_p[0, 0], idx_p[0, 0]
+    dev = idx_p.device
+    nqb, nkb = idx_p.shape
+    q_len, kv_len = block_mask.seq_lengths
+    torch._assert(q_len == kv_len, "a BlockMask for self-attention must be square")
+    T = q_len
+    partial = _marked_blocks(num_p, idx_p)
+    if block_mask.full_kv_num_blocks is not None:
+        full = _marked_blocks(block_mask.full_kv_num_blocks[0, 0], block_mask.full_kv_indices[0, 0])
+    else:
+        full = torch.zeros_like(partial)
+    mask_mod = block_mask.mask_mod
+    big = T + kb_size
+    q_of_block = torch.arange(nqb, device=dev)[:, None] * qb_size + torch.arange(qb_size, device=dev)[None, :]   # [nqb, qb]
+    # full blocks: every key of the block is visible to every row of the query block
+    kb_first = torch.arange(nkb, device=dev) * kb_size
+    kb_last = torch.clamp_max(kb_first + kb_size, T) - 1
+    first_full = torch.where(full, kb_first[None, :], big).min(dim=1).values                     # [nqb]
+    last_full = torch.where(full, kb_last[None, :], -1).max(dim=1).values
+    count_full = (full * (kb_last - kb_first + 1)[None, :]).sum(dim=1)
+    lo = first_full[:, None].expand(nqb, qb_size).clone()
+    hi = last_full[:, None].expand(nqb, qb_size).clone()
+    count = count_full[:, None].expand(nqb, qb_size).clone()
+    # partial blocks: mask_mod decides pair by pair
+    pairs = torch.nonzero(partial & ~full)
+    zero = torch.zeros((), dtype=torch.long, device=dev)
+    for s in range(0, pairs.shape[0], pairs_per_pass):
+        qi, kj = pairs[s:s + pairs_per_pass, 0], pairs[s:s + pairs_per_pass, 1]
+        qs = (qi[:, None] * qb_size + torch.arange(qb_size, device=dev)[None, :])[:, :, None]     # [P, qb, 1]
+        ks = (kj[:, None] * kb_size + torch.arange(kb_size, device=dev)[None, :])[:, None, :]     # [P, 1, kb]
+        inside = (qs < T) & (ks < T)
+        seen = mask_mod(zero, zero, torch.clamp_max(qs, T - 1), torch.clamp_max(ks, T - 1)) & inside
+        row_lo = torch.where(seen, ks, big).amin(dim=2)                                           # [P, qb]
+        row_hi = torch.where(seen, ks, -1).amax(dim=2)
+        row_n = seen.sum(dim=2)
+        rows_of = qi[:, None].expand_as(row_lo)
+        lo.scatter_reduce_(0, rows_of, row_lo, "amin")
+        hi.scatter_reduce_(0, rows_of, row_hi, "amax")
+        count.index_add_(0, qi, row_n)
+    lo, hi, count = lo.reshape(-1)[:T], hi.reshape(-1)[:T], count.reshape(-1)[:T]
+    q = q_of_block.reshape(-1)[:T]
+    if not bool(((hi == q) & (count == q - lo + 1)).all()):
+        raise ValueError("block_mask does not describe one run of keys ending at each query; only causal "
+                         "window / document masks are supported")
+    if not bool((lo[1:] >= lo[:-1]).all()):
+        raise ValueError("block_mask's first visible key decreases along the sequence; not supported")
+    return WindowMask(None, lo.to(torch.int32).contiguous())
+
+
+def _is_flex_block_mask(obj) -> bool:
+    return all(hasattr(obj, a) for a in ("kv_num_blocks", "kv_indices", "mask_mod", "BLOCK_SIZE"))
+
+
+MaskLike = Union[None, WindowMask, Tensor, "torch.nn.attention.flex_attention.BlockMask"]
+
+
+class _ConvertedMasks:
+    """Remembers the descriptors made from dense masks and BlockMask objects.
+
+    The reference hands one mask object to every layer of a pass (daisy_core.py:251-262,338-345) and
+    a conversion reads every entry of the mask and synchronises, so it is done once per object: the
+    entries are keyed by the object's identity, hold it weakly and, for tensors, are dropped when the
+    tensor was written to since (its version counter moved).
+    """
+
+    def __init__(self, limit: int = 16):
+        self._entries: dict = {}
+        self._limit = limit
+
+    def get(self, obj, convert) -> WindowMask:
+        key = id(obj)
+        version = getattr(obj, "_version", 0)
+        hit = self._entries.get(key)
+        if hit is not None and hit[0]() is obj and hit[1] == version:
+            return hit[2]
+        converted = convert(obj)
+        if len(self._entries) >= self._limit:
+            self._entries = {k: e for k, e in self._entries.items() if e[0]() is not None}
+            while len(self._entries) >= self._limit:
+                self._entries.pop(next(iter(self._entries)))
+        try:
+            self._entries[key] = (weakref.ref(obj), version, converted)
+        except TypeError:     # an object that cannot be referenced weakly is converted every time
+            pass
+        return converted
+
+
+_converted_masks = _ConvertedMasks()
+
+
+def _as_window_mask(attn_mask) -> WindowMask:
     if attn_mask is None:
         return WindowMask(None, None)
     if isinstance(attn_mask, WindowMask):
         return attn_mask
     if isinstance(attn_mask, Tensor):
-        # The reference hands one dense mask to every layer of a prefill (daisy_core.py:338-345):
-        # it is converted once (the conversion reads all T x T entries and synchronises twice).
-        global _last_dense_mask
-        ref, version, converted = _last_dense_mask
-        if ref is not None and ref() is attn_mask and attn_mask._version == version:
-            return converted
-        converted = dense_mask_to_window(attn_mask)
-        _last_dense_mask = (weakref.ref(attn_mask), attn_mask._version, converted)
-        return converted
+        return _converted_masks.get(attn_mask, dense_mask_to_window)
+    if _is_flex_block_mask(attn_mask):
+        return _converted_masks.get(attn_mask, block_mask_to_window)
     raise TypeError(f"unsupported attn_mask type {type(attn_mask).__name__}")
-
-
-_last_dense_mask = (None, -1, None)
 
 
 def _apply_rope(x_BTHD: Tensor, cos: Tensor, sin: Tensor) -> Tensor:
@@ -278,45 +392,63 @@ class CausalSelfAttention(nn.Module):
         return ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, pos0=pos0, ve=ve, gate=gate,
                             k_out=k_out, v_out=v_out)
 
-    def _attend(self, x: Tensor, ve: Optional[Tensor], attn_mask: MaskLike):
+    def _attend(self, x: Tensor, ve: Optional[Tensor], attn_mask, kv_out=None):
+        """Returns ``y [B, T, dim]`` and q (rotated), k (rotated), v as ``[B, T, H, D]``."""
         B, T = x.size(0), x.size(1)
         mask = _as_window_mask(attn_mask)
-        # One-shot destination for k and v set by the caller of the enclosing block (the model glue
-        # points it at the ring cache's slots so that no copy into the cache follows).
-        dest = self.__dict__.pop("_kv_destination", None)
+        if mask.doc_start is not None and mask.doc_start.device != x.device:    # e.g. converted from a mask built on the CPU
+            mask = WindowMask(mask.window, mask.doc_start.to(x.device), mask.kv_out)
+        dest = kv_out if kv_out is not None else mask.kv_out
         if self._fused_prep_ok():
             q, k_rot, v = self._project_qkv_fused(x, ve, 0, *(dest or (None, None)))
             o, _ = ops.prefill_attention(q, k_rot, v, window=mask.window, scale=self.attn_scale, doc_start=mask.doc_start)
             y = F.linear(o.view(B, T, self.m_dim), self.qkvo_w[3])
-            return y, k_rot, v
+            return y, q, k_rot, v
+        torch._assert(dest is None, "writing keys and values to a destination needs the fused pre-attention kernel")
         q, k, v = self._project_qkv(x)
         dtype = q.dtype
         v = self._mix_ve(v, ve)
         cos, sin = self.rotary._get_cos_sin(T)
+        if dtype == torch.float32:
+            # fp32 parameters (the reference's unit tests build the module so): fp32 tensors and fp32
+            # arithmetic through the attention too, nothing is rounded to bf16 on the way.
+            q_rot = _apply_rope(q, cos[None, :, None, :], sin[None, :, None, :])
+            o, k_rot = ops.prefill_attention_f32(q, k, v, window=mask.window, scale=self.attn_scale, cos=cos, sin=sin,
+                                                 doc_start=mask.doc_start)
+            y = F.linear(o.view(B, T, self.m_dim), self.qkvo_w[3])
+            return y, q_rot, k_rot, v
         o, k_rot = ops.prefill_attention(
             self._kernel_dtype(q), self._kernel_dtype(k), self._kernel_dtype(v),
             window=mask.window, scale=self.attn_scale, cos=cos, sin=sin, doc_start=mask.doc_start,
             rotate_k_in_kernel=self.rotate_k_in_kernel)
         y = o.view(B, T, self.m_dim).to(dtype)
         y = F.linear(y, self.qkvo_w[3])
-        return y, k_rot.to(dtype), v
+        q_rot = _apply_rope(q, cos[None, :, None, :], sin[None, :, None, :])
+        return y, q_rot, k_rot.to(dtype), v
 
     # -- reference interface -----------------------------------------------
     def forward(self, x: Tensor, ve: Optional[Tensor], block_mask=None, attn_mask: MaskLike = None):
-        if block_mask is not None and not isinstance(block_mask, WindowMask):
-            raise NotImplementedError(
-                "flex_attention BlockMask objects (training) are not supported; pass a WindowMask")
-        y, _, _ = self._attend(x, ve, block_mask if block_mask is not None else attn_mask)
+        """``block_mask``: a ``WindowMask``, or the ``flex_attention`` ``BlockMask`` the reference's
+        training forward builds (models/daisy/daisy_core.py:209-221), converted once per object to
+        per-row bounds (``block_mask_to_window``).  Forward only: the kernels have no backward."""
+        y, _, _, _ = self._attend(x, ve, block_mask if block_mask is not None else attn_mask)
         return y
 
     def forward_sdpa(self, x: Tensor, ve: Optional[Tensor], attn_mask: MaskLike = None):
         return self.forward(x, ve, attn_mask=attn_mask)
 
-    def prefill(self, x: Tensor, ve: Optional[Tensor], attn_mask: MaskLike = None, debug: bool = False):
-        """Returns ``y [B, T, dim]``, ``k [B, H, T, D]`` (normed + rotated), ``v [B, H, T, D]``."""
-        y, k, v = self._attend(x, ve, attn_mask)
+    def prefill(self, x: Tensor, ve: Optional[Tensor], attn_mask: MaskLike = None, debug: bool = False, kv_out=None):
+        """Returns ``y [B, T, dim]``, ``k [B, H, T, D]`` (normed + rotated), ``v [B, H, T, D]``.
+
+        ``kv_out``: ``(k, v)`` destination views ``[B, T, H, D]`` (see ``WindowMask.kv_out``, which is
+        the way through a ``Block`` that passes only the reference's arguments on).
+        ``debug`` keeps the rotated q and k as ``last_q`` / ``last_k`` like the reference
+        (attention.py:176-178), as copies when they alias a destination that later steps overwrite."""
+        y, q, k, v = self._attend(x, ve, attn_mask, kv_out)
         if debug:
-            self.last_k = k
+            aliased = kv_out is not None or getattr(_as_window_mask(attn_mask), "kv_out", None) is not None
+            self.last_q = q
+            self.last_k = k.clone() if aliased else k
         return y, k.transpose(1, 2), v.transpose(1, 2)
 
     def step(self, x, k_ctx: Union[Tensor, RingContext], v_ctx: Union[Tensor, RingContext], pos: Union[int, Tensor],
@@ -356,6 +488,8 @@ class CausalSelfAttention(nn.Module):
             v = self._mix_ve(v, ve)
             cos, sin = self.rotary._get_cos_sin(pos + 1)
             cos_row, sin_row = cos[pos], sin[pos]
+        if dtype == torch.float32:
+            return self._step_f32(q, k, v, k_ctx, v_ctx, pos, window, cos_row, sin_row)
         qk, kk, vk = (self._kernel_dtype(t)[:, 0] for t in (q, k, v))  # [B, H, D]
 
         if ring is not None and (window != ring.W or ring.k.dtype != torch.bfloat16 or pos != ring.t):
@@ -391,6 +525,24 @@ class CausalSelfAttention(nn.Module):
         y = F.linear(y, self.qkvo_w[3])
         return y, k_new, v_new
 
+    def _step_f32(self, q, k, v, k_ctx, v_ctx, pos, window, cos_row, sin_row):
+        """The step of a module with fp32 parameters: fp32 tensors and arithmetic throughout
+        (``ops.decode_attention_f32``); the cached rows are taken as fp32 whatever the cache holds."""
+        B = q.size(0)
+        if isinstance(k_ctx, RingContext):
+            k_ctx, v_ctx = k_ctx.cache.view(k_ctx.layer)
+        n = k_ctx.size(1)
+        r = n if window is None else min(n, max(window - 1, 0))
+        kc = vc = None
+        if r > 0:
+            kc = k_ctx[:, n - r:n].float().transpose(1, 2)      # [B, H, r, D] view
+            vc = v_ctx[:, n - r:n].float().transpose(1, 2)
+        o = ops.decode_attention_f32(q[:, 0], k[:, 0], v[:, 0], kc, vc, n_rows=r + 1, new_idx=r, scale=self.attn_scale,
+                                     cos_row=cos_row.contiguous(), sin_row=sin_row.contiguous())
+        y = F.linear(o.reshape(B, 1, self.m_dim), self.qkvo_w[3])
+        k_new = _apply_rope(k, cos_row[None, None, None, :], sin_row[None, None, None, :])
+        return y, k_new, v
+
     def _step_in_ring(self, x, ring: RingContext, pos: Union[int, Tensor], ve: Optional[Tensor]):
         """The step as two projections around one kernel: norm, RoPE, value-embedding mix, the new
         rows' way into slot ``pos % W`` and the attention over the ring all happen in
@@ -405,7 +557,7 @@ class CausalSelfAttention(nn.Module):
             gate = torch.sigmoid(self.g_ve.detach()).to(torch.bfloat16).float().reshape(1)
         o = ops.attn_step(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], ring.k, ring.v, pos,
                           cos=self.rotary.cos, sin=self.rotary.sin, eps=NORM_EPS_BF16, ve=ve_rows, gate=gate,
-                          scale=self.attn_scale)
+                          scale=self.attn_scale, status=ring.status if isinstance(pos, Tensor) else None)
         ring.mark_written()
         y = F.linear(o.reshape(B, 1, self.m_dim), self.qkvo_w[3])
         if isinstance(pos, Tensor):

@@ -16,8 +16,8 @@ Same parameters and names as the reference's ``KimiLinearSelfAttention`` (``q_pr
 The delta-rule core runs on the HIP kernels (``chunk_kda`` for sequences, ``fused_recurrent_kda``
 with the state updated in place for single-token steps), and so do the four-tap convolutions
 with their SiLU and the gated norm (one streaming kernel each, ``daisy_short_conv_fwd`` and
-``daisy_gated_rmsnorm_fwd``; on the CPU the same arithmetic runs as PyTorch ops); the projections
-are library GEMMs.  Three pieces of the reference come from the absent
+``daisy_gated_rmsnorm_fwd``; like every op of this package they run on the GPU only and raise
+for CPU tensors); the projections are library GEMMs.  Three pieces of the reference come from the absent
 ``flash-linear-attention`` package and are restated from their documented behaviour, not pinned
 against it: ``ShortConvolution`` (depthwise causal conv + SiLU with a ``[B, C, K]`` state) and
 the gated RMS norm (``FusedRMSNormGated(activation="sigmoid", eps=1e-5)``, the module the
@@ -54,38 +54,15 @@ class ShortConvolution(nn.Module):
 
     def forward(self, x: Tensor, cache: Optional[Tensor] = None, output_final_state: bool = False,
                 cu_seqlens: Optional[Tensor] = None, inplace_cache: bool = False) -> Tuple[Tensor, Optional[Tensor]]:
-        """``inplace_cache`` (GPU kernel path, a few steps at a time): the window is updated inside
-        ``cache`` and that tensor is returned, so that its address stays the same from step to step."""
+        """One streaming kernel (``ops.short_conv``); tensors must be bf16 on the GPU, like every op of
+        this package.  ``cu_seqlens``: sequences packed along T of a batch of one -- the window does not
+        reach across a boundary and the caches are ``[N, C, K]``; the bounds stay on the device.
+        ``inplace_cache`` (a few steps at a time): the window is updated inside ``cache`` and that
+        tensor is returned, so that its address stays the same from step to step."""
         if cu_seqlens is not None:
-            # Sequences packed along T of a batch of one: the window must not reach across a
-            # boundary, so every sequence is convolved by itself; caches are [N, C, K].
-            bounds = [int(v) for v in cu_seqlens.tolist()]
-            ys, caches = [], []
-            for i in range(len(bounds) - 1):
-                c_i = cache[i:i + 1] if cache is not None else None
-                if bounds[i + 1] == bounds[i]:
-                    if output_final_state:
-                        caches.append(c_i.clone() if c_i is not None else x.new_zeros(1, x.size(2), self.kernel_size))
-                    continue
-                y_i, nc_i = self.forward(x[:, bounds[i]:bounds[i + 1]], c_i, output_final_state)
-                ys.append(y_i)
-                caches.append(nc_i)
-            return torch.cat(ys, dim=1), (torch.cat(caches, dim=0) if output_final_state else None)
-        B, T, C = x.shape
-        K = self.kernel_size
-        if x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and 2 <= K <= 4 and C % 8 == 0:
-            # one streaming pass on the GPU (no transposes, no concatenation)
-            return ops.short_conv(x, self.weight, self.bias, cache, output_final_state, "silu", inplace_cache=inplace_cache)
-        torch._assert(not inplace_cache, "the window is updated in place by the GPU kernel only")
-        xt = x.transpose(1, 2)                                        # [B, C, T]
-        prev = cache[..., 1:] if cache is not None else xt.new_zeros(B, C, K - 1)
-        window = torch.cat([prev.to(xt.dtype), xt], dim=-1)           # [B, C, K - 1 + T]
-        y = F.conv1d(window, self.weight, self.bias, groups=C)        # [B, C, T]
-        new_cache = None
-        if output_final_state:
-            tail = window[..., -K:]
-            new_cache = tail if tail.shape[-1] == K else F.pad(tail, (K - tail.shape[-1], 0))
-        return F.silu(y).transpose(1, 2).contiguous(), new_cache
+            cu_seqlens = cu_seqlens.to(device=x.device, dtype=torch.int32).contiguous()
+        return ops.short_conv(x, self.weight, self.bias, cache, output_final_state, "silu",
+                              inplace_cache=inplace_cache, cu_seqlens=cu_seqlens)
 
 
 class GatedRMSNorm(nn.Module):
@@ -97,12 +74,7 @@ class GatedRMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype))
 
     def forward(self, x: Tensor, gate: Tensor) -> Tensor:
-        if (x.is_cuda and x.dtype == gate.dtype == self.weight.dtype == torch.bfloat16
-                and self.hidden_size in (64, 128) and x.shape == gate.shape):
-            return ops.gated_rmsnorm(x, gate, self.weight, self.eps)
-        xf = x.float()
-        normed = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()
-        return (normed * torch.sigmoid(gate.float())).to(x.dtype)
+        return ops.gated_rmsnorm(x, gate, self.weight, self.eps)
 
 
 class KimiLinearSelfAttention(nn.Module):
@@ -153,10 +125,11 @@ class KimiLinearSelfAttention(nn.Module):
         self._recurrent_state: Optional[Tensor] = None
         self._conv_state = None
         self._seen = 0
-        # Buffers that held the states before the last reset_history: the next prompt's states are
-        # stored into them when they fit, so that the addresses a recorded decode step reads and
-        # writes stay the same for the life of the module.
-        self._state_homes = (None, None, None, None)
+        # Buffers that held the states before a reset_history, by batch size: the next prompt's states
+        # of that batch size are stored into them, so that the addresses a recorded decode step reads
+        # and writes stay the same for the life of the module, also when calls of different batch
+        # sizes alternate (a recorded step checks the addresses before every replay all the same).
+        self._state_homes: dict = {}
 
     def _apply(self, fn, recurse=True):
         # The decay parameters stay fp32 under module-wide casts, as the reference creates them.
@@ -172,7 +145,8 @@ class KimiLinearSelfAttention(nn.Module):
 
     def reset_history(self):
         if self._recurrent_state is not None:
-            self._state_homes = (self._recurrent_state,) + tuple(self._conv_state or (None, None, None))
+            self._state_homes[self._recurrent_state.shape[0]] = \
+                (self._recurrent_state,) + tuple(self._conv_state or (None, None, None))
         self._recurrent_state = None
         self._conv_state = None
         self._seen = 0
@@ -211,7 +185,7 @@ class KimiLinearSelfAttention(nn.Module):
         convs = self._conv_state if (use_cache and self._conv_state is not None) else (None, None, None)
         if self.use_short_conv:
             # a decode step shifts its windows in place (same tensors, same addresses, every step)
-            shift = (use_cache and T == 1 and cu_seqlens is None and x.is_cuda
+            shift = (use_cache and T == 1 and cu_seqlens is None
                      and all(c is not None and c.dtype == torch.bfloat16 and c.is_contiguous() for c in convs))
             q, cq = self.q_conv1d(self.q_proj(x), convs[0], use_cache, cu_seqlens, shift)
             k, ck = self.k_conv1d(self.k_proj(x), convs[1], use_cache, cu_seqlens, shift)
@@ -233,10 +207,10 @@ class KimiLinearSelfAttention(nn.Module):
             o, state = chunk_kda(q, k, v, g, beta, initial_state=state, output_final_state=use_cache,
                                  use_qk_l2norm_in_kernel=True, cu_seqlens=cu_seqlens)
         if use_cache:
-            homes = self._state_homes
+            homes = self._state_homes.get(state.shape[0], (None, None, None, None))
             self._recurrent_state = self._store(homes[0], state)
             self._conv_state = tuple(self._store(h, c) for h, c in zip(homes[1:], (cq, ck, cv)))
-            self._state_homes = (self._recurrent_state,) + self._conv_state
+            self._state_homes[state.shape[0]] = (self._recurrent_state,) + self._conv_state
             self._seen += T
         gate = self.g_proj(x).view(B, T, H, Dv)
         o = self.o_norm(o.to(gate.dtype), gate)

@@ -15,7 +15,12 @@ from concurrent.futures import ThreadPoolExecutor
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_NAME = "libdaisy_hip.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
-SOURCES = ["abi.hip", "decode.hip", "prefill.hip", "kda.hip", "kda_step.hip", "prep.hip", "kimi.hip", "probe.hip"]
+SOURCES = ["abi.hip", "decode.hip", "prefill.hip", "kda.hip", "kda_step.hip", "prep.hip", "kimi.hip"]
+# Diagnostic kernels for the benchmark (matrix-pipe and read-stream ceilings, a copy kernel of known
+# size): their own library, not part of the product ABI.
+PROBE_LIB_NAME = "libdaisy_probe.so"
+PROBE_LIB_PATH = os.path.join(CSRC, PROBE_LIB_NAME)
+PROBE_SOURCES = ["abi.hip", "probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -53,17 +58,24 @@ def _compile(src: str, verbose: bool) -> str:
     return obj
 
 
-def build(verbose: bool = True, sources=None) -> str:
-    """Compiles every source and links the shared library; returns its path."""
-    srcs = list(sources or SOURCES)
-    with ThreadPoolExecutor(max_workers=min(4, len(srcs))) as ex:
-        objs = list(ex.map(lambda s: _compile(s, verbose), srcs))
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH]
+def _link(objs, out: str, verbose: bool) -> None:
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+
+
+def build(verbose: bool = True, sources=None) -> str:
+    """Compiles every source and links the product library (and the benchmark's probe library);
+    returns the product library's path."""
+    srcs = list(sources or SOURCES)
+    every = srcs + [s for s in PROBE_SOURCES if s not in srcs]
+    with ThreadPoolExecutor(max_workers=min(4, len(every))) as ex:
+        objs = dict(zip(every, ex.map(lambda s: _compile(s, verbose), every)))
+    _link([objs[s] for s in srcs], LIB_PATH, verbose)
+    _link([objs[s] for s in PROBE_SOURCES], PROBE_LIB_PATH, verbose)
     return LIB_PATH
 
 

@@ -20,6 +20,8 @@ from __future__ import annotations
 
 from typing import Dict, List, Optional, Tuple
 
+import dataclasses
+
 import torch
 import torch.nn.functional as F
 from torch import Tensor
@@ -75,13 +77,12 @@ def prefill(model, input_seq: Tensor, cache: Optional[KVCache] = None, debug: bo
         attn = getattr(model.blocks[i], "attn", None)
         direct = (cache is not None and cache.dtype == torch.bfloat16 and T <= cache.W - 1
                   and isinstance(attn, CausalSelfAttention) and attn._fused_prep_ok())
+        layer_mask = attn_mask
         if direct:
-            attn._kv_destination = (cache.k[i][:, :, :T].transpose(1, 2), cache.v[i][:, :, :T].transpose(1, 2))
-        try:
-            x, k, v = model.blocks[i].prefill(x, ve_map.get(i), x0, attn_mask=attn_mask, debug=debug)
-        finally:
-            if direct:
-                attn.__dict__.pop("_kv_destination", None)
+            # the destination rides on the mask descriptor, which a block hands to its attention untouched
+            layer_mask = dataclasses.replace(attn_mask, kv_out=(cache.k[i][:, :, :T].transpose(1, 2),
+                                                                cache.v[i][:, :, :T].transpose(1, 2)))
+        x, k, v = model.blocks[i].prefill(x, ve_map.get(i), x0, attn_mask=layer_mask, debug=debug)
         skip_connections.append(x)
         if cache is not None:
             if k is not None and not direct:
@@ -122,9 +123,10 @@ def step(model, token_ids: Tensor, cache: KVCache) -> Tensor:
     return logits
 
 
-def _walk_step(model, token_ids: Tensor, cache: KVCache, pos) -> Tensor:
+def _walk_step(model, token_ids: Tensor, cache: KVCache, pos, status: Optional[Tensor] = None) -> Tensor:
     """The layer walk of ``step`` at position ``pos`` (a host int, or a one-element int32 device
-    tensor when the walk is being recorded for replay); leaves ``cache.advance()`` to the caller."""
+    tensor when the walk is being recorded for replay); leaves ``cache.advance()`` to the caller.
+    ``status``: the int32 word in which the attention kernels report a device position they cannot use."""
     token_ids = token_ids.reshape(-1, 1)
     B = token_ids.size(0)
     torch._assert(B == cache.B, "token batch does not match the cache")
@@ -145,6 +147,7 @@ def _walk_step(model, token_ids: Tensor, cache: KVCache, pos) -> Tensor:
             k_ctx = v_ctx = None        # no attention, or one that keeps its own state (KDA layers)
         elif in_place and getattr(blk.attn, "accepts_ring_context", False):
             k_ctx = v_ctx = cache.ring(i)
+            k_ctx.status = status
         else:
             torch._assert(not on_device, "a recorded step needs attention layers that take the ring in place")
             k_ctx, v_ctx = cache.view(i)
@@ -181,12 +184,29 @@ class GraphedStep:
         self._pos_host: Optional[int] = None      # what self.pos holds, None = unknown
         self._graph: Optional[torch.cuda.CUDAGraph] = None
         self._logits: Optional[Tensor] = None
+        self._recorded_addresses: Optional[tuple] = None
+        self.status = torch.zeros(1, dtype=torch.int32, device=dev)   # raised by the kernels, see check()
         tables = [blk.attn.rotary.cos.shape[0] for blk in model.blocks
                   if getattr(blk, "attn", None) is not None and hasattr(blk.attn, "rotary")]
         self.max_positions = min(tables) if tables else None
 
+    def _stateful_tensors(self) -> List[Tensor]:
+        """State that layers keep by themselves (the KDA layer's recurrent state and convolution windows)."""
+        return [t for blk in self.model.blocks if hasattr(getattr(blk, "attn", None), "state_tensors")
+                for t in blk.attn.state_tensors()]
+
+    def _addresses(self) -> tuple:
+        """Every address the recorded launches carry besides the parameters: the ring and the layers' own state."""
+        return (self.cache.k.data_ptr(), self.cache.v.data_ptr()) + tuple(t.data_ptr() for t in self._stateful_tensors())
+
+    def check(self) -> None:
+        """Raises what the kernels of the replayed steps reported (a position past the rotary tables).
+        Reads one word from the device, so it synchronises: call it after a run of steps, not per step."""
+        from . import ops
+        ops.raise_for_status(self.status)
+
     def _body(self) -> Tensor:
-        logits = _walk_step(self.model, self.tokens, self.cache, self.pos)
+        logits = _walk_step(self.model, self.tokens, self.cache, self.pos, self.status)
         self.pos.add_(1)
         return logits
 
@@ -196,9 +216,9 @@ class GraphedStep:
         # One eager pass on a side stream first (library handles, workspaces, the allocator's pools);
         # in the ring it writes the same row the first replay writes again.
         # Layers that keep their own state (KDA) would advance it twice: it is put back afterwards.
-        stateful = [t for blk in self.model.blocks if hasattr(getattr(blk, "attn", None), "state_tensors")
-                    for t in blk.attn.state_tensors()]
+        stateful = self._stateful_tensors()
         saved = [t.clone() for t in stateful]
+        before = self._addresses()
         side = torch.cuda.Stream(device=dev)
         side.wait_stream(torch.cuda.current_stream(dev))
         with torch.cuda.stream(side):
@@ -211,6 +231,14 @@ class GraphedStep:
         with torch.cuda.graph(self._graph):
             self._logits = self._body()
         self.cache._staged = [False] * self.cache.L    # recording ran no kernel
+        # The graph carries raw addresses.  A layer that made a new state tensor during the walk (no
+        # prefill before the first step, a window that could not be shifted in place) would leave the
+        # graph pointing at memory that belongs to the capture: refuse to replay such a recording.
+        self._recorded_addresses = self._addresses()
+        if self._recorded_addresses != before:
+            self._graph = None
+            raise RuntimeError("a recorded step needs layers that update their state in place: run a prefill first "
+                               "(the KDA layer creates its state there) and keep the cache's tensors")
 
     @torch.no_grad()
     def __call__(self, token_ids: Tensor) -> Tensor:
@@ -220,6 +248,10 @@ class GraphedStep:
         self.tokens.copy_(token_ids.reshape(-1))
         if self._pos_host != cache.t:
             self.pos.fill_(cache.t)
+        if self._graph is not None and self._addresses() != self._recorded_addresses:
+            # A prefill of another batch size, a new cache tensor, a reset that moved a layer's state: the
+            # recording points at memory that may have been freed.  Record again at the current addresses.
+            self._graph = None
         if self._graph is None:
             self._record()
         self._graph.replay()

@@ -70,6 +70,20 @@ __device__ __forceinline__ float rope_hi(float x1, float x2, float c, float s) {
   return a + b;
 }
 
+// Element access for kernels templated on the tensor element: uint16_t = bf16 bits, float = fp32.
+// round_elem rounds a computed value the way a tensor of that element type would hold it.
+template <typename E> __device__ __forceinline__ float load_elem(const E* p, int64_t i);
+template <> __device__ __forceinline__ float load_elem<uint16_t>(const uint16_t* p, int64_t i) { return bf16lo_to_f32(p[i]); }
+template <> __device__ __forceinline__ float load_elem<float>(const float* p, int64_t i) { return p[i]; }
+template <typename E> __device__ __forceinline__ void store_elem(E* p, int64_t i, float x);
+template <> __device__ __forceinline__ void store_elem<uint16_t>(uint16_t* p, int64_t i, float x) {
+  p[i] = (uint16_t)(pack_bf16x2(x, 0.f) & 0xffffu);
+}
+template <> __device__ __forceinline__ void store_elem<float>(float* p, int64_t i, float x) { p[i] = x; }
+template <typename E> __device__ __forceinline__ float round_elem(float x);
+template <> __device__ __forceinline__ float round_elem<uint16_t>(float x) { return round_bf16(x); }
+template <> __device__ __forceinline__ float round_elem<float>(float x) { return x; }
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // ---- cross-lane sums with DPP (no LDS traffic) -------------------------------

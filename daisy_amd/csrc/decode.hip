@@ -41,6 +41,7 @@ struct DecodeParams {
   // argument, the rotation tables, and the optional second value row with its gate.
   int pos_host; const float* cos_tab; const float* sin_tab; int table_rows; float eps;
   const uint16_t* ve; int64_t ve_sb, ve_sh; const float* gate;
+  int32_t* status;   // optional: receives DAISY_STATUS_* bits the kernel raises (never cleared by it)
 };
 
 struct DecodeRange { int n_rows, new_idx, rows_per_split; };
@@ -198,8 +199,18 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
   u32x4 vn_packed;
   if constexpr (PREP) {
     const int t = p.pos_dev != nullptr ? max(p.pos_dev[0], 0) : p.pos_host;
+    // A position past the rotation tables (possible only when it comes from device memory) reads the
+    // last table row, to stay inside the allocation, and is reported: the status word gets its bit and
+    // the outputs of the step are NaN, so that the step cannot pass for a valid one.
+    const bool past_tables = t >= p.table_rows;
     const int64_t trow = (int64_t)min(t, p.table_rows - 1) * (D / 2);
     norm_rot<D>(p.q + b * p.q_sb + h * p.q_sh, dl, p.cos_tab + trow, p.sin_tab + trow, p.eps, qf);
+    if (past_tables) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[i] = __builtin_nanf("");
+      if (p.status != nullptr && tid == 0 && split == 0 && h == 0 && b == 0)
+        __hip_atomic_fetch_or(p.status, DAISY_STATUS_POSITION_PAST_TABLES, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     // Only the split that holds the new token's slot needs the new key and value rows.
     const DecodeRange own = decode_range(p);
     const int own0 = split * own.rows_per_split;
@@ -410,33 +421,34 @@ static int resolve_nsplit(int B, int H, int n_rows, int nsplit) {
 // Any even head dim up to 256 (the reference's unit tests use 2 and 8): one wavefront per
 // (batch, head), lane l owns channels l, l + 64, ...; rows are visited one after the other with a
 // wavefront-wide reduction per score.  Correctness path for small shapes, not a fast one.
+template <typename E>
 __global__ __launch_bounds__(64) void decode_scalar_kernel(DecodeParams p, int D) {
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const int half = D / 2;
   const DecodeRange rg = decode_range(p);
-  const uint16_t* qp = p.q + b * p.q_sb + h * p.q_sh;
-  const uint16_t* knp = p.k_new + b * p.kn_sb + h * p.kn_sh;
-  const uint16_t* vnp = p.v_new + b * p.vn_sb + h * p.vn_sh;
-  uint16_t* kc = p.kc + b * p.kc_sb + h * p.kc_sh;
-  uint16_t* vc = p.vc + b * p.vc_sb + h * p.vc_sh;
+  const E* qp = reinterpret_cast<const E*>(p.q) + b * p.q_sb + h * p.q_sh;
+  const E* knp = reinterpret_cast<const E*>(p.k_new) + b * p.kn_sb + h * p.kn_sh;
+  const E* vnp = reinterpret_cast<const E*>(p.v_new) + b * p.vn_sb + h * p.vn_sh;
+  E* kc = reinterpret_cast<E*>(p.kc) + b * p.kc_sb + h * p.kc_sh;
+  E* vc = reinterpret_cast<E*>(p.vc) + b * p.vc_sb + h * p.vc_sh;
   float qv[4], kn[4], vn[4], acc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int d = lane + 64 * i;
     qv[i] = kn[i] = vn[i] = acc[i] = 0.f;
     if (d < D) {
-      float x = bf16lo_to_f32(qp[d]), y = bf16lo_to_f32(knp[d]);
+      float x = load_elem<E>(qp, d), y = load_elem<E>(knp, d);
       if (p.cos_row != nullptr) {
         const bool lower = d < half;
         const int dp = lower ? d + half : d - half;   // RoPE partner channel
         const float c = p.cos_row[lower ? d : dp], sn = p.sin_row[lower ? d : dp];
-        const float xp = bf16lo_to_f32(qp[dp]), yp = bf16lo_to_f32(knp[dp]);
-        x = round_bf16(lower ? rope_lo(x, xp, c, sn) : rope_hi(xp, x, c, sn));
-        y = round_bf16(lower ? rope_lo(y, yp, c, sn) : rope_hi(yp, y, c, sn));
+        const float xp = load_elem<E>(qp, dp), yp = load_elem<E>(knp, dp);
+        x = round_elem<E>(lower ? rope_lo(x, xp, c, sn) : rope_hi(xp, x, c, sn));
+        y = round_elem<E>(lower ? rope_lo(y, yp, c, sn) : rope_hi(yp, y, c, sn));
       }
       qv[i] = x;
       kn[i] = y;
-      vn[i] = bf16lo_to_f32(vnp[d]);
+      vn[i] = load_elem<E>(vnp, d);
     }
   }
   float m = -INFINITY, l = 0.f;
@@ -448,8 +460,8 @@ __global__ __launch_bounds__(64) void decode_scalar_kernel(DecodeParams p, int D
       const int d = lane + 64 * i;
       kr[i] = vr[i] = 0.f;
       if (d < D) {
-        kr[i] = is_new ? kn[i] : bf16lo_to_f32(kc[(int64_t)r * p.kc_sr + d]);
-        vr[i] = is_new ? vn[i] : bf16lo_to_f32(vc[(int64_t)r * p.vc_sr + d]);
+        kr[i] = is_new ? kn[i] : load_elem<E>(kc, (int64_t)r * p.kc_sr + d);
+        vr[i] = is_new ? vn[i] : load_elem<E>(vc, (int64_t)r * p.vc_sr + d);
       }
       part += qv[i] * kr[i];
     }
@@ -463,15 +475,15 @@ __global__ __launch_bounds__(64) void decode_scalar_kernel(DecodeParams p, int D
     for (int i = 0; i < 4; ++i) acc[i] = acc[i] * alpha + pr * vr[i];
     m = m_new;
   }
-  uint16_t* op = p.o + b * p.o_sb + h * p.o_sh;
+  E* op = reinterpret_cast<E*>(p.o) + b * p.o_sb + h * p.o_sh;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int d = lane + 64 * i;
     if (d < D) {
-      op[d] = (uint16_t)(pack_bf16x2(acc[i] / l, 0.f) & 0xffffu);
+      store_elem<E>(op, d, acc[i] / l);
       if (p.write_back) {
-        kc[(int64_t)rg.new_idx * p.kc_sr + d] = (uint16_t)(pack_bf16x2(kn[i], 0.f) & 0xffffu);
-        vc[(int64_t)rg.new_idx * p.vc_sr + d] = (uint16_t)(pack_bf16x2(vn[i], 0.f) & 0xffffu);
+        store_elem<E>(kc, (int64_t)rg.new_idx * p.kc_sr + d, kn[i]);
+        store_elem<E>(vc, (int64_t)rg.new_idx * p.vc_sr + d, vn[i]);
       }
     }
   }
@@ -493,7 +505,7 @@ extern "C" size_t daisy_decode_workspace_bytes(int B, int H, int D, int n_rows, 
 struct StepPrep {
   int pos_host; const float* cos; const float* sin; int table_rows; float eps;
   const void* ve; const int64_t* ve_strides; const float* gate;
-  int cache_f16;
+  int cache_f16; int32_t* status;
 };
 
 // Shared by the entry points.  With pos_dev set, n_rows is the ring's slot count (it fixes the
@@ -508,13 +520,14 @@ static int decode_launch(const void* q, const int64_t* q_strides,
                          int B, int H, int D,
                          int n_rows, int new_idx, const int32_t* pos_dev, int write_back,
                          float scale, int nsplit,
-                         void* workspace, size_t workspace_bytes, void* stream, const StepPrep* prep = nullptr) {
+                         void* workspace, size_t workspace_bytes, void* stream, const StepPrep* prep = nullptr,
+                         bool f32_io = false) {
   DAISY_CHECK_ARG(q && k_new && v_new && o, "decode: q, k_new, v_new and o must be non-NULL");
   DAISY_CHECK_ARG(q_strides && k_new_strides && v_new_strides && o_strides, "decode: stride arrays must be non-NULL");
   DAISY_CHECK_ARG(B > 0 && H > 0, "decode: B=%d and H=%d must be positive", B, H);
   DAISY_CHECK_ARG(B <= 65535 && H <= 65535, "decode: B=%d and H=%d must each be <= 65535", B, H);
   DAISY_CHECK_SUPPORTED(D >= 2 && D <= 256 && D % 2 == 0, "decode: head_dim %d not supported (even, 2..256)", D);
-  const bool fast = D == 64 || D == 128;
+  const bool fast = (D == 64 || D == 128) && !f32_io;   // fp32 tensors always take the one-wavefront kernel
   DAISY_CHECK_ARG(n_rows >= 1, "decode: n_rows=%d must be >= 1 (the new token is always attended)", n_rows);
   DAISY_CHECK_ARG(new_idx >= 0 && new_idx < n_rows, "decode: new_idx=%d outside [0, %d)", new_idx, n_rows);
   DAISY_CHECK_ARG((cos_row == nullptr) == (sin_row == nullptr), "decode: cos_row and sin_row must both be given or both NULL");
@@ -555,10 +568,10 @@ static int decode_launch(const void* q, const int64_t* q_strides,
   p.rows_per_split = (n_rows + p.nsplit - 1) / p.nsplit;
   p.pos_dev = pos_dev; p.ring_rows = n_rows;
   p.pos_host = 0; p.cos_tab = p.sin_tab = nullptr; p.table_rows = 0; p.eps = 0.f;
-  p.ve = nullptr; p.ve_sb = p.ve_sh = 0; p.gate = nullptr;
+  p.ve = nullptr; p.ve_sb = p.ve_sh = 0; p.gate = nullptr; p.status = nullptr;
   if (prep != nullptr) {
     p.pos_host = prep->pos_host; p.cos_tab = prep->cos; p.sin_tab = prep->sin; p.table_rows = prep->table_rows;
-    p.eps = prep->eps; p.ve = (const uint16_t*)prep->ve; p.gate = prep->gate;
+    p.eps = prep->eps; p.ve = (const uint16_t*)prep->ve; p.gate = prep->gate; p.status = prep->status;
     if (prep->ve) { p.ve_sb = prep->ve_strides[0]; p.ve_sh = prep->ve_strides[1]; }
   }
   p.scale_log2e = scale * kLog2e;
@@ -574,7 +587,8 @@ static int decode_launch(const void* q, const int64_t* q_strides,
 
   hipStream_t s = (hipStream_t)stream;
   if (!fast) {
-    hipLaunchKernelGGL(decode_scalar_kernel, dim3(H, B), dim3(64), 0, s, p, D);
+    if (f32_io) hipLaunchKernelGGL(decode_scalar_kernel<float>, dim3(H, B), dim3(64), 0, s, p, D);
+    else hipLaunchKernelGGL(decode_scalar_kernel<uint16_t>, dim3(H, B), dim3(64), 0, s, p, D);
     DAISY_CHECK_LAUNCH("decode_scalar_kernel");
     return DAISY_OK;
   }
@@ -617,6 +631,21 @@ extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
                        write_back, scale, nsplit, workspace, workspace_bytes, stream);
 }
 
+extern "C" int daisy_decode_fwd_f32(const float* q, const int64_t* q_strides,
+                                    const float* k_new, const int64_t* k_new_strides,
+                                    const float* v_new, const int64_t* v_new_strides,
+                                    float* k_cache, const int64_t* k_cache_strides,
+                                    float* v_cache, const int64_t* v_cache_strides,
+                                    const float* cos_row, const float* sin_row,
+                                    float* o, const int64_t* o_strides,
+                                    int B, int H, int D,
+                                    int n_rows, int new_idx, int write_back,
+                                    float scale, void* stream) {
+  return decode_launch(q, q_strides, k_new, k_new_strides, v_new, v_new_strides, k_cache, k_cache_strides,
+                       v_cache, v_cache_strides, cos_row, sin_row, o, o_strides, B, H, D, n_rows, new_idx, nullptr,
+                       write_back, scale, 1, nullptr, 0, stream, nullptr, /*f32_io=*/true);
+}
+
 extern "C" int daisy_decode_fwd_at(const void* q, const int64_t* q_strides,
                                    const void* k_new, const int64_t* k_new_strides,
                                    const void* v_new, const int64_t* v_new_strides,
@@ -641,7 +670,7 @@ extern "C" int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
                                    const void* v, const int64_t* v_strides,
                                    const void* ve, const int64_t* ve_strides, const float* gate,
                                    const float* cos, const float* sin, int table_rows,
-                                   int pos, const int32_t* pos_dev, float eps,
+                                   int pos, const int32_t* pos_dev, int32_t* status, float eps,
                                    void* k_cache, const int64_t* k_cache_strides,
                                    void* v_cache, const int64_t* v_cache_strides, int cache_is_f16,
                                    void* o, const int64_t* o_strides,
@@ -659,7 +688,7 @@ extern "C" int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
   auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
   DAISY_CHECK_ARG(al16(ve) && (!ve || (ve_strides[0] % 8 == 0 && ve_strides[1] % 8 == 0)),
                   "attn_step: ve must be 16-byte aligned with strides that are multiples of 8 elements");
-  StepPrep prep{pos, cos, sin, table_rows, eps, ve, ve_strides, gate, cache_is_f16 != 0};
+  StepPrep prep{pos, cos, sin, table_rows, eps, ve, ve_strides, gate, cache_is_f16 != 0, status};
   // With the position on the host the live rows and the slot are launch arguments (and the split
   // count follows the live rows); with the position on the device the kernel derives them.
   const int n_rows = pos_dev ? ring_rows : (pos + 1 < ring_rows ? pos + 1 : ring_rows);

@@ -117,7 +117,69 @@ struct KdaParams {
   const float* s0; uint16_t* o; float* s_out;
   int B, T, H, NC; float scale; int l2norm; float l2eps;
   uint16_t* Wn; uint16_t* Qg; uint16_t* Pm; uint16_t* KtH; uint16_t* KtL; float* U0T; float* dec;
+  // Sequences packed along the token axis of a batch of one (B == 1, T = all tokens): n_seq > 0,
+  // bounds [n_seq + 1] = sanitised running lengths, seq_chunk0 [n_seq + 1] = first chunk slot of
+  // every sequence, chunk_seq [NC] = sequence of every chunk slot; all three are written on the
+  // device by kda_chunk_table_kernel, NC is the host's upper bound T / 64 + n_seq on the slots.
+  int n_seq; const int32_t* bounds; const int32_t* seq_chunk0; const int32_t* chunk_seq;
+  int nc_total;   // chunk slots per head in the workspace: B * NC, or NC for a packed batch
 };
+
+// Where a sequence lives: token rows [tok0, tok_end) of the flattened [B * T] token axis and
+// chunk slots [c0, c0 + nc) of the workspace.  A batch element is a sequence of its own.
+struct SeqSpan { int tok0, tok_end, c0, nc; };
+__device__ __forceinline__ SeqSpan seq_span(const KdaParams& p, int seq) {
+  SeqSpan s;
+  if (p.n_seq > 0) {
+    s.tok0 = p.bounds[seq]; s.tok_end = p.bounds[seq + 1];
+    s.c0 = p.seq_chunk0[seq]; s.nc = p.seq_chunk0[seq + 1] - s.c0;
+  } else {
+    s.tok0 = seq * p.T; s.tok_end = s.tok0 + p.T;
+    s.c0 = seq * p.NC; s.nc = p.NC;
+  }
+  return s;
+}
+
+// Chunk slots of packed sequences, built on the device so that the host never reads the bounds.
+// bounds = cu_seqlens forced to start at 0, to stay within 0..T and not to decrease (whatever the
+// caller passed, no kernel then leaves the tensors); seq_chunk0 = running sum of ceil(len / 64);
+// chunk_seq = the sequence of every slot.  One workgroup; thread i takes a run of sequences.
+__global__ __launch_bounds__(256) void kda_chunk_table_kernel(const int32_t* cu, int n_seq, int T, int nc_max,
+                                                              int32_t* bounds, int32_t* seq_chunk0, int32_t* chunk_seq) {
+  __shared__ int part[256];
+  const int tid = threadIdx.x;
+  const int per = (n_seq + 1 + 255) / 256;
+  const int a = min(tid * per, n_seq + 1), b = min(a + per, n_seq + 1);
+  int hi = 0;
+  for (int i = a; i < b; ++i) hi = max(hi, min(max(cu[i], 0), T));
+  part[tid] = hi;
+  __syncthreads();
+  hi = 0;
+  for (int w = 0; w < tid; ++w) hi = max(hi, part[w]);
+  for (int i = a; i < b; ++i) {
+    hi = max(hi, min(max(cu[i], 0), T));
+    bounds[i] = (i == 0) ? 0 : hi;
+  }
+  __threadfence_block();
+  __syncthreads();
+  const int per_s = (n_seq + 255) / 256;
+  const int sa = min(tid * per_s, n_seq), sb = min(sa + per_s, n_seq);
+  int mine = 0;
+  for (int i = sa; i < sb; ++i) mine += (bounds[i + 1] - bounds[i] + KC - 1) / KC;
+  __syncthreads();
+  part[tid] = mine;
+  __syncthreads();
+  int run = 0;
+  for (int w = 0; w < tid; ++w) run += part[w];
+  for (int i = sa; i < sb; ++i) {
+    const int nc = (bounds[i + 1] - bounds[i] + KC - 1) / KC;
+    seq_chunk0[i] = min(run, nc_max);
+    for (int c = 0; c < nc; ++c)
+      if (run + c < nc_max) chunk_seq[run + c] = i;
+    run += nc;
+  }
+  if (tid == 255) seq_chunk0[n_seq] = min(run, nc_max);   // the last thread's run ends at the total
+}
 
 // Stored position of contraction index x inside its aligned group of 32: bits (4,3,2) -> (3,2,4).
 __host__ __device__ constexpr int perm32(int x) { return (x & ~0x1c) | ((x & 0x0c) << 1) | ((x & 0x10) >> 2); }
@@ -143,11 +205,24 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   auto& Qr = QV;
   auto& Vr = QV;
 
-  const int n = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  // Chunk slot gc of the workspace; token rows t0 .. t_end - 1 of the flattened token axis are this
+  // chunk's share of its sequence (t_end = end of the sequence: the last chunk may be short).
+  const int h = blockIdx.y;
+  const int gc = blockIdx.z * p.NC + blockIdx.x;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int t0 = n * KC;
-  const int64_t ci = ((int64_t)b * p.H + h) * p.NC + n;
-  auto row_off = [&](int r) -> int64_t { return (((int64_t)b * p.T + t0 + r) * p.H + h) * KD; };
+  int t0, t_end;
+  if (p.n_seq > 0) {
+    if (gc >= p.seq_chunk0[p.n_seq]) return;      // a surplus slot (the grid covers the upper bound)
+    const SeqSpan sp = seq_span(p, p.chunk_seq[gc]);
+    t0 = sp.tok0 + (gc - sp.c0) * KC;
+    t_end = sp.tok_end;
+  } else {
+    t0 = blockIdx.z * p.T + blockIdx.x * KC;
+    t_end = (blockIdx.z + 1) * p.T;
+  }
+  const int n_live = t_end - t0;                  // live rows of the chunk when < 64
+  const int64_t ci = (int64_t)h * p.nc_total + gc;
+  auto row_off = [&](int r) -> int64_t { return (((int64_t)t0 + r) * p.H + h) * KD; };
 
   // ---- phase 0a: G = cumsum(g) -----------------------------------------------
   // Every global load of the chunk (g here, then q, k, v and beta of phase 0b) goes out before
@@ -169,13 +244,13 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
     if (p.g_bf16) {
 #pragma unroll
       for (int i = 0; i < 32; ++i) {
-        const int64_t off = row_off(min(32 * half + i, p.T - 1 - t0)) + d;
+        const int64_t off = row_off(min(32 * half + i, n_live - 1)) + d;
         graw[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p.g) + (off >> 1));
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 32; ++i) {
-        const int64_t off = row_off(min(32 * half + i, p.T - 1 - t0)) + d;
+        const int64_t off = row_off(min(32 * half + i, n_live - 1)) + d;
         graw[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p.g) + off);
       }
     }
@@ -183,17 +258,17 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       const float x = g16 ? (odd ? bf16hi_to_f32(graw[i]) : bf16lo_to_f32(graw[i])) : __uint_as_float(graw[i]);
-      gv[i] = (t0 + 32 * half + i < p.T) ? x : 0.f;
+      gv[i] = (32 * half + i < n_live) ? x : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = r4 + 16 * i;
-      const int rc = min(r, p.T - 1 - t0);
+      const int rc = min(r, n_live - 1);
       const int64_t off = row_off(rc) + 8 * cc;
       kraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.k + off));
       vraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.v + off));
       qraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.q + off));
-      btv[i] = p.beta[((int64_t)b * p.T + t0 + rc) * p.H + h];
+      btv[i] = p.beta[((int64_t)t0 + rc) * p.H + h];
     }
     __builtin_amdgcn_sched_barrier(0);
     // G holds the running sum in units of log 2 (g * log2(e)): every exponential below is a bare
@@ -231,7 +306,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = r4 + 16 * i;
-    const bool live = t0 + r < p.T;
+    const bool live = r < n_live;
     const u32x4 zero4 = {0, 0, 0, 0};
     if (!live) { kraw[i] = zero4; vraw[i] = zero4; qraw[i] = zero4; }
     float kf[8], qf[8];
@@ -748,7 +823,10 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
   if ((gridDim.x & 7) == 0) vid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   constexpr int NGRP = KD / (KVS * KCT);
   const int grp = vid % NGRP, bh = vid / NGRP;
-  const int h = bh % p.H, b = bh / p.H;
+  const int h = bh % p.H, b = bh / p.H;     // b: batch element, or sequence of a packed batch
+  const SeqSpan sp = seq_span(p, b);
+  const int nc = sp.nc;                      // chunks of this sequence (0 for an empty one)
+  const int64_t ci0 = (int64_t)h * p.nc_total + sp.c0;
   const int lane = threadIdx.x & 63, ln = lane & 15, q4 = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
@@ -764,7 +842,7 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
 #pragma unroll
     for (int v = 0; v < 2; ++v) src128[v] = (8 * v + (lane >> 3)) * 128 + 16 * ((lane & 7) ^ ((4 * v + (lane >> 4)) & 7));
     auto issue_copies = [&](int n, int st) {
-      const int64_t ci = (int64_t)bh * p.NC + n;
+      const int64_t ci = ci0 + n;
       const uint32_t dst = stage_lds + st * kStageBytes;
       const uint16_t* wn = p.Wn + ci * KC * KD;
       const uint16_t* qg = p.Qg + ci * KC * KD;
@@ -790,7 +868,7 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
     uint32_t touched = 0;
     constexpr int kAhead = 3;
     auto touch_ahead = [&](int n) {
-      const int64_t ci = (int64_t)bh * p.NC + n;
+      const int64_t ci = ci0 + n;
       const uint16_t* base = (grp == 0) ? p.Wn + ci * KC * KD : (grp == 1) ? p.Qg + ci * KC * KD
                            : (grp == 2) ? p.KtH + ci * KD * KC : p.KtL + ci * KD * KC;
       asm volatile("global_load_dword %0, %1, %2" : "+v"(touched) : "v"(pw * 4096 + lane * 64), "s"(base) : "memory");
@@ -801,19 +879,19 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
       for (int k = pw; k < 4; k += KPW) {
         const int idx = 64 * k + lane, row = idx >> 2, piece = idx & 3;
         const u32x4 v = *reinterpret_cast<const u32x4*>(&ost[n & 1][row][8 * piece]);
-        const int t = n * KC + row;
-        if (t < p.T)
-          *reinterpret_cast<u32x4*>(p.o + (((int64_t)b * p.T + t) * p.H + h) * KD + KVS * KCT * grp + 8 * piece) = v;
+        const int tok = sp.tok0 + n * KC + row;
+        if (tok < sp.tok_end)
+          *reinterpret_cast<u32x4*>(p.o + ((int64_t)tok * p.H + h) * KD + KVS * KCT * grp + 8 * piece) = v;
       }
     };
-    issue_copies(0, 0);
+    if (nc > 0) issue_copies(0, 0);
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     asm volatile("" ::: "memory");
     __syncthreads();
-    for (int n = 0; n < p.NC; ++n) {
+    for (int n = 0; n < nc; ++n) {
       if (n > 0) store_o(n - 1);
-      if (n + 1 < p.NC) issue_copies(n + 1, (n + 1) & 1);
-      if (NGRP == 4 && n + kAhead < p.NC) {
+      if (n + 1 < nc) issue_copies(n + 1, (n + 1) & 1);
+      if (NGRP == 4 && n + kAhead < nc) {
         touch_ahead(n + kAhead);
         __builtin_amdgcn_s_waitcnt(0x0F71);   // vmcnt(1)
       } else {
@@ -822,7 +900,7 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
       asm volatile("" ::: "memory");
       __syncthreads();
     }
-    store_o(p.NC - 1);
+    if (nc > 0) store_o(nc - 1);
     __builtin_amdgcn_s_waitcnt(0x0F70);
     asm volatile("" :: "v"(touched));
     return;
@@ -859,7 +937,7 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
   // ahead: U0 (accumulator initial value of U), the chunk's total decay of this wavefront's
   // state rows, and this wavefront's rows of P as left operand.
   auto load_direct = [&](int n, f32x4* u0, f32x4* dcy, bf16x8 (*pa)[2]) {
-    const int64_t ci = (int64_t)bh * p.NC + n;
+    const int64_t ci = ci0 + n;
     const float* src = p.U0T + (ci * KD + vcol) * KC + 4 * q4;
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) u0[mt] = *reinterpret_cast<const f32x4*>(src + 16 * mt);
@@ -880,7 +958,7 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
   Sb[1] = pack_acc2(S[2], S[3]);
   xch[0][wave][0][lane] = __builtin_bit_cast(u32x4, Sb[0]);
   xch[0][wave][1][lane] = __builtin_bit_cast(u32x4, Sb[1]);
-  load_direct(0, u0[0], dcy[0], pa[0]);
+  if (nc > 0) load_direct(0, u0[0], dcy[0], pa[0]);
   __syncthreads();
 
   auto chunk_step = [&](int n, auto parity) {
@@ -892,7 +970,7 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
     // data-moving wavefronts (the memory pipeline of a CU is one queue: behind that burst they
     // would block this wavefront for thousands of cycles), and are waited for at the end of the
     // chunk, so that no wait for them can end up behind newer loads.
-    if (n + 1 < p.NC) load_direct(n + 1, u0[st ^ 1], dcy[st ^ 1], pa[st ^ 1]);
+    if (n + 1 < nc) load_direct(n + 1, u0[st ^ 1], dcy[st ^ 1], pa[st ^ 1]);
     __builtin_amdgcn_sched_barrier(0);
     lds_cptr sb = stage0 + st * kStageBytes;
 
@@ -986,9 +1064,9 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the direct loads of the next chunk
     __syncthreads();
   };
-  for (int n = 0; n < p.NC; n += 2) {
+  for (int n = 0; n < nc; n += 2) {
     chunk_step(n, std::integral_constant<int, 0>{});
-    if (n + 1 < p.NC) chunk_step(n + 1, std::integral_constant<int, 1>{});
+    if (n + 1 < nc) chunk_step(n + 1, std::integral_constant<int, 1>{});
   }
   if (p.s_out != nullptr) {
 #pragma unroll
@@ -1024,10 +1102,84 @@ extern "C" int daisy_kda_gate_fwd(const void* g, const float* A_log, const float
 }
 
 
+// Chunk slots of the workspace: B * ceil(T / 64), or for n_seq packed sequences of T tokens in all
+// the upper bound T / 64 + n_seq on sum(ceil(len / 64)).
+static size_t kda_chunk_slots(int B, int T, int n_seq) {
+  return n_seq > 0 ? (size_t)T / KC + (size_t)n_seq : (size_t)B * ((size_t)(T + KC - 1) / KC);
+}
+static size_t kda_table_bytes(int T, int n_seq) {
+  if (n_seq <= 0) return 0;
+  const size_t ints = 2 * ((size_t)n_seq + 1) + kda_chunk_slots(1, T, n_seq);
+  return (ints * sizeof(int32_t) + 255) & ~(size_t)255;
+}
+
 extern "C" size_t daisy_kda_workspace_bytes(int B, int T, int H, int Dk, int Dv, int chunk) {
   if (B <= 0 || T <= 0 || H <= 0 || Dk != KD || Dv != KD || chunk != KC) return 0;
-  const size_t nc = (size_t)(T + KC - 1) / KC;
-  return (size_t)B * H * nc * kChunkBytes;
+  return kda_chunk_slots(B, T, 0) * H * kChunkBytes;
+}
+
+extern "C" size_t daisy_kda_varlen_workspace_bytes(int T, int n_seq, int H, int Dk, int Dv, int chunk) {
+  if (T <= 0 || n_seq <= 0 || H <= 0 || Dk != KD || Dv != KD || chunk != KC) return 0;
+  return kda_chunk_slots(1, T, n_seq) * H * kChunkBytes + kda_table_bytes(T, n_seq);
+}
+
+// Shared by the batched and the packed entry point (n_seq == 0: batched).
+static int kda_chunk_launch(const void* q, const void* k, const void* v,
+                            const void* g, int g_is_bf16, const float* beta,
+                            const int32_t* cu_seqlens, int n_seq,
+                            const float* initial_state, void* o, float* final_state,
+                            int B, int T, int H, int Dk, int Dv, int chunk,
+                            float scale, int l2norm_qk, float l2_eps,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+  DAISY_CHECK_SUPPORTED(Dk == KD && Dv == KD, "kda: Dk=%d, Dv=%d not supported (both must be %d)", Dk, Dv, KD);
+  DAISY_CHECK_SUPPORTED(chunk == KC, "kda: chunk=%d not supported (must be %d)", chunk, KC);
+  DAISY_CHECK_ARG(q && k && v && g && beta && o, "kda: q, k, v, g, beta and o must be non-NULL");
+  DAISY_CHECK_ARG(B > 0 && T > 0 && H > 0, "kda: B=%d, T=%d, H=%d must be positive", B, T, H);
+  DAISY_CHECK_ARG(B <= 65535 && H <= 65535, "kda: B and H must each be <= 65535");
+  DAISY_CHECK_ARG((int64_t)B * T <= 0x7fffffff, "kda: B*T too large");
+  auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+  DAISY_CHECK_ARG(al16(q) && al16(k) && al16(v) && al16(g) && al16(o) && al16(workspace),
+                  "kda: tensors and workspace must be 16-byte aligned");
+  const size_t slots = kda_chunk_slots(B, T, n_seq);
+  const size_t need = slots * H * kChunkBytes + kda_table_bytes(T, n_seq);
+  if (!workspace || workspace_bytes < need) {
+    set_error("kda: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    return DAISY_ERR_WORKSPACE;
+  }
+  DAISY_CHECK_ARG(slots <= 0x7fffffff && (int64_t)(n_seq > 0 ? n_seq : B) * H * (KD / (KVS * KCT)) <= 0x7fffffff,
+                  "kda: too many chunks or sequences");
+  KdaParams p;
+  p.q = (const uint16_t*)q; p.k = (const uint16_t*)k; p.v = (const uint16_t*)v;
+  p.g = g; p.g_bf16 = g_is_bf16; p.beta = beta;
+  p.s0 = initial_state; p.o = (uint16_t*)o; p.s_out = final_state;
+  p.B = B; p.T = T; p.H = H;
+  p.NC = n_seq > 0 ? (int)slots : (T + KC - 1) / KC;
+  p.nc_total = (int)slots;
+  p.scale = scale; p.l2norm = l2norm_qk; p.l2eps = l2_eps;
+  const size_t chunks = slots * H;
+  char* w = (char*)workspace;
+  p.Wn = (uint16_t*)w;  w += chunks * KC * KD * 2;
+  p.Qg = (uint16_t*)w;  w += chunks * KC * KD * 2;
+  p.KtH = (uint16_t*)w; w += chunks * KD * KC * 2;
+  p.KtL = (uint16_t*)w; w += chunks * KD * KC * 2;
+  p.U0T = (float*)w;    w += chunks * KD * KC * 4;
+  p.Pm = (uint16_t*)w;  w += chunks * KC * KC * 2;
+  p.dec = (float*)w;    w += chunks * KD * 4;
+  p.n_seq = n_seq; p.bounds = p.seq_chunk0 = p.chunk_seq = nullptr;
+  hipStream_t s = (hipStream_t)stream;
+  if (n_seq > 0) {
+    int32_t* tab = (int32_t*)w;
+    int32_t* bounds = tab; int32_t* seq_chunk0 = tab + n_seq + 1; int32_t* chunk_seq = tab + 2 * (n_seq + 1);
+    hipLaunchKernelGGL(kda_chunk_table_kernel, dim3(1), dim3(256), 0, s, cu_seqlens, n_seq, T, (int)slots, bounds, seq_chunk0, chunk_seq);
+    DAISY_CHECK_LAUNCH("kda_chunk_table_kernel");
+    p.bounds = bounds; p.seq_chunk0 = seq_chunk0; p.chunk_seq = chunk_seq;
+  }
+  const int n_streams = n_seq > 0 ? n_seq : B;    // independent recurrences per head
+  hipLaunchKernelGGL(kda_prep_kernel, dim3(p.NC, H, n_seq > 0 ? 1 : B), dim3(256), 0, s, p);
+  DAISY_CHECK_LAUNCH("kda_prep_kernel");
+  hipLaunchKernelGGL(kda_state_kernel, dim3((unsigned)(n_streams * H * (KD / (KVS * KCT)))), dim3(64 * (KSW + KPW)), 0, s, p);
+  DAISY_CHECK_LAUNCH("kda_state_kernel");
+  return DAISY_OK;
 }
 
 extern "C" int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
@@ -1036,38 +1188,18 @@ extern "C" int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
                                    int B, int T, int H, int Dk, int Dv, int chunk,
                                    float scale, int l2norm_qk, float l2_eps,
                                    void* workspace, size_t workspace_bytes, void* stream) {
-  DAISY_CHECK_SUPPORTED(Dk == KD && Dv == KD, "kda: Dk=%d, Dv=%d not supported (both must be %d)", Dk, Dv, KD);
-  DAISY_CHECK_SUPPORTED(chunk == KC, "kda: chunk=%d not supported (must be %d)", chunk, KC);
-  DAISY_CHECK_ARG(q && k && v && g && beta && o, "kda: q, k, v, g, beta and o must be non-NULL");
-  DAISY_CHECK_ARG(B > 0 && T > 0 && H > 0, "kda: B=%d, T=%d, H=%d must be positive", B, T, H);
-  DAISY_CHECK_ARG(B <= 65535 && H <= 65535, "kda: B and H must each be <= 65535");
-  auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
-  DAISY_CHECK_ARG(al16(q) && al16(k) && al16(v) && al16(g) && al16(o) && al16(workspace),
-                  "kda: tensors and workspace must be 16-byte aligned");
-  const size_t need = daisy_kda_workspace_bytes(B, T, H, Dk, Dv, chunk);
-  if (!workspace || workspace_bytes < need) {
-    set_error("kda: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
-    return DAISY_ERR_WORKSPACE;
-  }
-  KdaParams p;
-  p.q = (const uint16_t*)q; p.k = (const uint16_t*)k; p.v = (const uint16_t*)v;
-  p.g = g; p.g_bf16 = g_is_bf16; p.beta = beta;
-  p.s0 = initial_state; p.o = (uint16_t*)o; p.s_out = final_state;
-  p.B = B; p.T = T; p.H = H; p.NC = (T + KC - 1) / KC;
-  p.scale = scale; p.l2norm = l2norm_qk; p.l2eps = l2_eps;
-  const size_t chunks = (size_t)B * H * p.NC;
-  char* w = (char*)workspace;
-  p.Wn = (uint16_t*)w;  w += chunks * KC * KD * 2;
-  p.Qg = (uint16_t*)w;  w += chunks * KC * KD * 2;
-  p.KtH = (uint16_t*)w; w += chunks * KD * KC * 2;
-  p.KtL = (uint16_t*)w; w += chunks * KD * KC * 2;
-  p.U0T = (float*)w;    w += chunks * KD * KC * 4;
-  p.Pm = (uint16_t*)w;  w += chunks * KC * KC * 2;
-  p.dec = (float*)w;
-  hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(kda_prep_kernel, dim3(p.NC, H, B), dim3(256), 0, s, p);
-  DAISY_CHECK_LAUNCH("kda_prep_kernel");
-  hipLaunchKernelGGL(kda_state_kernel, dim3((unsigned)(B * H * (KD / (KVS * KCT)))), dim3(64 * (KSW + KPW)), 0, s, p);
-  DAISY_CHECK_LAUNCH("kda_state_kernel");
-  return DAISY_OK;
+  return kda_chunk_launch(q, k, v, g, g_is_bf16, beta, nullptr, 0, initial_state, o, final_state, B, T, H, Dk, Dv, chunk,
+                          scale, l2norm_qk, l2_eps, workspace, workspace_bytes, stream);
+}
+
+extern "C" int daisy_kda_chunk_varlen_fwd(const void* q, const void* k, const void* v,
+                                          const void* g, int g_is_bf16, const float* beta,
+                                          const int32_t* cu_seqlens, int n_seq,
+                                          const float* initial_state, void* o, float* final_state,
+                                          int T, int H, int Dk, int Dv, int chunk,
+                                          float scale, int l2norm_qk, float l2_eps,
+                                          void* workspace, size_t workspace_bytes, void* stream) {
+  DAISY_CHECK_ARG(cu_seqlens != nullptr && n_seq >= 1, "kda_varlen: cu_seqlens and n_seq >= 1 are required");
+  return kda_chunk_launch(q, k, v, g, g_is_bf16, beta, cu_seqlens, n_seq, initial_state, o, final_state, 1, T, H, Dk, Dv,
+                          chunk, scale, l2norm_qk, l2_eps, workspace, workspace_bytes, stream);
 }

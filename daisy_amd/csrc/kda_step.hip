@@ -26,6 +26,8 @@ struct KdaStepParams {
   uint16_t* o;
   int B, T, H;
   float scale; int l2norm; float l2eps;
+  // Packed sequences (B == 1, T = all tokens): workgroup (s, h) walks rows cu[s] .. cu[s+1]-1.
+  const int32_t* cu; int n_seq;
 };
 
 // Sum over the 8 lanes that share jc (lane bits 3, 4, 5).
@@ -57,8 +59,15 @@ __global__ __launch_bounds__(256) void kda_recurrent_kernel(KdaStepParams p) {
     for (int i = 0; i < 16; ++i) S[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int t = 0; t < p.T; ++t) {
-    const int64_t row = ((int64_t)b * p.T + t) * p.H + h;
+  // Token rows of this recurrence on the flattened token axis; bounds read from the device are
+  // forced into 0 <= first <= end <= T so that no input can lead outside the tensors.
+  int tok0 = b * p.T, tok_end = tok0 + p.T;
+  if (p.cu != nullptr) {
+    tok0 = min(max(p.cu[b], 0), p.T);
+    tok_end = min(max(p.cu[b + 1], tok0), p.T);
+  }
+  for (int tok = tok0; tok < tok_end; ++tok) {
+    const int64_t row = (int64_t)tok * p.H + h;
     // ---- stage k, q (L2-normalised) and exp(g) of this token in LDS ---------
     float kx = 0.f, qx = 0.f;
     if (tid < RD) {
@@ -135,15 +144,17 @@ __global__ __launch_bounds__(256) void kda_recurrent_kernel(KdaStepParams p) {
 
 using namespace daisy;
 
-extern "C" int daisy_kda_recurrent_fwd(const void* q, const void* k, const void* v,
-                                       const void* g, int g_is_bf16, const float* beta,
-                                       const float* initial_state, void* o, float* final_state,
-                                       int B, int T, int H, int Dk, int Dv,
-                                       float scale, int l2norm_qk, float l2_eps, void* stream) {
+// Shared by the two entry points.  cu_seqlens == NULL: B sequences of T tokens each; otherwise
+// B sequences packed into T tokens in all.
+static int recurrent_launch(const void* q, const void* k, const void* v,
+                            const void* g, int g_is_bf16, const float* beta, const int32_t* cu_seqlens,
+                            const float* initial_state, void* o, float* final_state,
+                            int B, int T, int H, int Dk, int Dv,
+                            float scale, int l2norm_qk, float l2_eps, void* stream) {
   DAISY_CHECK_SUPPORTED(Dk == RD && Dv == RD, "kda_recurrent: Dk=%d, Dv=%d not supported (both must be %d)", Dk, Dv, RD);
   DAISY_CHECK_ARG(q && k && v && g && beta && o, "kda_recurrent: q, k, v, g, beta and o must be non-NULL");
   DAISY_CHECK_ARG(B > 0 && T > 0 && H > 0, "kda_recurrent: B=%d, T=%d, H=%d must be positive", B, T, H);
-  DAISY_CHECK_ARG((int64_t)B * H <= 0x7fffffff, "kda_recurrent: B*H too large");
+  DAISY_CHECK_ARG((int64_t)B * H <= 0x7fffffff && (int64_t)B * T <= 0x7fffffff, "kda_recurrent: B*H or B*T too large");
   auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
   DAISY_CHECK_ARG(al16(o) && al16(v) && al16(initial_state) && al16(final_state), "kda_recurrent: v, o and the states must be 16-byte aligned");
   KdaStepParams p;
@@ -152,7 +163,28 @@ extern "C" int daisy_kda_recurrent_fwd(const void* q, const void* k, const void*
   p.s_in = initial_state; p.s_out = final_state; p.o = (uint16_t*)o;
   p.B = B; p.T = T; p.H = H;
   p.scale = scale; p.l2norm = l2norm_qk; p.l2eps = l2_eps;
+  p.cu = cu_seqlens; p.n_seq = cu_seqlens ? B : 0;
   hipLaunchKernelGGL(kda_recurrent_kernel, dim3((unsigned)(B * H)), dim3(256), 0, (hipStream_t)stream, p);
   DAISY_CHECK_LAUNCH("kda_recurrent_kernel");
   return DAISY_OK;
+}
+
+extern "C" int daisy_kda_recurrent_fwd(const void* q, const void* k, const void* v,
+                                       const void* g, int g_is_bf16, const float* beta,
+                                       const float* initial_state, void* o, float* final_state,
+                                       int B, int T, int H, int Dk, int Dv,
+                                       float scale, int l2norm_qk, float l2_eps, void* stream) {
+  return recurrent_launch(q, k, v, g, g_is_bf16, beta, nullptr, initial_state, o, final_state, B, T, H, Dk, Dv,
+                          scale, l2norm_qk, l2_eps, stream);
+}
+
+extern "C" int daisy_kda_recurrent_varlen_fwd(const void* q, const void* k, const void* v,
+                                              const void* g, int g_is_bf16, const float* beta,
+                                              const int32_t* cu_seqlens, int n_seq,
+                                              const float* initial_state, void* o, float* final_state,
+                                              int T, int H, int Dk, int Dv,
+                                              float scale, int l2norm_qk, float l2_eps, void* stream) {
+  DAISY_CHECK_ARG(cu_seqlens != nullptr && n_seq >= 1, "kda_recurrent_varlen: cu_seqlens and n_seq >= 1 are required");
+  return recurrent_launch(q, k, v, g, g_is_bf16, beta, cu_seqlens, initial_state, o, final_state, n_seq, T, H, Dk, Dv,
+                          scale, l2norm_qk, l2_eps, stream);
 }

@@ -151,6 +151,91 @@ __global__ __launch_bounds__(256) void short_conv_kernel(ConvParams p) {
   }
 }
 
+// Sequences packed along T of a batch of one: the taps of a step must not reach across the start of
+// the step's sequence (they read the sequence's carried window [n_seq, C, K] or zero instead), and
+// every sequence leaves its own window.  The bounds cu [n_seq + 1] are read on the device and forced
+// into 0..T; a thread finds the sequence of its first step by bisection and walks on from there.
+// Taps are re-read from global memory (they hit the cache) instead of kept in registers, which keeps
+// the boundary handling in one place.
+template <int K>
+__global__ __launch_bounds__(256) void short_conv_varlen_kernel(ConvParams p, const int32_t* cu, int n_seq) {
+  const int cg = blockIdx.x * 256 + threadIdx.x;
+  const int c0 = 8 * cg;
+  if (c0 >= p.C) return;
+  const int t0 = blockIdx.y * kConvSeg;
+  const int t1 = min(t0 + kConvSeg, p.T);
+  auto bound = [&](int i) { return min(max(cu[i], 0), p.T); };
+
+  float w[K][8], acc0[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+#pragma unroll
+    for (int j = 0; j < K; ++j) w[j][e] = bf16lo_to_f32(p.w[(int64_t)(c0 + e) * K + j]);
+    acc0[e] = p.bias ? bf16lo_to_f32(p.bias[c0 + e]) : 0.f;
+  }
+  // Input of sequence `seq` (first row `start`) at row ti; rows before the start come from the window.
+  auto input_at = [&](int seq, int start, int ti, float* f) {
+    if (ti >= start) {
+      unpack8(*reinterpret_cast<const u32x4*>(p.x + (int64_t)ti * p.x_st + c0), f);
+    } else {
+      const int slot = K + (ti - start);     // window slot: K-1 is the input just before the sequence
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        f[e] = (p.cache_in != nullptr && seq < n_seq && slot >= 0) ? bf16lo_to_f32(p.cache_in[((int64_t)seq * p.C + c0 + e) * K + slot]) : 0.f;
+    }
+  };
+  auto leave_window = [&](int seq, int start, int end) {
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      float f[8];
+      input_at(seq, start, end - K + j, f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) p.cache_out[((int64_t)seq * p.C + c0 + e) * K + j] = (uint16_t)(pack_bf16x2(f[e], 0.f) & 0xffffu);
+    }
+  };
+
+  // smallest seq in [0, n_seq] whose end lies beyond t0 (n_seq: rows behind the last bound, a sequence
+  // of their own without a window)
+  int lo = 0, hi = n_seq;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (bound(mid + 1) > t0) hi = mid; else lo = mid + 1;
+  }
+  int seq = lo;
+  int start = bound(min(seq, n_seq)), end = seq < n_seq ? bound(seq + 1) : p.T;
+  for (int t = t0; t < t1; ++t) {
+    while (t >= end && seq < n_seq) {
+      ++seq;
+      start = bound(min(seq, n_seq));
+      end = seq < n_seq ? bound(seq + 1) : p.T;
+    }
+    float a[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) a[e] = acc0[e];
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      float f[8];
+      input_at(seq, start, t - (K - 1) + j, f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a[e] = fmaf(w[j][e], f[e], a[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      a[e] = round_bf16(a[e]);
+      if (p.silu) a[e] = a[e] * __builtin_amdgcn_rcpf(1.f + __expf(-a[e]));
+    }
+    *reinterpret_cast<u32x4*>(p.y + (int64_t)t * p.y_st + c0) = pack8(a);
+    if (p.cache_out != nullptr && seq < n_seq && t == end - 1) leave_window(seq, start, end);
+  }
+  // Empty sequences keep their window; the threads of the first time segment see to it.
+  if (p.cache_out != nullptr && blockIdx.y == 0) {
+    for (int i = 0; i < n_seq; ++i) {
+      const int b0 = bound(i), b1 = bound(i + 1);
+      if (b1 <= b0) leave_window(i, b0, b0);
+    }
+  }
+}
+
 struct GatedNormParams {
   const uint16_t* x; const uint16_t* gate; const uint16_t* weight; uint16_t* out;
   int64_t rows; float eps;
@@ -210,6 +295,35 @@ extern "C" int daisy_short_conv_fwd(const void* x, const int64_t* x_strides, con
   else if (K == 3) hipLaunchKernelGGL(short_conv_kernel<3>, grid, dim3(256), 0, s, p);
   else hipLaunchKernelGGL(short_conv_kernel<2>, grid, dim3(256), 0, s, p);
   DAISY_CHECK_LAUNCH("short_conv_kernel");
+  return DAISY_OK;
+}
+
+extern "C" int daisy_short_conv_varlen_fwd(const void* x, int64_t x_row_stride, const void* weight, const void* bias,
+                                           const int32_t* cu_seqlens, int n_seq, const void* cache_in,
+                                           void* y, int64_t y_row_stride, void* cache_out,
+                                           int T, int C, int K, int apply_silu, void* stream) {
+  DAISY_CHECK_ARG(x && weight && y, "short_conv_varlen: x, weight and y must be non-NULL");
+  DAISY_CHECK_ARG(cu_seqlens != nullptr && n_seq >= 1, "short_conv_varlen: cu_seqlens and n_seq >= 1 are required");
+  DAISY_CHECK_ARG(T > 0 && C > 0, "short_conv_varlen: T=%d, C=%d must be positive", T, C);
+  DAISY_CHECK_SUPPORTED(K >= 2 && K <= 4, "short_conv_varlen: kernel size %d not supported (2..4)", K);
+  DAISY_CHECK_SUPPORTED(C % 8 == 0, "short_conv_varlen: channels (%d) must be a multiple of 8", C);
+  auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+  DAISY_CHECK_ARG(al16(x) && al16(y) && x_row_stride % 8 == 0 && y_row_stride % 8 == 0,
+                  "short_conv_varlen: x and y must be 16-byte aligned with row strides that are multiples of 8 elements");
+  DAISY_CHECK_ARG(cache_out == nullptr || cache_out != cache_in, "short_conv_varlen: the windows cannot be updated in place");
+  ConvParams p;
+  p.x = (const uint16_t*)x; p.x_sb = 0; p.x_st = x_row_stride;
+  p.w = (const uint16_t*)weight; p.bias = (const uint16_t*)bias; p.cache_in = (const uint16_t*)cache_in;
+  p.y = (uint16_t*)y; p.y_sb = 0; p.y_st = y_row_stride;
+  p.cache_out = (uint16_t*)cache_out;
+  p.B = 1; p.T = T; p.C = C; p.silu = apply_silu;
+  const dim3 grid((unsigned)((C / 8 + 255) / 256), (unsigned)((T + kConvSeg - 1) / kConvSeg), 1);
+  DAISY_CHECK_ARG(grid.y <= 65535, "short_conv_varlen: T=%d too long for one launch", T);
+  hipStream_t s = (hipStream_t)stream;
+  if (K == 4) hipLaunchKernelGGL(short_conv_varlen_kernel<4>, grid, dim3(256), 0, s, p, cu_seqlens, n_seq);
+  else if (K == 3) hipLaunchKernelGGL(short_conv_varlen_kernel<3>, grid, dim3(256), 0, s, p, cu_seqlens, n_seq);
+  else hipLaunchKernelGGL(short_conv_varlen_kernel<2>, grid, dim3(256), 0, s, p, cu_seqlens, n_seq);
+  DAISY_CHECK_LAUNCH("short_conv_varlen_kernel");
   return DAISY_OK;
 }
 

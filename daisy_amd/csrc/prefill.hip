@@ -867,24 +867,30 @@ __global__ __launch_bounds__(256) void rope_k_kernel(PrefillParams p) {
   *reinterpret_cast<u32x4*>(op + HALF) = pack8(y2);
 }
 
-// Scalar kernel for head dims the MFMA kernel does not cover (any even D <= 256).
-// One wavefront per (batch, head, query); lanes split the head dim.  Slow by
-// design: it serves tiny shapes only.
+// Scalar kernel for head dims the MFMA kernel does not cover (any even D <= 256) and for fp32
+// tensors.  One wavefront per (batch, head, query); lanes split the head dim.  Slow by
+// design: it serves tiny shapes and the full-precision mode only.  E = uint16_t (bf16 bits;
+// rotated values are rounded to bf16 as the bf16 tensors of the reference are) or float
+// (nothing is rounded: fp32 in, fp32 arithmetic, fp32 out).
+template <typename E>
 __global__ __launch_bounds__(64) void prefill_scalar_kernel(PrefillParams p) {
   const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int lane = threadIdx.x;
   const int D = p.D, HALF = D / 2;
   constexpr int MAXPL = 4;  // channels per lane (D <= 256)
   float qv[MAXPL], acc[MAXPL];
-  const uint16_t* qp = p.q + b * p.q_sb + (int64_t)t * p.q_st + h * p.q_sh;
-  auto rot_load = [&](const uint16_t* vec, int pos, int d) -> float {
-    float x = bf16lo_to_f32(vec[d]);
+  const E* qbase = reinterpret_cast<const E*>(p.q);
+  const E* kbase = reinterpret_cast<const E*>(p.k);
+  const E* vbase = reinterpret_cast<const E*>(p.v);
+  const E* qp = qbase + b * p.q_sb + (int64_t)t * p.q_st + h * p.q_sh;
+  auto rot_load = [&](const E* vec, int pos, int d) -> float {
+    float x = load_elem<E>(vec, d);
     if (p.cos != nullptr) {
       const bool lower = d < HALF;
-      const float xp = bf16lo_to_f32(vec[lower ? d + HALF : d - HALF]);
+      const float xp = load_elem<E>(vec, lower ? d + HALF : d - HALF);
       const float c = p.cos[(int64_t)pos * HALF + (lower ? d : d - HALF)];
       const float s = p.sin[(int64_t)pos * HALF + (lower ? d : d - HALF)];
-      x = round_bf16(lower ? rope_lo(x, xp, c, s) : rope_hi(xp, x, c, s));
+      x = round_elem<E>(lower ? rope_lo(x, xp, c, s) : rope_hi(xp, x, c, s));
     }
     return x;
   };
@@ -895,15 +901,15 @@ __global__ __launch_bounds__(64) void prefill_scalar_kernel(PrefillParams p) {
     acc[i] = 0.f;
   }
   if (p.k_out != nullptr && p.cos != nullptr) {
-    const uint16_t* kp = p.k + b * p.k_sb + (int64_t)t * p.k_st + h * p.k_sh;
-    uint16_t* op = p.k_out + b * p.ko_sb + (int64_t)t * p.ko_st + h * p.ko_sh;
-    for (int d = lane; d < D; d += 64) op[d] = (uint16_t)(pack_bf16x2(rot_load(kp, t, d), 0.f) & 0xffffu);
+    const E* kp = kbase + b * p.k_sb + (int64_t)t * p.k_st + h * p.k_sh;
+    E* op = reinterpret_cast<E*>(p.k_out) + b * p.ko_sb + (int64_t)t * p.ko_st + h * p.ko_sh;
+    for (int d = lane; d < D; d += 64) store_elem<E>(op, d, rot_load(kp, t, d));
   }
   float m = -INFINITY, l = 0.f;
   const int lo = row_lo(p, t);
   for (int kv = lo; kv <= t; ++kv) {
-    const uint16_t* kp = p.k + b * p.k_sb + (int64_t)kv * p.k_st + h * p.k_sh;
-    const uint16_t* vp = p.v + b * p.v_sb + (int64_t)kv * p.v_st + h * p.v_sh;
+    const E* kp = kbase + b * p.k_sb + (int64_t)kv * p.k_st + h * p.k_sh;
+    const E* vp = vbase + b * p.v_sb + (int64_t)kv * p.v_st + h * p.v_sh;
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < MAXPL; ++i) {
@@ -919,15 +925,15 @@ __global__ __launch_bounds__(64) void prefill_scalar_kernel(PrefillParams p) {
 #pragma unroll
     for (int i = 0; i < MAXPL; ++i) {
       const int d = lane + 64 * i;
-      if (d < D) acc[i] = acc[i] * alpha + pw * bf16lo_to_f32(vp[d]);
+      if (d < D) acc[i] = acc[i] * alpha + pw * load_elem<E>(vp, d);
     }
     m = mn;
   }
-  uint16_t* op = p.o + b * p.o_sb + (int64_t)t * p.o_st + h * p.o_sh;
+  E* op = reinterpret_cast<E*>(p.o) + b * p.o_sb + (int64_t)t * p.o_st + h * p.o_sh;
 #pragma unroll
   for (int i = 0; i < MAXPL; ++i) {
     const int d = lane + 64 * i;
-    if (d < D) op[d] = (uint16_t)(pack_bf16x2(acc[i] / l, 0.f) & 0xffffu);
+    if (d < D) store_elem<E>(op, d, acc[i] / l);
   }
 }
 
@@ -945,12 +951,43 @@ static int launch_mfma(PrefillParams p, bool rope_in_kernel, hipStream_t s) {
     DAISY_CHECK_LAUNCH("rope_k_kernel");
     p.k = p.k_out; p.k_sb = p.ko_sb; p.k_st = p.ko_st; p.k_sh = p.ko_sh;
     hipLaunchKernelGGL((prefill_pipe_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
+    DAISY_CHECK_LAUNCH("prefill_pipe_kernel");
   } else if (p.cos != nullptr) {
     hipLaunchKernelGGL((prefill_mfma_kernel<D, true>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
+    DAISY_CHECK_LAUNCH("prefill_mfma_kernel");
   } else {
     hipLaunchKernelGGL((prefill_pipe_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
+    DAISY_CHECK_LAUNCH("prefill_pipe_kernel");
   }
-  DAISY_CHECK_LAUNCH("prefill_mfma_kernel");
+  return DAISY_OK;
+}
+
+// Argument checks and parameter block shared by the bf16 and the fp32 entry point.
+static int fill_prefill_params(PrefillParams& p, const void* q, const int64_t* q_strides,
+                               const void* k, const int64_t* k_strides,
+                               const void* v, const int64_t* v_strides,
+                               const float* cos, const float* sin, const int32_t* doc_start,
+                               void* o, const int64_t* o_strides,
+                               void* k_out, const int64_t* k_out_strides,
+                               int B, int T, int H, int D, int window, float scale) {
+  DAISY_CHECK_ARG(q && k && v && o, "prefill: q, k, v and o must be non-NULL");
+  DAISY_CHECK_ARG(q_strides && k_strides && v_strides && o_strides, "prefill: stride arrays must be non-NULL");
+  DAISY_CHECK_ARG(B > 0 && T > 0 && H > 0, "prefill: B=%d, T=%d, H=%d must be positive", B, T, H);
+  DAISY_CHECK_ARG((cos == nullptr) == (sin == nullptr), "prefill: cos and sin must both be given or both NULL");
+  DAISY_CHECK_ARG(k_out == nullptr || k_out_strides != nullptr, "prefill: k_out needs k_out_strides");
+  DAISY_CHECK_SUPPORTED(D >= 2 && D <= 256 && D % 2 == 0, "prefill: head_dim %d not supported (even, 2..256)", D);
+  p.q = (const uint16_t*)q; p.q_sb = q_strides[0]; p.q_st = q_strides[1]; p.q_sh = q_strides[2];
+  p.k = (const uint16_t*)k; p.k_sb = k_strides[0]; p.k_st = k_strides[1]; p.k_sh = k_strides[2];
+  p.v = (const uint16_t*)v; p.v_sb = v_strides[0]; p.v_st = v_strides[1]; p.v_sh = v_strides[2];
+  p.cos = cos; p.sin = sin; p.doc_start = doc_start;
+  p.o = (uint16_t*)o; p.o_sb = o_strides[0]; p.o_st = o_strides[1]; p.o_sh = o_strides[2];
+  p.k_out = (uint16_t*)k_out;
+  p.ko_sb = k_out ? k_out_strides[0] : 0; p.ko_st = k_out ? k_out_strides[1] : 0; p.ko_sh = k_out ? k_out_strides[2] : 0;
+  p.B = B; p.T = T; p.H = H; p.D = D; p.window = window;
+  p.nqb = (T + kBM - 1) / kBM;
+  p.period = (window > 0 && window < T) ? (kBM - 1) / kBN + 1 + (window - 1 + kBN - 1) / kBN : 0;
+  p.n_light = (window > 0 && window < T) ? min((window - 1 + kBM - 1) / kBM, p.nqb) : 0;
+  p.scale_log2e = scale * kLog2e;
   return DAISY_OK;
 }
 
@@ -967,26 +1004,10 @@ extern "C" int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
                                  void* k_out, const int64_t* k_out_strides,
                                  int B, int T, int H, int D,
                                  int window, float scale, int flags, void* stream) {
-  DAISY_CHECK_ARG(q && k && v && o, "prefill: q, k, v and o must be non-NULL");
-  DAISY_CHECK_ARG(q_strides && k_strides && v_strides && o_strides, "prefill: stride arrays must be non-NULL");
-  DAISY_CHECK_ARG(B > 0 && T > 0 && H > 0, "prefill: B=%d, T=%d, H=%d must be positive", B, T, H);
-  DAISY_CHECK_ARG((cos == nullptr) == (sin == nullptr), "prefill: cos and sin must both be given or both NULL");
-  DAISY_CHECK_ARG(k_out == nullptr || k_out_strides != nullptr, "prefill: k_out needs k_out_strides");
-  DAISY_CHECK_SUPPORTED(D >= 2 && D <= 256 && D % 2 == 0, "prefill: head_dim %d not supported (even, 2..256)", D);
-
   PrefillParams p;
-  p.q = (const uint16_t*)q; p.q_sb = q_strides[0]; p.q_st = q_strides[1]; p.q_sh = q_strides[2];
-  p.k = (const uint16_t*)k; p.k_sb = k_strides[0]; p.k_st = k_strides[1]; p.k_sh = k_strides[2];
-  p.v = (const uint16_t*)v; p.v_sb = v_strides[0]; p.v_st = v_strides[1]; p.v_sh = v_strides[2];
-  p.cos = cos; p.sin = sin; p.doc_start = doc_start;
-  p.o = (uint16_t*)o; p.o_sb = o_strides[0]; p.o_st = o_strides[1]; p.o_sh = o_strides[2];
-  p.k_out = (uint16_t*)k_out;
-  p.ko_sb = k_out ? k_out_strides[0] : 0; p.ko_st = k_out ? k_out_strides[1] : 0; p.ko_sh = k_out ? k_out_strides[2] : 0;
-  p.B = B; p.T = T; p.H = H; p.D = D; p.window = window;
-  p.nqb = (T + kBM - 1) / kBM;
-  p.period = (window > 0 && window < T) ? (kBM - 1) / kBN + 1 + (window - 1 + kBN - 1) / kBN : 0;
-  p.n_light = (window > 0 && window < T) ? min((window - 1 + kBM - 1) / kBM, p.nqb) : 0;
-  p.scale_log2e = scale * kLog2e;
+  const int rc = fill_prefill_params(p, q, q_strides, k, k_strides, v, v_strides, cos, sin, doc_start, o, o_strides,
+                                     k_out, k_out_strides, B, T, H, D, window, scale);
+  if (rc != DAISY_OK) return rc;
   hipStream_t s = (hipStream_t)stream;
 
   if (D == 64 || D == 128) {
@@ -1003,7 +1024,26 @@ extern "C" int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
   }
 
   DAISY_CHECK_ARG(B <= 65535 && H <= 65535, "prefill: B and H must each be <= 65535 for the scalar kernel");
-  hipLaunchKernelGGL(prefill_scalar_kernel, dim3(T, H, B), dim3(64), 0, s, p);
+  hipLaunchKernelGGL(prefill_scalar_kernel<uint16_t>, dim3(T, H, B), dim3(64), 0, s, p);
   DAISY_CHECK_LAUNCH("prefill_scalar_kernel");
+  return DAISY_OK;
+}
+
+extern "C" int daisy_prefill_fwd_f32(const float* q, const int64_t* q_strides,
+                                     const float* k, const int64_t* k_strides,
+                                     const float* v, const int64_t* v_strides,
+                                     const float* cos, const float* sin,
+                                     const int32_t* doc_start,
+                                     float* o, const int64_t* o_strides,
+                                     float* k_out, const int64_t* k_out_strides,
+                                     int B, int T, int H, int D,
+                                     int window, float scale, void* stream) {
+  PrefillParams p;
+  const int rc = fill_prefill_params(p, q, q_strides, k, k_strides, v, v_strides, cos, sin, doc_start, o, o_strides,
+                                     k_out, k_out_strides, B, T, H, D, window, scale);
+  if (rc != DAISY_OK) return rc;
+  DAISY_CHECK_ARG(B <= 65535 && H <= 65535, "prefill: B and H must each be <= 65535 for the fp32 kernel");
+  hipLaunchKernelGGL(prefill_scalar_kernel<float>, dim3(T, H, B), dim3(64), 0, (hipStream_t)stream, p);
+  DAISY_CHECK_LAUNCH("prefill_scalar_kernel<float>");
   return DAISY_OK;
 }

@@ -27,6 +27,7 @@ struct PrepParams {
   // When set, the first position is read from device memory at run time (so that a recorded
   // launch can be replayed for later positions) and held inside the table's rows.
   const int32_t* pos0_dev; int table_rows;
+  int32_t* status;   // optional: receives DAISY_STATUS_* bits the kernel raises
   int64_t rows;
   float eps;
 };
@@ -83,12 +84,25 @@ __global__ __launch_bounds__(256) void qkv_prep_kernel(PrepParams p) {
   float cs[8], sn[8];
   if (p.cos != nullptr) {
     int pos0 = p.pos0;
-    if (p.pos0_dev != nullptr) pos0 = max(0, min(p.pos0_dev[0], p.table_rows - p.T));
+    bool past_tables = false;
+    if (p.pos0_dev != nullptr) {
+      // Rows past the rotation tables read the tables' end (memory safety) and are reported: the status
+      // word gets its bit and the rotated outputs are NaN.
+      const int want = max(0, p.pos0_dev[0]);
+      past_tables = want > p.table_rows - p.T;
+      pos0 = min(want, p.table_rows - p.T);
+      if (past_tables && p.status != nullptr && blockIdx.x == 0 && threadIdx.x == 0)
+        __hip_atomic_fetch_or(p.status, DAISY_STATUS_POSITION_PAST_TABLES, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     const int64_t off = (int64_t)(pos0 + t) * HALF + 8 * c;
     const f32x4 c0 = *reinterpret_cast<const f32x4*>(p.cos + off), c1 = *reinterpret_cast<const f32x4*>(p.cos + off + 4);
     const f32x4 s0 = *reinterpret_cast<const f32x4*>(p.sin + off), s1 = *reinterpret_cast<const f32x4*>(p.sin + off + 4);
 #pragma unroll
     for (int e = 0; e < 4; ++e) { cs[e] = c0[e]; cs[4 + e] = c1[e]; sn[e] = s0[e]; sn[4 + e] = s1[e]; }
+    if (past_tables) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) cs[e] = __builtin_nanf("");
+    }
   }
 
   rms_normalise(ql, qh);
@@ -131,7 +145,7 @@ static int prep_launch(const void* q, const int64_t* q_strides,
                        const void* k, const int64_t* k_strides,
                        const void* v, const int64_t* v_strides,
                        const void* ve, const int64_t* ve_strides, const float* gate,
-                       const float* cos, const float* sin, int pos0, const int32_t* pos0_dev, int table_rows,
+                       const float* cos, const float* sin, int pos0, const int32_t* pos0_dev, int table_rows, int32_t* status,
                        void* q_out, const int64_t* q_out_strides,
                        void* k_out, const int64_t* k_out_strides,
                        void* v_out, const int64_t* v_out_strides,
@@ -166,7 +180,7 @@ static int prep_launch(const void* q, const int64_t* q_strides,
   p.ko = (uint16_t*)k_out; p.ko_sb = k_out_strides[0]; p.ko_st = k_out_strides[1]; p.ko_sh = k_out_strides[2];
   p.vo = (uint16_t*)v_out; p.vo_sb = v_out_strides[0]; p.vo_st = v_out_strides[1]; p.vo_sh = v_out_strides[2];
   p.B = B; p.T = T; p.H = H; p.pos0 = pos0; p.eps = eps;
-  p.pos0_dev = pos0_dev; p.table_rows = table_rows;
+  p.pos0_dev = pos0_dev; p.table_rows = table_rows; p.status = status;
   p.rows = (int64_t)B * T * H;
   const int lpr = D / 16;
   const int64_t nwg = (p.rows * lpr + 255) / 256;
@@ -187,7 +201,7 @@ extern "C" int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
                                   void* k_out, const int64_t* k_out_strides,
                                   void* v_out, const int64_t* v_out_strides,
                                   int B, int T, int H, int D, float eps, void* stream) {
-  return prep_launch(q, q_strides, k, k_strides, v, v_strides, ve, ve_strides, gate, cos, sin, pos0, nullptr, 0,
+  return prep_launch(q, q_strides, k, k_strides, v, v_strides, ve, ve_strides, gate, cos, sin, pos0, nullptr, 0, nullptr,
                      q_out, q_out_strides, k_out, k_out_strides, v_out, v_out_strides, B, T, H, D, eps, stream);
 }
 
@@ -195,7 +209,7 @@ extern "C" int daisy_qkv_prep_fwd_at(const void* q, const int64_t* q_strides,
                                      const void* k, const int64_t* k_strides,
                                      const void* v, const int64_t* v_strides,
                                      const void* ve, const int64_t* ve_strides, const float* gate,
-                                     const float* cos, const float* sin, const int32_t* pos0, int table_rows,
+                                     const float* cos, const float* sin, const int32_t* pos0, int table_rows, int32_t* status,
                                      void* q_out, const int64_t* q_out_strides,
                                      void* k_out, const int64_t* k_out_strides,
                                      void* v_out, const int64_t* v_out_strides,
@@ -203,6 +217,6 @@ extern "C" int daisy_qkv_prep_fwd_at(const void* q, const int64_t* q_strides,
   DAISY_CHECK_ARG(pos0 != nullptr, "qkv_prep_at: the device position pointer must be non-NULL");
   DAISY_CHECK_ARG(cos && sin, "qkv_prep_at: the rotary tables are required");
   DAISY_CHECK_ARG(table_rows >= T, "qkv_prep_at: table_rows=%d must cover the %d rows of the call", table_rows, T);
-  return prep_launch(q, q_strides, k, k_strides, v, v_strides, ve, ve_strides, gate, cos, sin, 0, pos0, table_rows,
+  return prep_launch(q, q_strides, k, k_strides, v, v_strides, ve, ve_strides, gate, cos, sin, 0, pos0, table_rows, status,
                      q_out, q_out_strides, k_out, k_out_strides, v_out, v_out_strides, B, T, H, D, eps, stream);
 }

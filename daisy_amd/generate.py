@@ -135,6 +135,9 @@ class Generator:
         # T x T mask, no [2, L, B, H, T, D] stack, every layer's keys and values go straight into
         # the cache (same requirements on the model as record_steps).
         self.direct_prefill = bool(direct_prefill)
+        # generate_batch: one bf16 ring, and one recorded step, per batch size
+        self._batch_caches: dict = {}
+        self._batch_steps: dict = {}
 
         torch.manual_seed(seed)
         self._tokens = torch.empty(256, dtype=torch.long, device=self.device)
@@ -280,20 +283,17 @@ class Generator:
         assert prompt_ids.ndim == 2 and prompt_ids.size(1) > 0 and max_new_tokens > 0
         ids = prompt_ids.to(self.device)
         B = ids.size(0)
-        cache = self._batch_caches.get(B) if hasattr(self, "_batch_caches") else None
+        cache = self._batch_caches.get(B)
         if cache is None:
-            cache = KVCache(L=self.cache.L, B=B, H=self.cache.H, W=self.cache.W, D=self.cache.D,
-                            device=self.device, dtype=torch.bfloat16)
-            self._batch_caches = {**getattr(self, "_batch_caches", {}), B: cache}
+            cache = self._batch_caches[B] = KVCache(L=self.cache.L, B=B, H=self.cache.H, W=self.cache.W, D=self.cache.D,
+                                                    device=self.device, dtype=torch.bfloat16)
         cache.reset_history()
-        self.model.reset_history() if hasattr(self.model, "reset_history") else None
+        self.model.reset_history()
         step = lambda tokens: core.step(self.model, tokens, cache)
         if record_steps:
-            recorded = getattr(self, "_recorded_steps", {})
-            if B not in recorded:
-                recorded[B] = core.GraphedStep(self.model, cache)
-                self._recorded_steps = recorded
-            step = recorded[B]
+            if B not in self._batch_steps:
+                self._batch_steps[B] = core.GraphedStep(self.model, cache)
+            step = self._batch_steps[B]
         logits, _ = core.prefill(self.model, ids, cache)
         seen = torch.empty(B, ids.size(1) + max_new_tokens, dtype=torch.long, device=self.device)
         seen[:, :ids.size(1)] = ids

@@ -11,7 +11,7 @@ writes the new row itself, and no chronological copy is ever made.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 from torch import Tensor
@@ -31,6 +31,9 @@ class RingContext:
     v: Tensor
     t: int
     W: int
+    # one int32 on the GPU in which a step whose position lives in device memory reports what the
+    # host cannot check beforehand (a position past the rotary tables); None = not wanted
+    status: Optional[Tensor] = None
 
     def mark_written(self) -> None:
         self.cache._staged[self.layer] = True

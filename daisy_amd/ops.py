@@ -36,6 +36,10 @@ def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *,
     counts the visible keys including the query itself (``None``/``<=0`` = full
     causal).  Returns ``(o, k_rot)``: ``o`` is ``[B, T, H, D]`` bf16 and ``k_rot``
     the rotated keys (``None`` without ``cos``/``sin``).
+
+    Contract of ``doc_start``: ``0 <= doc_start[t] <= t`` and non-decreasing in ``t`` (the kernel
+    picks the key tiles of a block of queries from the block's first row).  It is not checked
+    here, since that would synchronise; ``check_doc_start`` does, for callers that want it.
     """
     dev = _lib.require_gpu(q, k, v, cos, sin, doc_start, out, k_out)
     for name, t in (("q", q), ("k", k), ("v", v)):
@@ -77,6 +81,92 @@ def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *,
             B, T, H, D, w, float(scale), flags, _lib.current_stream(dev))
     _lib.check(rc, "daisy_prefill_fwd")
     return out, k_out
+
+
+def _check_f32(name: str, t: torch.Tensor, ndim: int) -> None:
+    if t.dtype != torch.float32:
+        raise TypeError(f"{name} must be float32, got {t.dtype}")
+    if t.dim() != ndim:
+        raise ValueError(f"{name} must have {ndim} dims, got shape {tuple(t.shape)}")
+    if t.stride(-1) != 1:
+        raise ValueError(f"{name} must be contiguous in its last dim")
+
+
+def prefill_attention_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *,
+                          window: Optional[int], scale: float = ATTN_SCALE,
+                          cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                          doc_start: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """``prefill_attention`` on fp32 ``[B, T, H, D]`` tensors with fp32 arithmetic (``daisy_prefill_fwd_f32``):
+    the mode of a module with fp32 parameters.  Any even ``D <= 256``.  Returns fp32 ``(o, k_rot)``."""
+    dev = _lib.require_gpu(q, k, v, cos, sin, doc_start)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_f32(name, t, 4)
+    B, T, H, D = q.shape
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError(f"q, k, v shapes differ: {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    if (cos is None) != (sin is None):
+        raise ValueError("cos and sin must be given together")
+    if cos is not None:
+        for name, t in (("cos", cos), ("sin", sin)):
+            if t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != D // 2 or not t.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous fp32 [rows, {D // 2}] table, got {tuple(t.shape)} {t.dtype}")
+            torch._assert(T <= t.shape[0], f"Rotary buffers too small {t.shape[0]} < {T}")
+    if doc_start is not None:
+        if doc_start.dtype != torch.int32 or doc_start.shape != (T,) or not doc_start.is_contiguous():
+            raise ValueError("doc_start must be a contiguous int32 [T] tensor")
+    out = torch.empty((B, T, H, D), dtype=torch.float32, device=dev)
+    k_out = torch.empty((B, T, H, D), dtype=torch.float32, device=dev) if cos is not None else None
+    d3 = (0, 1, 2)
+    lib = _lib.load()
+    with _lib.on_device(dev):
+        rc = lib.daisy_prefill_fwd_f32(
+            q.data_ptr(), _lib.strides(q, d3), k.data_ptr(), _lib.strides(k, d3), v.data_ptr(), _lib.strides(v, d3),
+            _lib.ptr(cos), _lib.ptr(sin), _lib.ptr(doc_start),
+            out.data_ptr(), _lib.strides(out, d3),
+            _lib.ptr(k_out), None if k_out is None else _lib.strides(k_out, d3),
+            B, T, H, D, 0 if window is None else int(window), float(scale), _lib.current_stream(dev))
+    _lib.check(rc, "daisy_prefill_fwd_f32")
+    return out, k_out
+
+
+def decode_attention_f32(q: torch.Tensor, k_new: torch.Tensor, v_new: torch.Tensor,
+                         k_rows: Optional[torch.Tensor], v_rows: Optional[torch.Tensor], *,
+                         n_rows: int, new_idx: int, scale: float = ATTN_SCALE,
+                         cos_row: Optional[torch.Tensor] = None, sin_row: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``decode_attention`` on fp32 tensors with fp32 arithmetic (``daisy_decode_fwd_f32``); the
+    cache rows ``[B, H, rows, D]`` are only read."""
+    dev = _lib.require_gpu(q, k_new, v_new, k_rows, v_rows, cos_row, sin_row)
+    for name, t in (("q", q), ("k_new", k_new), ("v_new", v_new)):
+        _check_f32(name, t, 3)
+    B, H, D = q.shape
+    if k_new.shape != q.shape or v_new.shape != q.shape:
+        raise ValueError("q, k_new, v_new must all be [B, H, D]")
+    if k_rows is not None:
+        _check_f32("k_rows", k_rows, 4)
+        _check_f32("v_rows", v_rows, 4)
+    out = torch.empty((B, H, D), dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    with _lib.on_device(dev):
+        rc = lib.daisy_decode_fwd_f32(
+            q.data_ptr(), _lib.strides(q, (0, 1)), k_new.data_ptr(), _lib.strides(k_new, (0, 1)),
+            v_new.data_ptr(), _lib.strides(v_new, (0, 1)),
+            _lib.ptr(k_rows), None if k_rows is None else _lib.strides(k_rows, (0, 1, 2)),
+            _lib.ptr(v_rows), None if v_rows is None else _lib.strides(v_rows, (0, 1, 2)),
+            _lib.ptr(cos_row), _lib.ptr(sin_row), out.data_ptr(), _lib.strides(out, (0, 1)),
+            B, H, D, int(n_rows), int(new_idx), 0, float(scale), _lib.current_stream(dev))
+    _lib.check(rc, "daisy_decode_fwd_f32")
+    return out
+
+
+def check_doc_start(doc_start: torch.Tensor) -> None:
+    """Raises ``ValueError`` unless ``0 <= doc_start[t] <= t`` and ``doc_start`` does not decrease
+    (the contract of ``prefill_attention``).  Synchronises with the device."""
+    pos = torch.arange(doc_start.numel(), device=doc_start.device, dtype=doc_start.dtype)
+    ok = (doc_start >= 0) & (doc_start <= pos)
+    if doc_start.numel() > 1:
+        ok[1:] &= doc_start[1:] >= doc_start[:-1]
+    if not bool(ok.all()):
+        raise ValueError("doc_start must satisfy 0 <= doc_start[t] <= t and must not decrease")
 
 
 def decode_workspace_bytes(B: int, H: int, D: int, n_rows: int, nsplit: int = 0) -> int:
@@ -185,7 +275,8 @@ def attn_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_ring: torch.T
               pos: Union[int, torch.Tensor], *, cos: torch.Tensor, sin: torch.Tensor, eps: float,
               ve: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
               scale: float = ATTN_SCALE, out: Optional[torch.Tensor] = None,
-              workspace: Optional[torch.Tensor] = None, nsplit: int = 0) -> torch.Tensor:
+              workspace: Optional[torch.Tensor] = None, nsplit: int = 0,
+              status: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The attention part of one decode step in one launch (``daisy_attn_step_fwd``).
 
     ``q``, ``k``, ``v``: the new token's rows of the QKV projection output, bf16 ``[B, H, D]`` views;
@@ -193,9 +284,14 @@ def attn_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_ring: torch.T
     ``[rows, D/2]``), mixes ``v`` with ``ve [B, H, D]`` through ``gate`` (one fp32), writes the new rows
     into slot ``pos % W`` of ``k_ring``/``v_ring [B, H, W, D]`` (bf16 or fp16) and attends the live rows.  ``pos`` is an
     int or a one-element int32 device tensor (read when the kernel runs).  Returns ``o [B, H, D]``.
+
+    ``status``: one-element int32 device tensor.  A device position past the rotary tables cannot
+    be refused on the host; the kernel then writes NaN outputs and raises bit
+    ``_lib.STATUS_POSITION_PAST_TABLES`` in ``status`` (see ``raise_for_status``).
     """
     pos_dev = pos if isinstance(pos, torch.Tensor) else None
-    dev = _lib.require_gpu(q, k, v, k_ring, v_ring, cos, sin, ve, gate, pos_dev, out, workspace)
+    dev = _lib.require_gpu(q, k, v, k_ring, v_ring, cos, sin, ve, gate, pos_dev, out, workspace, status)
+    _check_status(status)
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_bf16(name, t, 3)
     if k_ring.dtype == torch.float16 and v_ring.dtype == torch.float16 and k_ring.dim() == 4 and k_ring.stride(-1) == 1 \
@@ -242,7 +338,7 @@ def attn_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_ring: torch.T
             q.data_ptr(), _lib.strides(q, d2), k.data_ptr(), _lib.strides(k, d2), v.data_ptr(), _lib.strides(v, d2),
             _lib.ptr(ve), None if ve is None else _lib.strides(ve, d2), _lib.ptr(gate),
             cos.data_ptr(), sin.data_ptr(), int(cos.shape[0]),
-            0 if pos_dev is not None else int(pos), _lib.ptr(pos_dev), float(eps),
+            0 if pos_dev is not None else int(pos), _lib.ptr(pos_dev), _lib.ptr(status), float(eps),
             k_ring.data_ptr(), _lib.strides(k_ring, (0, 1, 2)), v_ring.data_ptr(), _lib.strides(v_ring, (0, 1, 2)),
             1 if ring_f16 else 0,
             out.data_ptr(), _lib.strides(out, d2), B, H, D, int(W), float(scale), int(nsplit),
@@ -251,17 +347,33 @@ def attn_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_ring: torch.T
     return out
 
 
+def _check_status(status: Optional[torch.Tensor]) -> None:
+    if status is not None and (status.dtype != torch.int32 or status.numel() != 1):
+        raise ValueError("status must be a one-element int32 tensor")
+
+
+def raise_for_status(status: torch.Tensor) -> None:
+    """Reads a status word (synchronises) and raises what the kernels reported in it."""
+    bits = int(status.item())
+    if bits & _lib.STATUS_POSITION_PAST_TABLES:
+        raise RuntimeError("a decode step ran at a position past the rotary tables (Rotary buffers too small); "
+                           "its outputs are NaN")
+
+
 def kda_workspace_bytes(B: int, T: int, H: int, Dk: int, Dv: int, chunk: int = 64) -> int:
     return int(_lib.load().daisy_kda_workspace_bytes(B, T, H, Dk, Dv, chunk))
 
 
-def kda_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, *,
-                  scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
-                  output_final_state: bool = False, use_qk_l2norm_in_kernel: bool = True,
-                  l2_eps: float = 1e-6, chunk: int = 64,
-                  workspace: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-    """Chunked KDA forward; see ``daisy_kda_chunk_fwd`` in ``include/daisy_hip.h``."""
-    dev = _lib.require_gpu(q, k, v, g, beta, initial_state, workspace)
+def _check_cu_seqlens(cu_seqlens: torch.Tensor, B: int) -> int:
+    """Validates what the host can see of packed-sequence bounds; returns the sequence count."""
+    if B != 1:
+        raise ValueError("cu_seqlens needs batch size 1 (sequences packed along T)")
+    if cu_seqlens.dtype != torch.int32 or cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2 or not cu_seqlens.is_contiguous():
+        raise ValueError("cu_seqlens must be a contiguous int32 [n_seq + 1] tensor")
+    return cu_seqlens.numel() - 1
+
+
+def _kda_inputs(q, k, v, g, beta, initial_state, n_states, scale, fresh_state_copy=True):
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_bf16(name, t, 4)
     B, T, H, Dk = q.shape
@@ -275,23 +387,50 @@ def kda_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
     if scale is None:
         scale = Dk ** -0.5
     if initial_state is not None:
-        if initial_state.shape != (B, H, Dk, Dv):
-            raise ValueError(f"initial_state must be [B,H,Dk,Dv], got {tuple(initial_state.shape)}")
-        initial_state = initial_state.to(torch.float32).contiguous()
-    o = torch.empty((B, T, H, Dv), dtype=torch.bfloat16, device=dev)
-    final = torch.empty((B, H, Dk, Dv), dtype=torch.float32, device=dev) if output_final_state else None
+        if initial_state.shape != (n_states, H, Dk, Dv):
+            raise ValueError(f"initial_state must be [{n_states},H,Dk,Dv], got {tuple(initial_state.shape)}")
+        if fresh_state_copy:
+            initial_state = initial_state.to(torch.float32).contiguous()
+    return q, k, v, g, beta, initial_state, scale
+
+
+def kda_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, *,
+                  scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
+                  output_final_state: bool = False, use_qk_l2norm_in_kernel: bool = True,
+                  l2_eps: float = 1e-6, chunk: int = 64, cu_seqlens: Optional[torch.Tensor] = None,
+                  workspace: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Chunked KDA forward; see ``daisy_kda_chunk_fwd`` / ``daisy_kda_chunk_varlen_fwd`` in ``include/daisy_hip.h``.
+
+    ``cu_seqlens`` (int32 ``[N + 1]`` on the GPU, from 0 to T, non-decreasing): the batch is 1 and
+    holds N sequences packed along T, each with its own state ``[N, H, Dk, Dv]``.  The kernels read
+    the bounds on the device; the host never does, so the call does not synchronise.
+    """
+    dev = _lib.require_gpu(q, k, v, g, beta, initial_state, workspace, cu_seqlens)
+    B, T, H, Dk = q.shape
+    Dv = v.shape[-1]
+    n_seq = _check_cu_seqlens(cu_seqlens, B) if cu_seqlens is not None else 0
+    n_states = n_seq if n_seq else B
+    q, k, v, g, beta, initial_state, scale = _kda_inputs(q, k, v, g, beta, initial_state, n_states, scale)
+    # rows that belong to no sequence (bounds that stop short of T) are not written by the kernels
+    o = (torch.zeros if n_seq else torch.empty)((B, T, H, Dv), dtype=torch.bfloat16, device=dev)
+    final = torch.empty((n_states, H, Dk, Dv), dtype=torch.float32, device=dev) if output_final_state else None
     lib = _lib.load()
-    need = int(lib.daisy_kda_workspace_bytes(B, T, H, Dk, Dv, chunk))
+    if n_seq:
+        need = int(lib.daisy_kda_varlen_workspace_bytes(T, n_seq, H, Dk, Dv, chunk))
+    else:
+        need = int(lib.daisy_kda_workspace_bytes(B, T, H, Dk, Dv, chunk))
     if need > 0 and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    with _lib.on_device(dev):
-        rc = lib.daisy_kda_chunk_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(),
-            g.data_ptr(), 1 if g.dtype == torch.bfloat16 else 0, beta.data_ptr(),
-            _lib.ptr(initial_state), o.data_ptr(), _lib.ptr(final),
-            B, T, H, Dk, Dv, int(chunk), float(scale), 1 if use_qk_l2norm_in_kernel else 0, float(l2_eps),
+    head = (q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), 1 if g.dtype == torch.bfloat16 else 0, beta.data_ptr())
+    tail = (int(chunk), float(scale), 1 if use_qk_l2norm_in_kernel else 0, float(l2_eps),
             _lib.ptr(workspace), ws_bytes, _lib.current_stream(dev))
+    with _lib.on_device(dev):
+        if n_seq:
+            rc = lib.daisy_kda_chunk_varlen_fwd(*head, cu_seqlens.data_ptr(), n_seq, _lib.ptr(initial_state), o.data_ptr(),
+                                                _lib.ptr(final), T, H, Dk, Dv, *tail)
+        else:
+            rc = lib.daisy_kda_chunk_fwd(*head, _lib.ptr(initial_state), o.data_ptr(), _lib.ptr(final), B, T, H, Dk, Dv, *tail)
     _lib.check(rc, "daisy_kda_chunk_fwd")
     return o, final
 
@@ -299,48 +438,40 @@ def kda_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Te
 def kda_recurrent_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, *,
                       scale: Optional[float] = None, initial_state: Optional[torch.Tensor] = None,
                       output_final_state: bool = True, use_qk_l2norm_in_kernel: bool = True,
-                      l2_eps: float = 1e-6, inplace_state: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+                      l2_eps: float = 1e-6, inplace_state: bool = False,
+                      cu_seqlens: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """Token-by-token KDA with the state in registers; see ``daisy_kda_recurrent_fwd``.
 
     With ``inplace_state`` the final state overwrites ``initial_state`` (which must then be a
     contiguous fp32 ``[B, H, Dk, Dv]`` tensor) and is returned as such -- the decode loop's mode.
+    ``cu_seqlens``: packed sequences as in ``kda_chunk_fwd``.
     """
-    dev = _lib.require_gpu(q, k, v, g, beta, initial_state)
-    for name, t in (("q", q), ("k", k), ("v", v)):
-        _check_bf16(name, t, 4)
+    dev = _lib.require_gpu(q, k, v, g, beta, initial_state, cu_seqlens)
     B, T, H, Dk = q.shape
     Dv = v.shape[-1]
-    if k.shape != q.shape or g.shape != q.shape or v.shape[:3] != q.shape[:3] or beta.shape != (B, T, H):
-        raise ValueError("kda: expected q,k,g [B,T,H,Dk], v [B,T,H,Dv], beta [B,T,H]")
-    if g.dtype not in (torch.float32, torch.bfloat16):
-        raise TypeError(f"g must be fp32 or bf16, got {g.dtype}")
-    q, k, v, g = q.contiguous(), k.contiguous(), v.contiguous(), g.contiguous()
-    beta = beta.to(torch.float32).contiguous()
-    if scale is None:
-        scale = Dk ** -0.5
-    if initial_state is not None:
-        if initial_state.shape != (B, H, Dk, Dv):
-            raise ValueError(f"initial_state must be [B,H,Dk,Dv], got {tuple(initial_state.shape)}")
-        if inplace_state:
-            if initial_state.dtype != torch.float32 or not initial_state.is_contiguous():
-                raise ValueError("inplace_state needs a contiguous fp32 initial_state")
-        else:
-            initial_state = initial_state.to(torch.float32).contiguous()
-    elif inplace_state:
-        raise ValueError("inplace_state needs an initial_state")
-    o = torch.empty((B, T, H, Dv), dtype=torch.bfloat16, device=dev)
+    n_seq = _check_cu_seqlens(cu_seqlens, B) if cu_seqlens is not None else 0
+    n_states = n_seq if n_seq else B
+    if inplace_state:
+        if initial_state is None:
+            raise ValueError("inplace_state needs an initial_state")
+        if initial_state.dtype != torch.float32 or not initial_state.is_contiguous():
+            raise ValueError("inplace_state needs a contiguous fp32 initial_state")
+    q, k, v, g, beta, initial_state, scale = _kda_inputs(q, k, v, g, beta, initial_state, n_states, scale,
+                                                         fresh_state_copy=not inplace_state)
+    o = (torch.zeros if n_seq else torch.empty)((B, T, H, Dv), dtype=torch.bfloat16, device=dev)
     if inplace_state:
         final = initial_state
     else:
-        final = torch.empty((B, H, Dk, Dv), dtype=torch.float32, device=dev) if output_final_state else None
+        final = torch.empty((n_states, H, Dk, Dv), dtype=torch.float32, device=dev) if output_final_state else None
     lib = _lib.load()
+    head = (q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), 1 if g.dtype == torch.bfloat16 else 0, beta.data_ptr())
+    tail = (float(scale), 1 if use_qk_l2norm_in_kernel else 0, float(l2_eps), _lib.current_stream(dev))
     with _lib.on_device(dev):
-        rc = lib.daisy_kda_recurrent_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(),
-            g.data_ptr(), 1 if g.dtype == torch.bfloat16 else 0, beta.data_ptr(),
-            _lib.ptr(initial_state), o.data_ptr(), _lib.ptr(final),
-            B, T, H, Dk, Dv, float(scale), 1 if use_qk_l2norm_in_kernel else 0, float(l2_eps),
-            _lib.current_stream(dev))
+        if n_seq:
+            rc = lib.daisy_kda_recurrent_varlen_fwd(*head, cu_seqlens.data_ptr(), n_seq, _lib.ptr(initial_state), o.data_ptr(),
+                                                    _lib.ptr(final), T, H, Dk, Dv, *tail)
+        else:
+            rc = lib.daisy_kda_recurrent_fwd(*head, _lib.ptr(initial_state), o.data_ptr(), _lib.ptr(final), B, T, H, Dk, Dv, *tail)
     _lib.check(rc, "daisy_kda_recurrent_fwd")
     return o, final
 
@@ -384,7 +515,8 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
              pos0: Union[int, torch.Tensor] = 0,
              ve: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
              q_out: Optional[torch.Tensor] = None, k_out: Optional[torch.Tensor] = None,
-             v_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+             v_out: Optional[torch.Tensor] = None, status: Optional[torch.Tensor] = None
+             ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """RMS norm of q, k, v + RoPE of q, k at rows ``pos0 + t`` + ``gate*v + (1-gate)*ve`` in one pass.
 
     ``q``, ``k``, ``v`` (and ``ve``) are bf16 ``[B, T, H, D]`` tensors or views with a
@@ -394,7 +526,8 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
 
     ``pos0`` may be a one-element int32 device tensor: the kernel then reads the position when
     it runs (a launch recorded in a HIP graph follows the tensor's value from replay to replay);
-    the caller keeps ``pos0 + T`` within the tables, which cannot be checked here.
+    ``pos0 + T`` beyond the tables cannot be refused here: the kernel then writes NaN for the rotated
+    outputs and raises ``_lib.STATUS_POSITION_PAST_TABLES`` in ``status`` (one-element int32 tensor).
     """
     pos_dev = pos0 if isinstance(pos0, torch.Tensor) else None
     if pos_dev is not None:
@@ -403,7 +536,8 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
         if cos is None:
             raise ValueError("a device position needs the rotary tables")
         pos0 = 0
-    dev = _lib.require_gpu(q, k, v, ve, gate, cos, sin, q_out, k_out, v_out, pos_dev)
+    dev = _lib.require_gpu(q, k, v, ve, gate, cos, sin, q_out, k_out, v_out, pos_dev, status)
+    _check_status(status)
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_bf16(name, t, 4)
     B, T, H, D = q.shape
@@ -444,75 +578,30 @@ def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
         if pos_dev is None:
             rc = lib.daisy_qkv_prep_fwd(*ins, int(pos0), *outs, _lib.current_stream(dev))
         else:
-            rc = lib.daisy_qkv_prep_fwd_at(*ins, pos_dev.data_ptr(), int(cos.shape[0]), *outs, _lib.current_stream(dev))
+            rc = lib.daisy_qkv_prep_fwd_at(*ins, pos_dev.data_ptr(), int(cos.shape[0]), _lib.ptr(status), *outs,
+                                           _lib.current_stream(dev))
     _lib.check(rc, "daisy_qkv_prep_fwd")
     return qo, ko, vo
 
 
-def probe_matrix_rate(with_vector_mix: bool, iters: int = 50000, workgroups: int = 256, device="cuda:0") -> dict:
-    """Sustained rate of register-only bf16 MFMAs on every SIMD (optionally with the attention loop's vector mix).
-
-    Returns ``{"ms", "tflops", "clock_mhz"}``; see ``daisy_probe_matrix_rate`` in ``include/daisy_hip.h``.
-    """
-    import ctypes
-    dev = torch.device(device)
-    sink = torch.empty(4096, dtype=torch.float32, device=dev)
-    ticks = torch.zeros(2 * workgroups, dtype=torch.int64, device=dev)
-    lib = _lib.load()
-    flop = ctypes.c_double(0.0)
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    with _lib.on_device(dev):
-        stream = _lib.current_stream(dev)
-        rc = lib.daisy_probe_matrix_rate(int(with_vector_mix), workgroups, max(iters // 10, 1), sink.data_ptr(),
-                                         ticks.data_ptr(), ctypes.byref(flop), stream)   # warm-up
-        _lib.check(rc, "daisy_probe_matrix_rate")
-        start.record()
-        rc = lib.daisy_probe_matrix_rate(int(with_vector_mix), workgroups, iters, sink.data_ptr(),
-                                         ticks.data_ptr(), ctypes.byref(flop), stream)
-        end.record()
-        _lib.check(rc, "daisy_probe_matrix_rate")
-        torch.cuda.synchronize(dev)
-    ms = start.elapsed_time(end)
-    t = ticks.view(workgroups, 2).double().sum(0)
-    return {"ms": ms, "tflops": flop.value / ms / 1e9, "clock_mhz": float(t[0] / t[1] * 100.0)}
-
-
-def probe_read_rate(gib: int = 2, workgroups: int = 8192, repeats: int = 5, device="cuda:0") -> dict:
-    """Read-only streaming rate of the GPU over a ``gib`` GiB buffer (``daisy_probe_read_rate``).
-
-    Returns ``{"ms", "bytes", "gbs"}`` (mean over ``repeats`` launches after one warm-up).
-    """
-    dev = torch.device(device)
-    nbytes = gib << 30
-    buf = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
-    sink = torch.empty(4096, dtype=torch.int32, device=dev)
-    lib = _lib.load()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    with _lib.on_device(dev):
-        stream = _lib.current_stream(dev)
-        _lib.check(lib.daisy_probe_read_rate(buf.data_ptr(), nbytes, workgroups, sink.data_ptr(), stream), "daisy_probe_read_rate")
-        start.record()
-        for _ in range(repeats):
-            _lib.check(lib.daisy_probe_read_rate(buf.data_ptr(), nbytes, workgroups, sink.data_ptr(), stream), "daisy_probe_read_rate")
-        end.record()
-        torch.cuda.synchronize(dev)
-    ms = start.elapsed_time(end) / repeats
-    return {"ms": ms, "bytes": nbytes, "gbs": nbytes / ms / 1e6}
-
-
 def short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                cache: Optional[torch.Tensor] = None, output_final_state: bool = False,
-               activation: Optional[str] = "silu", inplace_cache: bool = False
+               activation: Optional[str] = "silu", inplace_cache: bool = False,
+               cu_seqlens: Optional[torch.Tensor] = None
                ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """Depthwise causal convolution over time + SiLU for ``x [B, T, C]`` bf16 (``daisy_short_conv_fwd``).
 
     ``weight [C, 1, K]`` or ``[C, K]``; ``cache [B, C, K]`` holds the last K inputs of the sequence
     so far.  Returns ``(y [B, T, C], new cache or None)``.  ``inplace_cache``: the new window is
     written into ``cache`` itself (bf16, contiguous, ``T <= 32``: decode steps) and ``cache`` is returned.
+    ``cu_seqlens`` (int32 ``[N + 1]`` on the GPU): ``B == 1`` and N sequences are packed along T; no tap
+    reaches across the start of its sequence and the windows are ``[N, C, K]`` (``daisy_short_conv_varlen_fwd``).
     """
-    dev = _lib.require_gpu(x, weight, bias, cache)
+    dev = _lib.require_gpu(x, weight, bias, cache, cu_seqlens)
     _check_bf16("x", x, 3)
     B, T, C = x.shape
+    n_seq = _check_cu_seqlens(cu_seqlens, B) if cu_seqlens is not None else 0
+    n_win = n_seq if n_seq else B
     w = weight.reshape(C, -1)
     K = w.shape[1]
     if w.dtype != torch.bfloat16 or (bias is not None and bias.dtype != torch.bfloat16):
@@ -523,8 +612,8 @@ def short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
         x = x.contiguous()
     w = w.contiguous()
     if cache is not None:
-        if cache.shape != (B, C, K):
-            raise ValueError(f"short_conv: cache must be [{B}, {C}, {K}], got {tuple(cache.shape)}")
+        if cache.shape != (n_win, C, K):
+            raise ValueError(f"short_conv: cache must be [{n_win}, {C}, {K}], got {tuple(cache.shape)}")
         if inplace_cache and (cache.dtype != torch.bfloat16 or not cache.is_contiguous()):
             raise ValueError("short_conv: a window updated in place must be a contiguous bf16 tensor")
         cache = cache.to(torch.bfloat16).contiguous()
@@ -534,8 +623,20 @@ def short_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
     if inplace_cache:
         new_cache = cache
     else:
-        new_cache = torch.empty(B, C, K, dtype=torch.bfloat16, device=dev) if output_final_state else None
+        new_cache = torch.empty(n_win, C, K, dtype=torch.bfloat16, device=dev) if output_final_state else None
     lib = _lib.load()
+    if n_seq:
+        if inplace_cache:
+            raise ValueError("short_conv: inplace_cache does not combine with cu_seqlens")
+        if bias is not None:
+            bias = bias.contiguous()
+        with _lib.on_device(dev):
+            rc = lib.daisy_short_conv_varlen_fwd(x.data_ptr(), x.stride(1), w.data_ptr(), _lib.ptr(bias),
+                                                 cu_seqlens.data_ptr(), n_seq, _lib.ptr(cache),
+                                                 y.data_ptr(), y.stride(1), _lib.ptr(new_cache),
+                                                 T, C, K, 1 if activation == "silu" else 0, _lib.current_stream(dev))
+        _lib.check(rc, "daisy_short_conv_varlen_fwd")
+        return y, new_cache
     with _lib.on_device(dev):
         rc = lib.daisy_short_conv_fwd(x.data_ptr(), _lib.strides(x, (0, 1)), w.data_ptr(), _lib.ptr(bias), _lib.ptr(cache),
                                       y.data_ptr(), _lib.strides(y, (0, 1)), _lib.ptr(new_cache),

@@ -33,6 +33,10 @@ extern "C" {
 #define DAISY_ERR_WORKSPACE (-3)
 #define DAISY_ERR_LAUNCH (-4)
 
+/* Bits a kernel raises in a caller-supplied status word (int32 in device memory, never cleared by
+ * the library) when it meets a condition that only the device can see. */
+#define DAISY_STATUS_POSITION_PAST_TABLES 1   /* a position read from device memory lies past the rotation tables */
+
 /* Text of the last error raised on this thread ("" if none). */
 const char* daisy_last_error(void);
 
@@ -58,8 +62,11 @@ int daisy_abi_version(void);
  *              q and k are already rotated.  Row t rotates position t with
  *              y1 = x1*cos + x2*sin, y2 = -x1*sin + x2*cos on pairs (i, i+D/2).
  * doc_start  : int32 [T] or NULL; doc_start[t] = index of the first token of the
- *              document containing t (non-decreasing).  Shared by all batches,
- *              like the reference's [1,1,T,T] mask.
+ *              document containing t.  Contract: 0 <= doc_start[t] <= t and
+ *              non-decreasing in t (the kernel picks the key tiles of a block of
+ *              128 queries from the block's first row; a bound that decreases
+ *              inside a block silently drops keys, a bound beyond t gives NaN).
+ *              Shared by all batches, like the reference's [1,1,T,T] mask.
  * k_out      : bf16 [B, T, H, D] with its own strides, or NULL.  When cos/sin
  *              are given, receives the rotated keys (what the reference's
  *              prefill returns for the KV cache, attention.py:179); the
@@ -81,6 +88,22 @@ int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
                       void* k_out, const int64_t* k_out_strides,
                       int B, int T, int H, int D,
                       int window, float scale, int flags, void* stream);
+
+/* The same attention on fp32 tensors with fp32 arithmetic throughout (nothing is rounded to bf16):
+ * the mode of a module whose parameters are fp32, as the reference's own unit tests build it
+ * (tests/test_attention.py:9, compared at 1e-4).  Any even D <= 256; one wavefront per query, so
+ * this is a correctness path, not a fast one.  Strides in fp32 elements; k_out receives the
+ * rotated keys in fp32 when cos/sin are given.
+ */
+int daisy_prefill_fwd_f32(const float* q, const int64_t* q_strides,
+                          const float* k, const int64_t* k_strides,
+                          const float* v, const int64_t* v_strides,
+                          const float* cos, const float* sin,
+                          const int32_t* doc_start,
+                          float* o, const int64_t* o_strides,
+                          float* k_out, const int64_t* k_out_strides,
+                          int B, int T, int H, int D,
+                          int window, float scale, void* stream);
 
 /* ---------------------------------------------------------------------------
  * Kernel 2: split-K single-token decode over a bf16 KV cache.
@@ -124,6 +147,20 @@ int daisy_decode_fwd(const void* q, const int64_t* q_strides,
                      float scale, int nsplit,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* daisy_decode_fwd on fp32 tensors with fp32 arithmetic (see daisy_prefill_fwd_f32): any even
+ * D <= 256, one wavefront per (batch, head), no splits and no workspace.
+ */
+int daisy_decode_fwd_f32(const float* q, const int64_t* q_strides,
+                         const float* k_new, const int64_t* k_new_strides,
+                         const float* v_new, const int64_t* v_new_strides,
+                         float* k_cache, const int64_t* k_cache_strides,
+                         float* v_cache, const int64_t* v_cache_strides,
+                         const float* cos_row, const float* sin_row,
+                         float* o, const int64_t* o_strides,
+                         int B, int H, int D,
+                         int n_rows, int new_idx, int write_back,
+                         float scale, void* stream);
+
 /* The same decode step with the position held in device memory: `pos` points at one
  * int32 t (the number of tokens already in the ring, as DaisyCore.step's `pos`,
  * models/daisy/daisy_core.py:294-323, and KVCache.t, inference/kv_cache.py:52-55).  The
@@ -159,13 +196,16 @@ int daisy_decode_fwd_at(const void* q, const int64_t* q_strides,
  * fp32 sums inside the norm.  D is 64 or 128.  cache_is_f16: the ring holds fp16 rows (the
  * default cache dtype of the reference's Generator, inference/generate.py:62) instead of bf16;
  * the new rows are converted on their way in, which loses nothing for normalised rows.
+ * status: NULL, or one int32 in device memory.  A position read from pos_dev that lies past the
+ * tables (the reference asserts this on the host, attention.py:66) makes the kernel read the last
+ * table row, write NaN outputs for the step and raise DAISY_STATUS_POSITION_PAST_TABLES in *status.
  */
 int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
                         const void* k, const int64_t* k_strides,
                         const void* v, const int64_t* v_strides,
                         const void* ve, const int64_t* ve_strides, const float* gate,
                         const float* cos, const float* sin, int table_rows,
-                        int pos, const int32_t* pos_dev, float eps,
+                        int pos, const int32_t* pos_dev, int32_t* status, float eps,
                         void* k_cache, const int64_t* k_cache_strides,
                         void* v_cache, const int64_t* v_cache_strides, int cache_is_f16,
                         void* o, const int64_t* o_strides,
@@ -201,6 +241,25 @@ int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
                         float scale, int l2norm_qk, float l2_eps,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same forward over sequences packed along the token axis of a batch of one, the layout the
+ * reference hands to chunk_kda(..., cu_seqlens=...) for a padded batch
+ * (models/daisy/attention_kimi.py:133-134,150-154).  q, k, g: [T, H, Dk]; v, o: [T, H, Dv];
+ * beta: [T, H]; cu_seqlens: int32 [n_seq + 1] in device memory, sequence i = rows
+ * cu_seqlens[i] .. cu_seqlens[i+1] - 1, cu_seqlens[0] = 0, cu_seqlens[n_seq] = T, non-decreasing
+ * (empty sequences allowed).  The bounds are read by the kernels, never by the host; bounds that
+ * break the contract are forced into 0..T and rows that belong to no sequence are left unwritten.
+ * initial_state / final_state: fp32 [n_seq, H, Dk, Dv].
+ */
+size_t daisy_kda_varlen_workspace_bytes(int T, int n_seq, int H, int Dk, int Dv, int chunk);
+
+int daisy_kda_chunk_varlen_fwd(const void* q, const void* k, const void* v,
+                               const void* g, int g_is_bf16, const float* beta,
+                               const int32_t* cu_seqlens, int n_seq,
+                               const float* initial_state, void* o, float* final_state,
+                               int T, int H, int Dk, int Dv, int chunk,
+                               float scale, int l2norm_qk, float l2_eps,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------
  * Token-by-token KDA (the recurrence of daisy_kda_chunk_fwd evaluated one token
  * at a time, state in registers).  This is the "fused_recurrent" mode that
@@ -215,6 +274,15 @@ int daisy_kda_recurrent_fwd(const void* q, const void* k, const void* v,
                             const float* initial_state, void* o, float* final_state,
                             int B, int T, int H, int Dk, int Dv,
                             float scale, int l2norm_qk, float l2_eps, void* stream);
+
+/* daisy_kda_recurrent_fwd over packed sequences (layout and cu_seqlens as in
+ * daisy_kda_chunk_varlen_fwd; states [n_seq, H, Dk, Dv]). */
+int daisy_kda_recurrent_varlen_fwd(const void* q, const void* k, const void* v,
+                                   const void* g, int g_is_bf16, const float* beta,
+                                   const int32_t* cu_seqlens, int n_seq,
+                                   const float* initial_state, void* o, float* final_state,
+                                   int T, int H, int Dk, int Dv,
+                                   float scale, int l2norm_qk, float l2_eps, void* stream);
 
 /* ---------------------------------------------------------------------------
  * KDA log-decay gate:  out[..., h, d] = -exp(A_log[h]) * softplus(g[..., h, d] + bias[h, d])
@@ -260,14 +328,15 @@ int daisy_qkv_prep_fwd(const void* q, const int64_t* q_strides,
 /* The same pass with the first position read from device memory when the kernel runs
  * (`pos0` points at one int32; the decode-step counterpart of Rotary.step's host `pos`,
  * models/daisy/attention.py:64-70).  cos, sin are fp32 [table_rows, D/2] and required; a
- * position whose rows would leave the table is held at the table's end (memory safety
- * only: the caller keeps *pos0 + T <= table_rows).
+ * position whose rows would leave the table is held at the table's end, the rotated outputs of
+ * the call are NaN and, when status (one int32 in device memory) is given,
+ * DAISY_STATUS_POSITION_PAST_TABLES is raised in it.
  */
 int daisy_qkv_prep_fwd_at(const void* q, const int64_t* q_strides,
                           const void* k, const int64_t* k_strides,
                           const void* v, const int64_t* v_strides,
                           const void* ve, const int64_t* ve_strides, const float* gate,
-                          const float* cos, const float* sin, const int32_t* pos0, int table_rows,
+                          const float* cos, const float* sin, const int32_t* pos0, int table_rows, int32_t* status,
                           void* q_out, const int64_t* q_out_strides,
                           void* k_out, const int64_t* k_out_strides,
                           void* v_out, const int64_t* v_out_strides,
@@ -293,32 +362,22 @@ int daisy_short_conv_fwd(const void* x, const int64_t* x_strides, const void* we
                          const void* cache_in, void* y, const int64_t* y_strides, void* cache_out,
                          int B, int T, int C, int K, int apply_silu, void* stream);
 
+/* daisy_short_conv_fwd over sequences packed along T of a batch of one (the cu_seqlens argument of
+ * the reference's ShortConvolution calls, attention_kimi.py:155-158): no tap reaches across the
+ * start of its sequence.  x, y: [T, C] with a row stride; cu_seqlens as in
+ * daisy_kda_chunk_varlen_fwd; cache_in / cache_out: [n_seq, C, K] or NULL (must differ).
+ */
+int daisy_short_conv_varlen_fwd(const void* x, int64_t x_row_stride, const void* weight, const void* bias,
+                                const int32_t* cu_seqlens, int n_seq, const void* cache_in,
+                                void* y, int64_t y_row_stride, void* cache_out,
+                                int T, int C, int K, int apply_silu, void* stream);
+
 /* daisy_gated_rmsnorm_fwd: out = x * rsqrt(mean(x^2) + eps) * weight * sigmoid(gate) over the last
  * dim, statistics in fp32, one rounding.  x, gate, out: [rows, D] bf16 contiguous; weight: [D] bf16;
  * D = 64 or 128.
  */
 int daisy_gated_rmsnorm_fwd(const void* x, const void* gate, const void* weight, void* out,
                             int64_t rows, int D, float eps, void* stream);
-
-/* ---------------------------------------------------------------------------
- * Diagnostic (no counterpart in the reference): launches `workgroups` workgroups
- * of 8 wavefronts (two per SIMD) that each issue 8 * iters independent
- * v_mfma_f32_32x32x16_bf16 from registers -- alone (with_vector_mix = 0) or with
- * 5 fma + 1 exp2 between consecutive MFMAs, the ratio of the attention inner
- * loop (1).  The caller times the launch; *flop_out receives the flop count.
- * sink: 4096 floats of scratch; ticks: 2 uint64 per workgroup = (shader clock
- * counter, 100 MHz counter) deltas over the loop, i.e. the clock the chip ran at.
- */
-int daisy_probe_matrix_rate(int with_vector_mix, int workgroups, int iters,
-                            float* sink, unsigned long long* ticks, double* flop_out, void* stream);
-
-/* Diagnostic (no counterpart in the reference): `workgroups` workgroups of 256 threads read
- * `bytes` bytes of `buf` once (contiguous slab each, 8 x 16 bytes in flight per lane) and keep
- * nothing.  The caller times the launch: bytes / time is the read-only streaming rate of the
- * GPU, the practical ceiling for the decode kernel.  bytes must be a multiple of
- * workgroups x 32 KiB; sink: 4096 x 4 bytes of scratch.
- */
-int daisy_probe_read_rate(const void* buf, size_t bytes, int workgroups, void* sink, void* stream);
 
 #ifdef __cplusplus
 }

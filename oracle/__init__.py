@@ -23,10 +23,21 @@ live in ``tests/test_oracle_pins.py``):
   ``F.scaled_dot_product_attention`` with an explicit additive mask, the
   ``is_causal=True`` special case, and per-row brute force.
 * ``attn_prefill`` / ``attn_step``  -- the invariant "T steps == one prefill"
-  used by the reference's own tests, plus per-token windowed brute force.
+  used by the reference's own tests, plus per-token windowed brute force; their
+  value-embedding mix by known answers (gate logit +30 -> v, -30 -> ve, and the
+  reference's first-layer logit 0.3228 -> 0.58 v + 0.42 ve worked by hand).
+* ``block_mask_dense``              -- torch's own ``BlockMask.from_kv_blocks`` built
+  from block lists and expanded pair by pair with its ``mask_mod``.
+* ``block_mask_cycle``              -- literal per-layer lists for 1, 2, 4, 5 and 8 layers.
 * ``RingKVCache``                   -- the integer-valued scenarios of the
   reference's KV-cache tests (stored as data in ``tests/golden``).
 * ``kda_gate``                      -- ``F.softplus`` / ``exp`` closed form.
+* ``l2norm``                        -- hand-worked vectors ((3, 4) -> (0.6, 0.8)) and the
+  epsilon's place inside the square root.
+* ``short_conv`` / ``gated_rms_norm`` / ``kimi_layer_forward`` -- ``F.conv1d`` on an explicitly
+  padded sequence + ``F.silu``, brute-force tap loops, "two calls with the carried window == one
+  call", ``F.rms_norm`` with a weight times ``torch.sigmoid``.  PARITY UNPINNED against the
+  absent flash-linear-attention modules they restate (see ``oracle/kimi.py``).
 * ``kda_recurrent``                 -- closed forms (T=1, beta=0, g=0 cases),
   split-with-carried-state equivalence and an independent float64 loop.
   PARITY UNPINNED at one boundary: the third-party ``fla.ops.kda.chunk_kda``
@@ -53,3 +64,4 @@ from .attention import (  # noqa: F401
 )
 from .kv_cache import RingKVCache  # noqa: F401
 from .kda import kda_gate, kda_recurrent, l2norm  # noqa: F401
+from .kimi import short_conv, gated_rms_norm, kimi_layer_forward  # noqa: F401

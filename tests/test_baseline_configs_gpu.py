@@ -24,6 +24,25 @@ def _rope_base10000(D, T):
     return theta.cos(), theta.sin()
 
 
+def _library_windowed_attention(q, k, v, window, scale, rows_per_block=1024):
+    """EVERY row of windowed causal attention from the tensor library's fp32 ops on the GPU (matmul, softmax,
+    matmul over the keys a block of queries can see): the full-size second check next to the CPU oracle's
+    sampled rows.  q, k, v: [B, T, H, D] on the GPU; returns fp32 [B, T, H, D]."""
+    B, T, H, D = q.shape
+    W = T if window is None else window
+    out = torch.empty(B, T, H, D, dtype=torch.float32, device=q.device)
+    for b in range(B):
+        qf, kf, vf = (t[b].transpose(0, 1).float() for t in (q, k, v))            # [H, T, D]
+        for r0 in range(0, T, rows_per_block):
+            r1 = min(r0 + rows_per_block, T)
+            lo = max(0, r0 - W + 1)
+            s_ = torch.matmul(qf[:, r0:r1], kf[:, lo:r1].transpose(1, 2)) * scale   # [H, rows, keys]
+            d = torch.arange(r0, r1, device=q.device)[:, None] - torch.arange(lo, r1, device=q.device)[None, :]
+            s_.masked_fill_(((d < 0) | (d >= W))[None], float("-inf"))
+            out[b, r0:r1] = torch.matmul(torch.softmax(s_, dim=-1), vf[:, lo:r1]).transpose(0, 1)
+    return out
+
+
 def test_config2_windowed_prefill_full_size():
     """B8 T4096 d1024 H8 D128 W1024: merged QKV, q/k/v RMS-normed, RoPE base 10000, bf16."""
     B, T, H, D, W, dim = 8, 4096, 8, 128, 1024, 1024
@@ -48,6 +67,12 @@ def test_config2_windowed_prefill_full_size():
     qp, kp, vp = ops.qkv_prep(*qkv.chunk(3, dim=-2), eps=torch.finfo(torch.float32).eps, cos=cos.to(DEV), sin=sin.to(DEV))
     o2, _ = ops.prefill_attention(qp, kp, vp, window=W, scale=SCALE)
     assert_close_bf16(o2[:, rows.to(DEV)], ref.transpose(1, 2), "config 2 (prep kernel) o[rows]")
+    # every row of every (batch, head) against the library's fp32 ops on the GPU, itself checked against the
+    # CPU oracle on the sampled rows
+    lib = _library_windowed_attention(oracle.apply_rope(q, cos.to(DEV), sin.to(DEV)), k_rot, v, W, SCALE)
+    assert (lib[:, rows.to(DEV)].cpu() - ref.transpose(1, 2)).abs().max().item() <= 1e-4
+    mx, mn = assert_close_bf16(o, lib, "config 2 o, all rows")
+    say(f"config 2, all {B * T * H} rows against fp32 library ops: max-abs {mx:.2e} mean-abs {mn:.2e}")
 
 
 @pytest.mark.parametrize("window", [2048, None])
@@ -64,6 +89,21 @@ def test_config3_long_context_prefill_full_size(window):
     mx, mn = assert_close_bf16(o[:, rows.to(DEV)], ref.transpose(1, 2), f"config 3 window={window} o[rows]")
     say(f"config 3 window={window}: max-abs {mx:.2e} mean-abs {mn:.2e}")
     assert torch.isfinite(o.float()).all()
+    if window is not None:
+        # every row against the library's fp32 ops on the GPU (a block of queries sees at most 2 * window keys)
+        lib = _library_windowed_attention(q.to(DEV), k.to(DEV), v.to(DEV), window, SCALE, rows_per_block=2048)
+        assert (lib[:, rows.to(DEV)].cpu() - ref.transpose(1, 2)).abs().max().item() <= 1e-4
+        mx, mn = assert_close_bf16(o, lib, "config 3 window o, all rows")
+        say(f"config 3 window={window}, all {T * H} rows against fp32 library ops: max-abs {mx:.2e} mean-abs {mn:.2e}")
+    else:
+        # full causal: every 64th row (offset 37, so tile and block edges rotate through) against the same ops
+        sub = torch.arange(37, T, 64, device=DEV)
+        qf, kf, vf = (t.to(DEV)[0].transpose(0, 1).float() for t in (q, k, v))
+        for h0 in range(0, H, 4):
+            s_ = torch.matmul(qf[h0:h0 + 4][:, sub], kf[h0:h0 + 4].transpose(1, 2)) * SCALE
+            s_.masked_fill_((torch.arange(T, device=DEV)[None, :] > sub[:, None])[None], float("-inf"))
+            lib = torch.matmul(torch.softmax(s_, dim=-1), vf[h0:h0 + 4]).transpose(0, 1)        # [rows, 4, D]
+            assert_close_bf16(o[0, sub, h0:h0 + 4], lib, f"config 3 full causal, heads {h0}..{h0 + 3}, every 64th row")
 
 
 def test_config4_decode_full_size_256_steps():

@@ -6,6 +6,8 @@ import torch
 
 import oracle
 from daisy_amd import build_block_window_masks
+from daisy_amd.attention import block_mask_to_window, dense_mask_to_window
+from helpers import block_mask_pairs, flex_block_mask
 
 
 def _ids(T, p_eos, seed):
@@ -41,6 +43,64 @@ def test_document_boundaries_at_block_edges_and_single_document():
             pos = torch.arange(T)
             mine = (pos[None, :] >= lo[:, None]) & (pos[None, :] <= pos[:, None])
             assert torch.equal(mine, oracle.block_mask_dense(x, w, 1, block)), (eos_at, w)
+
+
+@pytest.mark.parametrize("p_eos", [0.0, 0.01, 0.1])
+@pytest.mark.parametrize("w", [1, 2, 3, 4])
+def test_oracle_block_mask_equals_the_library_block_mask(p_eos, w):
+    """Pins oracle.block_mask_dense against torch's own BlockMask.from_kv_blocks, expanded pair by pair."""
+    T, block = 512, 64
+    ids = _ids(T, p_eos, seed=17 + w)
+    bm = flex_block_mask(ids, w, eos=1, block=block)
+    assert torch.equal(oracle.block_mask_dense(ids, w, eos_token_id=1, block=block), block_mask_pairs(bm))
+
+
+@pytest.mark.parametrize("p_eos", [0.0, 0.02, 0.2])
+@pytest.mark.parametrize("w", [1, 2, 5])
+def test_a_library_block_mask_converts_to_the_same_row_bounds(p_eos, w):
+    """What CausalSelfAttention.forward does with the BlockMask the reference's training forward passes."""
+    T, block = 512, 64
+    ids = _ids(T, p_eos, seed=29 + w)
+    bm = flex_block_mask(ids, w, eos=1, block=block)
+    mask = block_mask_to_window(bm, pairs_per_pass=7)
+    lo = mask.doc_start.long()
+    assert mask.window is None and lo.dtype == torch.int64 and mask.doc_start.dtype == torch.int32
+    pos = torch.arange(T)
+    mine = (pos[None, :] >= lo[:, None]) & (pos[None, :] <= pos[:, None])
+    assert torch.equal(mine, block_mask_pairs(bm))
+    assert torch.equal(mask.doc_start, build_block_window_masks(ids, w, 1, eos_token_id=1, block=block)[0].doc_start)
+
+
+def test_block_masks_that_are_not_causal_bands_are_refused():
+    from torch.nn.attention.flex_attention import create_block_mask
+    T = 256
+    with pytest.raises(ValueError, match="one run of keys"):      # bidirectional: keys after the query
+        block_mask_to_window(create_block_mask(lambda b, h, q, k: (q - k).abs() < 40, 1, 1, T, T, device="cpu", BLOCK_SIZE=64))
+    with pytest.raises(ValueError, match="one run of keys"):      # a hole in the middle of the run
+        block_mask_to_window(create_block_mask(lambda b, h, q, k: (q >= k) & ((q - k) % 2 == 0), 1, 1, T, T, device="cpu", BLOCK_SIZE=64))
+    ok = block_mask_to_window(create_block_mask(lambda b, h, q, k: (q >= k) & (q - k < 100), 1, 1, T, T, device="cpu", BLOCK_SIZE=64))
+    assert ok.doc_start.tolist() == [max(0, q - 99) for q in range(T)]
+
+
+def test_dense_masks_with_a_bound_that_moves_backwards_are_refused():
+    T = 12
+    pos = torch.arange(T)
+    lo = torch.tensor([0, 0, 1, 2, 1, 2, 3, 4, 5, 6, 7, 8])      # row 4 sees one key more than row 3 allows
+    dense = torch.where((pos[None, :] >= lo[:, None]) & (pos[None, :] <= pos[:, None]), 0.0, float("-inf"))[None, None]
+    with pytest.raises(ValueError, match="decreases"):
+        dense_mask_to_window(dense)
+    lo[4] = 2
+    dense = torch.where((pos[None, :] >= lo[:, None]) & (pos[None, :] <= pos[:, None]), 0.0, float("-inf"))[None, None]
+    assert dense_mask_to_window(dense).doc_start.tolist() == lo.tolist()
+
+
+def test_long_short_cycle_literal_lists():
+    """models/daisy/daisy_core.py:224-229: long, short, short, short, ... and the last layer long."""
+    L_, S_ = 6, 3
+    want = {1: [L_], 2: [L_, L_], 4: [L_, S_, S_, L_], 5: [L_, S_, S_, S_, L_], 8: [L_, S_, S_, S_, L_, S_, S_, L_]}
+    for n_layers, widths in want.items():
+        assert oracle.block_mask_cycle(n_layers, 6) == widths
+    assert oracle.block_mask_cycle(4, 7) == [7, 3, 3, 7]          # short = long // 2
 
 
 def test_long_short_cycle():

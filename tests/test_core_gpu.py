@@ -355,3 +355,43 @@ def test_generator_generate_batch():
         batch = penalise_repeats(logits, recent, gen.rep_p_t.float())
         for r in range(B):
             assert torch.allclose(batch[r], penalise_repeats(logits[r], recent[r], gen.rep_p_t.float()), rtol=1e-6, atol=1e-6)
+
+
+def test_recorded_steps_survive_alternating_batch_sizes_on_a_hybrid_stack():
+    """A recorded step carries raw addresses of the KDA layer's state.  One sequence with recorded steps,
+    then a batch of four, then one sequence again: the states of the two batch sizes live in buffers of
+    their own, every recording is checked against the current addresses before it is replayed, and the
+    tokens equal those of steps launched kernel by kernel."""
+    import copy
+    from daisy_amd import Generator, KimiLinearSelfAttention
+    with torch.no_grad():
+        model = _Core(window=48, max_seq_len=512)
+        torch.manual_seed(2)
+        model.blocks[0].attn = KimiLinearSelfAttention(256, 2, 512, 128, receives_ve=True).bfloat16()
+        model = model.to(DEV)
+        twin = copy.deepcopy(model)
+        kw = dict(window=48, seed=5, device=torch.device(DEV), dtype=torch.bfloat16, temperature=0.0)
+        plain, recorded = Generator(model, **kw), Generator(twin, record_steps=True, direct_prefill=True, **kw)
+        g = torch.Generator().manual_seed(21)
+        one_a = torch.randint(2, 96, (33,), generator=g).to(DEV)
+        four = torch.randint(2, 96, (4, 27), generator=g).to(DEV)
+        one_b = torch.randint(2, 96, (40,), generator=g).to(DEV)
+        for round_ in range(2):
+            say(f"alternating batch sizes, round {round_}: one sequence")
+            assert torch.equal(torch.cat(list(recorded.generate(one_a, 16))), torch.cat(list(plain.generate(one_a, 16))))
+            state_1 = twin.blocks[0].attn._recurrent_state
+            say(f"alternating batch sizes, round {round_}: batch of four")
+            assert torch.equal(recorded.generate_batch(four, 12, record_steps=True), plain.generate_batch(four, 12))
+            assert twin.blocks[0].attn._recurrent_state.shape[0] == 4
+            say(f"alternating batch sizes, round {round_}: one sequence again")
+            assert torch.equal(torch.cat(list(recorded.generate(one_b, 16))), torch.cat(list(plain.generate(one_b, 16))))
+            # the one-sequence state went back into the buffer it had before the batch of four came by
+            assert twin.blocks[0].attn._recurrent_state.data_ptr() == state_1.data_ptr()
+        recorded._recorded_step.check()                      # no step ran past the rotary tables
+        # a step recorded without a prefill would capture the creation of the layer's state: refused
+        twin.reset_history()
+        twin.blocks[0].attn._state_homes.clear()
+        # (inference mode like the generators above: torch keeps per-capture generator state that must be
+        # touched in the mode it was created in)
+        with torch.inference_mode(), pytest.raises(RuntimeError, match="in place"):
+            core.GraphedStep(twin, KVCache(4, 1, 2, 48, 128, DEV, torch.bfloat16))(one_a[:1])

@@ -1,9 +1,11 @@
 """KimiLinearSelfAttention drop-in (models/daisy/attention_kimi.py:64-200) on the GPU.
 
-The layer's delta-rule core runs on the HIP kernels; here it is checked against the same layer
-evaluated on the CPU with the oracle's gate and naive fp32 recurrence in place of the kernels, and
-against itself: prompt + single-token steps must equal one full forward (the property the
-reference's tests/test_attention_kimi.py:161-219 checks with tolerances 2e-2 / 3e-2).
+The layer runs on the HIP kernels; here it is checked against the oracle's restatement of the
+layer (oracle/kimi.py: fp32 short convolutions, gate, naive recurrence, gated norm; the projections as
+library GEMMs on the CPU), and against itself: prompt + single-token steps must equal one full
+forward (the property the reference's tests/test_attention_kimi.py:161-219 checks with tolerances
+2e-2 / 3e-2).  The streaming kernels (short convolution, gated norm) and the packed-sequence
+(cu_seqlens) forms of all kernels are checked against the oracle one by one.
 """
 import pytest
 import torch
@@ -29,22 +31,11 @@ def _layer(dim=256, H=2, seed=0, receives_ve=False):
     return m.eval()
 
 
-def _cpu_reference(m, x, ve=None):
-    """The layer on the CPU: same PyTorch pieces, oracle gate + naive recurrence instead of the kernels."""
-    B, T, _ = x.shape
-    H, D = m.num_heads, m.head_k_dim
-    q, _ = m.q_conv1d(m.q_proj(x))
-    k, _ = m.k_conv1d(m.k_proj(x))
-    v, _ = m.v_conv1d(m.v_proj(x))
-    q, k, v = (t.view(B, T, H, D) for t in (q, k, v))
-    if m.receives_ve:
-        g_x = torch.sigmoid(m.g_ve).to(v.dtype)
-        v = g_x * v + (1.0 - g_x) * ve.view_as(v)
-    g = oracle.kda_gate(m.f_proj(x), m.A_log, D, m.dt_bias)
-    beta = torch.sigmoid(m.b_proj(x)).float()
-    o, _ = oracle.kda_recurrent(q, k, v, g.float(), beta, use_qk_l2norm=True)
-    o = m.o_norm(o.to(torch.bfloat16), m.g_proj(x).view(B, T, H, D))
-    return m.o_proj(o.reshape(B, T, H * D))
+def _cpu_reference(m, x, ve=None, cu_seqlens=None):
+    """The oracle's layer on the parameters of ``m`` (a CPU copy of the module, used as a parameter store only)."""
+    params = {k: v.detach() for k, v in m.state_dict().items()}
+    g_ve = float(m.g_ve) if m.receives_ve else None
+    return oracle.kimi_layer_forward(x, params, m.num_heads, m.head_k_dim, ve=ve, g_ve=g_ve, cu_seqlens=cu_seqlens)
 
 
 def _close(a, b, what, tol):
@@ -140,35 +131,62 @@ def test_padding_mask_packs_sequences():
 @pytest.mark.parametrize("B,T,C,K,bias,with_cache", [(2, 70, 256, 4, False, False), (1, 1, 64, 4, True, True),
                                                      (3, 33, 128, 3, True, True), (1, 200, 2048, 4, False, True),
                                                      (2, 2, 64, 2, False, True)])
-def test_short_convolution_kernel_matches_library_ops(B, T, C, K, bias, with_cache):
-    """The streaming kernel against the same module on the CPU (grouped conv1d + SiLU in bf16)."""
-    from daisy_amd.attention_kimi import ShortConvolution
-    torch.manual_seed(T + C)
-    m = ShortConvolution(C, K, bias=bias)
-    if bias:
-        with torch.no_grad():
-            m.bias.copy_((torch.randn(C) * 0.3).bfloat16())
-    x = torch.randn(B, T, C).bfloat16()
-    cache = torch.randn(B, C, K).bfloat16() if with_cache else None
-    with torch.no_grad():
-        y_ref, c_ref = m(x, cache, output_final_state=True)
-        md = ShortConvolution(C, K, bias=bias).to(DEV)
-        md.load_state_dict(m.state_dict())
-        y, c = md(x.to(DEV), None if cache is None else cache.to(DEV), output_final_state=True)
-    assert y.shape == (B, T, C) and c.shape == (B, C, K)
-    assert torch.equal(c.cpu(), c_ref), "carried window differs"
-    # identical up to one bf16 rounding of the pre-activation (the summation order may differ)
-    err = (y.float().cpu() - y_ref.float()).abs()
-    tol = 2.0 ** -7 * y_ref.float().abs().clamp_min(0.25)
-    say(f"short conv B{B} T{T} C{C} K{K}: max-abs {err.max().item():.3e}, mismatching {(err > 0).float().mean().item():.2%}")
+def test_short_convolution_kernel_matches_oracle(B, T, C, K, bias, with_cache):
+    """The streaming kernel against oracle.short_conv (fp32 taps + SiLU on the same bf16 inputs)."""
+    from daisy_amd import ops
+    g = torch.Generator().manual_seed(T + C)
+    w = (torch.randn(C, 1, K, generator=g) * 0.4).bfloat16()
+    bs = (torch.randn(C, generator=g) * 0.3).bfloat16() if bias else None
+    x = torch.randn(B, T, C, generator=g).bfloat16()
+    cache = torch.randn(B, C, K, generator=g).bfloat16() if with_cache else None
+    y_ref, c_ref = oracle.short_conv(x, w, bs, cache, output_final_state=True)
+    pre_ref, _ = oracle.short_conv(x, w, bs, cache, activation=None)
+    dev = lambda t: None if t is None else t.to(DEV)
+    y, c = ops.short_conv(dev(x), dev(w), dev(bs), dev(cache), True)
+    assert y.shape == (B, T, C) and c.shape == (B, C, K) and y.dtype == torch.bfloat16
+    assert torch.equal(c.cpu().float(), c_ref), "carried window differs"
+    # the kernel rounds the pre-activation to bf16, applies SiLU and rounds again: two bf16 roundings
+    # of values of the pre-activation's size against the unrounded oracle
+    err = (y.float().cpu() - y_ref).abs()
+    tol = 2.0 ** -7 * pre_ref.abs().clamp_min(0.25)
+    say(f"short conv B{B} T{T} C{C} K{K}: max-abs {err.max().item():.3e}")
     assert bool((err <= tol).all())
     # a sequence cut in two with the window carried equals the sequence in one go
     if T >= 2:
-        with torch.no_grad():
-            h = T // 2
-            y1, c1 = md(x[:, :h].to(DEV), None if cache is None else cache.to(DEV), output_final_state=True)
-            y2, c2 = md(x[:, h:].to(DEV), c1, output_final_state=True)
+        h = T // 2
+        y1, c1 = ops.short_conv(dev(x[:, :h]), dev(w), dev(bs), dev(cache), True)
+        y2, c2 = ops.short_conv(dev(x[:, h:]), dev(w), dev(bs), c1, True)
         assert torch.equal(torch.cat([y1, y2], dim=1), y) and torch.equal(c2, c)
+
+
+@pytest.mark.parametrize("K,bias,with_cache", [(4, False, False), (4, True, True), (3, False, True), (2, True, False)])
+def test_short_convolution_over_packed_sequences_matches_oracle(K, bias, with_cache):
+    """cu_seqlens read on the device: ragged sequences (one empty, some shorter than the window, boundaries
+    inside and at the edges of the kernel's 32-step segments) against the oracle's per-sequence loop."""
+    from daisy_amd import ops
+    g = torch.Generator().manual_seed(40 + K)
+    C = 136
+    lens = [5, 0, 1, 31, 32, 33, 2, 64, 70, 3]
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    T, N = int(cu[-1]), len(lens)
+    x = torch.randn(1, T, C, generator=g).bfloat16()
+    w = (torch.randn(C, 1, K, generator=g) * 0.4).bfloat16()
+    bs = (torch.randn(C, generator=g) * 0.3).bfloat16() if bias else None
+    cache = torch.randn(N, C, K, generator=g).bfloat16() if with_cache else None
+    y_ref, c_ref = oracle.short_conv(x, w, bs, cache, output_final_state=True, cu_seqlens=cu)
+    pre_ref, _ = oracle.short_conv(x, w, bs, cache, cu_seqlens=cu, activation=None)
+    dev = lambda t: None if t is None else t.to(DEV)
+    y, c = ops.short_conv(dev(x), dev(w), dev(bs), dev(cache), True, cu_seqlens=cu.to(DEV))
+    assert c.shape == (N, C, K)
+    assert torch.equal(c.cpu().float(), c_ref), "carried windows differ"
+    err = (y.float().cpu() - y_ref).abs()
+    assert bool((err <= 2.0 ** -7 * pre_ref.abs().clamp_min(0.25)).all()), err.max().item()
+    # each sequence alone through the plain kernel gives the same bits
+    for i in range(N):
+        s, e = int(cu[i]), int(cu[i + 1])
+        if e > s:
+            y_i, c_i = ops.short_conv(dev(x[:, s:e]), dev(w), dev(bs), None if cache is None else dev(cache[i:i + 1]), True)
+            assert torch.equal(y_i, y[:, s:e]) and torch.equal(c_i[0], c[i]), f"sequence {i}"
 
 
 def test_short_convolution_window_updated_in_place():
@@ -194,18 +212,92 @@ def test_short_convolution_window_updated_in_place():
 
 
 @pytest.mark.parametrize("rows,D", [(5, 128), (1000, 128), (77, 64)])
-def test_gated_rmsnorm_kernel_matches_formula(rows, D):
-    from daisy_amd.attention_kimi import GatedRMSNorm
-    torch.manual_seed(rows)
-    m = GatedRMSNorm(D)
-    with torch.no_grad():
-        m.weight.copy_((1 + 0.2 * torch.randn(D)).bfloat16())
-    x, g = torch.randn(rows, D).bfloat16() * 3, torch.randn(rows, D).bfloat16() * 2
-    with torch.no_grad():
-        ref = m(x, g)
-        md = GatedRMSNorm(D).to(DEV)
-        md.load_state_dict(m.state_dict())
-        out = md(x.to(DEV), g.to(DEV))
-    err = (out.float().cpu() - ref.float()).abs()
+def test_gated_rmsnorm_kernel_matches_oracle(rows, D):
+    from daisy_amd import ops
+    g = torch.Generator().manual_seed(rows)
+    w = (1 + 0.2 * torch.randn(D, generator=g)).bfloat16()
+    x, gate = torch.randn(rows, D, generator=g).bfloat16() * 3, torch.randn(rows, D, generator=g).bfloat16() * 2
+    ref = oracle.gated_rms_norm(x, gate, w, 1e-5)
+    out = ops.gated_rmsnorm(x.to(DEV), gate.to(DEV), w.to(DEV), 1e-5)
+    err = (out.float().cpu() - ref).abs()
     say(f"gated norm rows{rows} D{D}: max-abs {err.max().item():.3e}")
-    assert bool((err <= 2.0 ** -7 * ref.float().abs().clamp_min(1e-3)).all())
+    assert bool((err <= 2.0 ** -7 * ref.abs().clamp_min(1e-3)).all())      # one bf16 rounding of the result
+
+
+def test_layer_ops_refuse_cpu_tensors():
+    """One path: the layer's streaming ops raise for CPU tensors like every other op of the package."""
+    from daisy_amd.attention_kimi import GatedRMSNorm, ShortConvolution
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ShortConvolution(64, 4)(torch.zeros(1, 8, 64, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        GatedRMSNorm(128)(torch.zeros(4, 128, dtype=torch.bfloat16), torch.zeros(4, 128, dtype=torch.bfloat16))
+
+
+def _kda_pack(lens, H=2, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    T = sum(lens)
+    q = torch.randn(1, T, H, 128, generator=g).bfloat16()
+    k = torch.randn(1, T, H, 128, generator=g).bfloat16()
+    v = torch.randn(1, T, H, 128, generator=g).bfloat16()
+    gl = F.logsigmoid(torch.randn(1, T, H, 128, generator=g))
+    beta = torch.sigmoid(torch.randn(1, T, H, generator=g))
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    return q, k, v, gl, beta, cu
+
+
+@pytest.mark.parametrize("lens,with_state", [([200, 64, 1, 0, 130], True), ([63, 65], False), ([5], True),
+                                             ([0, 0, 70, 0], True), ([128, 128, 128], False)])
+def test_chunk_kda_over_packed_sequences_matches_oracle(lens, with_state):
+    """daisy_kda_chunk_varlen_fwd: the sequence boundaries are read by the kernels (no host loop, no
+    synchronisation); every sequence against the oracle's recurrence on its own slice."""
+    from daisy_amd import chunk_kda
+    q, k, v, gl, beta, cu = _kda_pack(lens, seed=len(lens))
+    N, H = len(lens), q.shape[2]
+    S0 = torch.randn(N, H, 128, 128, generator=torch.Generator().manual_seed(9)) * 0.1 if with_state else None
+    dev = lambda t: None if t is None else t.to(DEV)
+    o, S = chunk_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), initial_state=dev(S0), output_final_state=True,
+                     use_qk_l2norm_in_kernel=True, cu_seqlens=cu.to(DEV))
+    assert o.shape == q.shape and S.shape == (N, H, 128, 128)
+    for i in range(N):
+        s, e = int(cu[i]), int(cu[i + 1])
+        s0 = None if S0 is None else S0[i:i + 1]
+        if e == s:
+            want = s0 if s0 is not None else torch.zeros(1, H, 128, 128)
+            assert torch.equal(S[i:i + 1].cpu(), want), f"an empty sequence ({i}) must keep its state"
+            continue
+        o_ref, S_ref = oracle.kda_recurrent(q[:, s:e], k[:, s:e], v[:, s:e], gl[:, s:e], beta[:, s:e], initial_state=s0)
+        err = (o[:, s:e].float().cpu() - o_ref).abs()
+        assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3, (i, err.max().item())
+        rel = ((S[i:i + 1].cpu() - S_ref).norm() / S_ref.norm()).item()
+        assert rel <= 1e-3, (i, rel)
+
+
+def test_fused_recurrent_kda_over_packed_sequences_matches_oracle():
+    from daisy_amd import fused_recurrent_kda
+    lens = [7, 0, 1, 20]
+    q, k, v, gl, beta, cu = _kda_pack(lens, seed=5)
+    N, H = len(lens), q.shape[2]
+    S0 = torch.randn(N, H, 128, 128, generator=torch.Generator().manual_seed(3)) * 0.1
+    dev = lambda t: t.to(DEV)
+    o, S = fused_recurrent_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), initial_state=dev(S0), output_final_state=True,
+                               use_qk_l2norm_in_kernel=True, cu_seqlens=cu.to(DEV))
+    for i in range(N):
+        s, e = int(cu[i]), int(cu[i + 1])
+        o_ref, S_ref = oracle.kda_recurrent(q[:, s:e], k[:, s:e], v[:, s:e], gl[:, s:e], beta[:, s:e], initial_state=S0[i:i + 1])
+        if e > s:
+            assert (o[:, s:e].float().cpu() - o_ref).abs().max().item() <= 2e-2
+        assert ((S[i:i + 1].cpu() - S_ref).norm() / S_ref.norm()).item() <= 1e-3
+
+
+def test_packed_bounds_that_break_the_contract_stay_inside_the_tensors():
+    """Bounds are forced into 0..T and made non-decreasing on the device: nonsense in, no fault out."""
+    from daisy_amd import chunk_kda
+    q, k, v, gl, beta, _ = _kda_pack([150], seed=8)
+    bad = torch.tensor([5, -3, 90, 40, 10 ** 6], dtype=torch.int32)      # reads as 0, 5, 90, 90, 150 (running maximum)
+    dev = lambda t: t.to(DEV)
+    o, S = chunk_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), output_final_state=True, use_qk_l2norm_in_kernel=True,
+                     cu_seqlens=bad.to(DEV))
+    good = torch.tensor([0, 5, 90, 90, 150], dtype=torch.int32)
+    o2, S2 = chunk_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), output_final_state=True, use_qk_l2norm_in_kernel=True,
+                       cu_seqlens=good.to(DEV))
+    assert torch.equal(o, o2) and torch.equal(S, S2) and bool(torch.isfinite(o.float()).all())

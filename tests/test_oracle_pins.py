@@ -283,3 +283,122 @@ def test_kda_gate_closed_form():
     # the [1,1,H,1] A_log and per-head bias layouts the reference accepts
     out2 = oracle.kda_gate(g, A_log.view(1, 1, 2, 1), 4, torch.tensor([0.0, 1.0]))
     assert torch.allclose(out2, out)
+
+
+def test_l2norm_known_answers():
+    x = torch.tensor([[3.0, 4.0], [0.0, 0.0], [1e-3, 0.0]])
+    y = oracle.l2norm(x, eps=0.0)
+    assert torch.allclose(y[0], torch.tensor([0.6, 0.8]), atol=1e-7)
+    # the epsilon sits inside the square root: x / sqrt(sum(x^2) + eps)
+    y = oracle.l2norm(x, eps=1e-6)
+    assert y[1].abs().max().item() == 0.0
+    assert y[2, 0].item() == pytest.approx(1e-3 / math.sqrt(1e-6 + 1e-6), rel=1e-5)
+    # and it is what kda_recurrent applies to q and k
+    q, k, v, g, beta = _kda_inputs(T=3)
+    o1, S1 = oracle.kda_recurrent(q, k, v, g, beta, use_qk_l2norm=True, l2_eps=1e-6)
+    o2, S2 = oracle.kda_recurrent(oracle.l2norm(q), oracle.l2norm(k), v, g, beta, use_qk_l2norm=False)
+    assert torch.allclose(o1, o2, atol=1e-6) and torch.allclose(S1, S2, atol=1e-6)
+
+
+# ---- value-embedding mix (models/daisy/attention.py:132-135,186-190) --------------------------
+def _mix_case(g_ve, T=7, window=4):
+    w, x, ve, cos, sin, H, D = _module_inputs(T, seed=11)
+    y, k, v = oracle.attn_prefill(x, w, H, D, cos, sin, window, ve=ve, g_ve=g_ve)
+    _, _, v_plain = oracle.attn_prefill(x, w, H, D, cos, sin, window)             # no mix: v = norm(v)
+    return v, v_plain, ve.view(1, T, H, D).transpose(1, 2), (w, x, ve, cos, sin, H, D, y)
+
+
+def test_value_embedding_mix_known_answers_in_prefill():
+    v, v_plain, ve_, _ = _mix_case(30.0)          # sigmoid(30) = 1 in fp32: v untouched
+    assert torch.equal(v, v_plain)
+    v, v_plain, ve_, _ = _mix_case(-30.0)         # sigmoid(-30) ~ 1e-13: ve takes over
+    assert torch.allclose(v, ve_, atol=1e-6)
+    # the reference's first-layer gate logit (attention.py:96): sigmoid(0.3228) = 0.58 by hand
+    g = 1.0 / (1.0 + math.exp(-0.3228))
+    assert g == pytest.approx(0.58, abs=1e-4)
+    v, v_plain, ve_, _ = _mix_case(0.3228)
+    assert torch.allclose(v, 0.58 * v_plain + 0.42 * ve_, atol=2e-4)
+    assert not torch.allclose(v, 0.42 * v_plain + 0.58 * ve_, atol=1e-2)          # the swapped gate is visibly different
+
+
+def test_value_embedding_mix_known_answers_in_step():
+    T, window = 6, 4
+    for g_ve, a, b in ((30.0, 1.0, 0.0), (-30.0, 0.0, 1.0), (0.3228, 0.58, 0.42)):
+        w, x, ve, cos, sin, H, D = _module_inputs(T, seed=12)
+        k_ctx = torch.randn(1, 3, H, D, generator=torch.Generator().manual_seed(1))
+        v_ctx = torch.randn(1, 3, H, D, generator=torch.Generator().manual_seed(2))
+        _, _, v_new = oracle.attn_step(x[:, 3:4], k_ctx, v_ctx, 3, w, H, D, cos, sin, window, ve=ve[:, 3:4], g_ve=g_ve)
+        _, _, v_plain = oracle.attn_step(x[:, 3:4], k_ctx, v_ctx, 3, w, H, D, cos, sin, window)
+        want = a * v_plain + b * ve[:, 3:4].view(1, 1, H, D)
+        assert torch.allclose(v_new, want, atol=2e-4), g_ve
+        # and the mixed value is what the step attends: with one cached row removed from play
+        # (window 1) the output is o_proj(v_new)
+        y1, _, v1 = oracle.attn_step(x[:, 3:4], k_ctx, v_ctx, 3, w, H, D, cos, sin, 1, ve=ve[:, 3:4], g_ve=g_ve)
+        assert torch.allclose(y1, F.linear(v1.reshape(1, 1, H * D), w[3]), atol=1e-5)
+
+
+# ---- the KDA layer's neighbours (models/daisy/attention_kimi.py:41-62,90-92,155-158) ----------
+def test_short_conv_matches_library_conv_and_silu():
+    g = torch.Generator().manual_seed(20)
+    B, T, C, K = 2, 19, 6, 4
+    x = torch.randn(B, T, C, generator=g)
+    w = torch.randn(C, 1, K, generator=g)
+    bias = torch.randn(C, generator=g)
+    y, cache = oracle.short_conv(x, w, bias, output_final_state=True)
+    padded = F.pad(x.transpose(1, 2), (K - 1, 0))                       # K-1 zeros before the sequence
+    want = F.silu(F.conv1d(padded, w, bias, groups=C)).transpose(1, 2)
+    assert torch.allclose(y, want, atol=1e-5)
+    assert torch.equal(cache, x[:, -K:].transpose(1, 2))                # the last K inputs, [B, C, K]
+    y_lin, _ = oracle.short_conv(x, w, None, activation=None)
+    assert torch.allclose(y_lin, F.conv1d(padded, w, None, groups=C).transpose(1, 2), atol=1e-5)
+
+
+def test_short_conv_brute_force_taps():
+    g = torch.Generator().manual_seed(21)
+    T, C, K = 7, 3, 4
+    x = torch.randn(1, T, C, generator=g)
+    w = torch.randn(C, K, generator=g)
+    win = torch.randn(1, C, K, generator=g)
+    y, _ = oracle.short_conv(x, w, cache=win, activation=None)
+    for t in range(T):
+        for c in range(C):
+            acc = 0.0
+            for j in range(K):
+                ti = t - (K - 1) + j                                     # the last tap multiplies the current input
+                xin = float(x[0, ti, c]) if ti >= 0 else float(win[0, c, K + ti])
+                acc += float(w[c, j]) * xin
+            assert y[0, t, c].item() == pytest.approx(acc, abs=1e-5)
+
+
+def test_short_conv_carried_window_and_packed_sequences():
+    g = torch.Generator().manual_seed(22)
+    T, C, K = 23, 8, 4
+    x = torch.randn(1, T, C, generator=g)
+    w = torch.randn(C, 1, K, generator=g)
+    whole, cache = oracle.short_conv(x, w, output_final_state=True)
+    for cut in (1, 2, 3, 9):                                             # also cuts shorter than the window
+        y1, c1 = oracle.short_conv(x[:, :cut], w, output_final_state=True)
+        y2, c2 = oracle.short_conv(x[:, cut:], w, cache=c1, output_final_state=True)
+        assert torch.allclose(torch.cat([y1, y2], 1), whole, atol=1e-6) and torch.allclose(c2, cache)
+    cu = torch.tensor([0, 5, 5, 6, 23])
+    packed, caches = oracle.short_conv(x, w, output_final_state=True, cu_seqlens=cu)
+    for i in range(4):
+        s, e = int(cu[i]), int(cu[i + 1])
+        if e > s:
+            alone, c = oracle.short_conv(x[:, s:e], w, output_final_state=True)
+            assert torch.allclose(packed[:, s:e], alone, atol=1e-6) and torch.allclose(caches[i], c[0])
+        else:
+            assert caches[i].abs().max().item() == 0.0                   # an empty sequence keeps its (zero) window
+
+
+def test_gated_rms_norm_matches_library_pieces():
+    g = torch.Generator().manual_seed(23)
+    x = torch.randn(3, 5, 2, 128, generator=g) * 3
+    gate = torch.randn(3, 5, 2, 128, generator=g) * 2
+    w = 1 + 0.1 * torch.randn(128, generator=g)
+    want = F.rms_norm(x, (128,), w, 1e-5) * torch.sigmoid(gate)
+    assert torch.allclose(oracle.gated_rms_norm(x, gate, w, 1e-5), want, atol=1e-5)
+    # eps matters for small rows and sits under the mean of squares
+    tiny = torch.full((1, 128), 1e-3)
+    out = oracle.gated_rms_norm(tiny, torch.zeros(1, 128), torch.ones(128), 1e-5)
+    assert out[0, 0].item() == pytest.approx(0.5 * 1e-3 / math.sqrt(1e-6 + 1e-5), rel=1e-5)

@@ -57,6 +57,14 @@ SIGNATURES = {
         c_int, c_int, c_int,                                    # B, H, D
         c_int, c_int, c_int,                                    # n_rows, new_idx, write_back
         c_float, c_void_p]),                                    # scale, stream
+    "daisy_decode_fwd_noalloc": (c_int, [
+        c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k_new, v_new (+strides)
+        c_void_p, _I64P, c_void_p, _I64P,                       # k_cache, v_cache (+strides)
+        c_void_p, c_void_p,                                     # cos_row, sin_row
+        c_void_p, _I64P,                                        # o (+strides)
+        c_int, c_int, c_int,                                    # B, H, D
+        c_int, c_int, c_int,                                    # n_rows, new_idx, write_back
+        c_float, c_int, c_void_p]),                             # scale, nsplit, stream
     "daisy_decode_fwd_at": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k_new, v_new (+strides)
         c_void_p, _I64P, c_void_p, _I64P,                       # k_cache, v_cache (+strides)

@@ -19,6 +19,8 @@
 // recorded launch (HIP graph) can be replayed for every later token.
 #include "common.h"
 
+#include <mutex>
+
 namespace daisy {
 
 struct DecodeParams {
@@ -629,6 +631,69 @@ extern "C" int daisy_decode_fwd(const void* q, const int64_t* q_strides,
   return decode_launch(q, q_strides, k_new, k_new_strides, v_new, v_new_strides, k_cache, k_cache_strides,
                        v_cache, v_cache_strides, cos_row, sin_row, o, o_strides, B, H, D, n_rows, new_idx, nullptr,
                        write_back, scale, nsplit, workspace, workspace_bytes, stream);
+}
+
+// ---- the entry point that allocates nothing ----------------------------------------------------
+// The split partials of daisy_decode_fwd_noalloc live in this array of the library's device image.
+// In host code the array's name is only a stand-in: the address a kernel can use comes from
+// hipGetSymbolAddress, once per device (each GPU holds its own copy at its own address).
+static __device__ __align__(256) unsigned char scratch[DAISY_DECODE_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device (looked up on the first call there).
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("decode_noalloc: cannot identify the current device (%s)", e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+    return DAISY_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      set_error("decode_noalloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return DAISY_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return DAISY_OK;
+}
+}  // namespace
+
+extern "C" int daisy_decode_fwd_noalloc(const void* q, const int64_t* q_strides,
+                                        const void* k_new, const int64_t* k_new_strides,
+                                        const void* v_new, const int64_t* v_new_strides,
+                                        void* k_cache, const int64_t* k_cache_strides,
+                                        void* v_cache, const int64_t* v_cache_strides,
+                                        const float* cos_row, const float* sin_row,
+                                        void* o, const int64_t* o_strides,
+                                        int B, int H, int D,
+                                        int n_rows, int new_idx, int write_back,
+                                        float scale, int nsplit, void* stream) {
+  const size_t need = daisy_decode_workspace_bytes(B, H, D, n_rows, nsplit);
+  if (need > DAISY_DECODE_STATIC_SCRATCH_BYTES) {
+    set_error("decode_noalloc: %zu bytes of split partials needed (B=%d, H=%d, D=%d, n_rows=%d, nsplit=%d), the built-in "
+              "buffer holds %u; use daisy_decode_fwd with a workspace or fewer splits",
+              need, B, H, D, n_rows, nsplit, (unsigned)DAISY_DECODE_STATIC_SCRATCH_BYTES);
+    return DAISY_ERR_WORKSPACE;
+  }
+  void* ws = nullptr;
+  if (need > 0) {
+    const int rc = static_scratch(&ws);
+    if (rc != DAISY_OK) return rc;
+  }
+  // Every split writes its whole partial before the combine kernel reads it: nothing of the last
+  // call's contents is ever read, so nothing needs clearing.
+  return decode_launch(q, q_strides, k_new, k_new_strides, v_new, v_new_strides, k_cache, k_cache_strides,
+                       v_cache, v_cache_strides, cos_row, sin_row, o, o_strides, B, H, D, n_rows, new_idx, nullptr,
+                       write_back, scale, nsplit, ws, need, stream);
 }
 
 extern "C" int daisy_decode_fwd_f32(const float* q, const int64_t* q_strides,

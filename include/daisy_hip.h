@@ -161,6 +161,27 @@ int daisy_decode_fwd_f32(const float* q, const int64_t* q_strides,
                          int n_rows, int new_idx, int write_back,
                          float scale, void* stream);
 
+/* daisy_decode_fwd for callers that cannot allocate device memory or pass a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart
+ * in the reference.  The split partials live in a buffer of DAISY_DECODE_STATIC_SCRATCH_BYTES that
+ * is part of the library's device image (each GPU the library runs on holds one copy until the
+ * process ends); the call allocates nothing and fails with DAISY_ERR_WORKSPACE when
+ * daisy_decode_workspace_bytes(B, H, D, n_rows, nsplit) exceeds that size.  All calls on one GPU
+ * share the buffer: calls that overlap on one GPU (different streams) race and must be ordered by
+ * the caller.  Same results as daisy_decode_fwd.
+ */
+#define DAISY_DECODE_STATIC_SCRATCH_BYTES (4u << 20)
+int daisy_decode_fwd_noalloc(const void* q, const int64_t* q_strides,
+                             const void* k_new, const int64_t* k_new_strides,
+                             const void* v_new, const int64_t* v_new_strides,
+                             void* k_cache, const int64_t* k_cache_strides,
+                             void* v_cache, const int64_t* v_cache_strides,
+                             const float* cos_row, const float* sin_row,
+                             void* o, const int64_t* o_strides,
+                             int B, int H, int D,
+                             int n_rows, int new_idx, int write_back,
+                             float scale, int nsplit, void* stream);
+
 /* The same decode step with the position held in device memory: `pos` points at one
  * int32 t (the number of tokens already in the ring, as DaisyCore.step's `pos`,
  * models/daisy/daisy_core.py:294-323, and KVCache.t, inference/kv_cache.py:52-55).  The

@@ -605,6 +605,10 @@ def main():
             "what": "register-only v_mfma_f32_32x32x16_bf16 on every SIMD, 2 wavefronts each, ~25 ms per run",
             "mfma_only": probe_matrix_rate(False, 80000),
             "mfma_with_attention_vector_mix": probe_matrix_rate(True, 60000),
+            "mfma_with_attention_mix_and_lds_operands": dict(
+                probe_matrix_rate(2, 50000),
+                what="per MFMA 3 fma + 1 exp2, A operands read from LDS with the kernel's K / V access patterns eight "
+                     "MFMAs ahead; no global memory, barriers or masks: the stream ceiling of the two-wavefronts-per-SIMD layout"),
         }
     if want("plumbing"):
         extra["plumbing_c1"] = bench_plumbing_c1(args.steps, args.warmup, cpu)

@@ -229,10 +229,10 @@ def cpu_prefill_baseline(q, k, v, cos, sin, W, sample):
 
 
 # HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (profiles/prefill_pipe_kernel_c2_hbm_traffic.txt), each scaled by the factor the same counter
+# (profiles/prefill_tile_kernel_c2_hbm_traffic.txt), each scaled by the factor the same counter
 # shows for the 1 GiB copy of `--only copy` (2.000 for reads, 1.000 for writes).
 PREFILL_C2_TRAFFIC_BYTES = (127271 * 2 + 65542) * 1024
-PREFILL_C2_TRAFFIC_SOURCE = ("recorded counter value from profiles/prefill_pipe_kernel_c2_hbm_traffic.txt "
+PREFILL_C2_TRAFFIC_SOURCE = ("recorded counter value from profiles/prefill_tile_kernel_c2_hbm_traffic.txt "
                              "(rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this kernel on this workload); not measured by this run")
 
 
@@ -645,7 +645,7 @@ def main():
         line["roofline"] = {"bound": "mfma", "achieved": min(burst, sus), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                             "frac": min(burst, sus) / PEAK_BF16_TFLOPS, "traffic": PREFILL_C2_TRAFFIC_BYTES,
                             "traffic_source": PREFILL_C2_TRAFFIC_SOURCE, "traffic_min_bytes": head["min_hbm_bytes"],
-                            "kernel": "prefill_pipe_kernel<128>",
+                            "kernel": "prefill_tile_kernel<128>",
                             "ms": head["sustained"]["ms_kernel"] if use_sus else head["ms_kernel"],
                             "timing": ("sustained: mean over %d back-to-back launches (%.2f s)" % (head["sustained"]["launches"], head["sustained"]["seconds"]))
                                       if use_sus else "median of per-launch HIP event pairs over the timed steps",

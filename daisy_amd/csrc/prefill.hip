@@ -2,8 +2,9 @@
 //
 // Work decomposition
 //   workgroup = 4 wavefronts = 128 consecutive query rows of one (batch, head);
-//   wavefront = 32 query rows.  Key/value rows are visited in tiles of 64, and
-//   only tiles that intersect [lo(q_first), q_last] are loaded at all, where
+//   wavefront = 32 query rows.  Key/value rows are visited in tiles (32 rows in
+//   prefill_tile_kernel, 64 in prefill_mfma_kernel), and only tiles that intersect
+//   [lo(q_first), q_last] are loaded at all, where
 //   lo(q) = max(q - window + 1, doc_start[q], 0) is non-decreasing in q.
 //
 // MFMA formulation (v_mfma_f32_32x32x16_bf16, wave64)
@@ -18,7 +19,7 @@
 //   A and B operands agree, so the V^T operand simply fetches, per lane, the key
 //   rows 16m + 8g + 4*(l/32) + 0..3 that the lane's P registers hold.
 //
-// LDS (double buffered): K and V tiles [64][D] bf16, row major, filled by direct
+// LDS (double buffered): K and V tiles [rows][D] bf16, row major, filled by direct
 // global->LDS copies (global_load_lds_dwordx4: no staging registers, no LDS
 // store instructions); the 16-byte chunks of each row are XOR-swizzled so that
 // operand reads are bank-conflict free.  V^T operands come out of the row-major
@@ -27,8 +28,8 @@
 // lanes L/4, L/4+4, L/4+8, L/4+12; with lane i of a block addressing key i/4,
 // channels 4*(i%4)..+3, lane i receives channel i of four consecutive keys.
 //
-// Two kernels share this structure: prefill_pipe_kernel (keys need no rotation
-// here; software pipelined) and prefill_mfma_kernel<D, true> (keys are rotated
+// Two kernels share this structure: prefill_tile_kernel (keys need no rotation
+// here; three wavefronts per SIMD) and prefill_mfma_kernel<D, true> (keys are rotated
 // while they are staged into LDS).
 //
 // Algorithmic work: 4*D flops per visible (query, key) pair.
@@ -47,7 +48,7 @@ struct PrefillParams {
   uint16_t* o; int64_t o_sb, o_st, o_sh;
   uint16_t* k_out; int64_t ko_sb, ko_st, ko_sh;
   int B, T, H, D, window, nqb;
-  int period;    // tiles in a full window's range (0 = no window): the rotation period of the tile order
+  int period;    // 32-key tiles in a full window's range (0 = no window): the rotation period of the tile order
   int n_light;   // leading query blocks that see fewer keys than a full window (0 = order by block only)
   float scale_log2e;
 };
@@ -465,21 +466,22 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
   }
 }
 
-// Software-pipelined variant (keys already rotated or no RoPE on keys): the O^T += V^T P^T
-// product of tile i-1 is issued in the same basic block as the softmax of tile i, so the matrix
-// pipe works while the vector ALU does max / exp2 / sum / convert, inside one wavefront and
-// not only across the two wavefronts that share a SIMD.  V therefore runs one tile behind K:
-//   iteration i:  copies  K(i+1) -> Kbuf[(i+1)&1],  V(i) -> Vbuf[i&1]
-//                 S(i) = K(i) Q^T;   then   O += V(i-1)^T P(i-1)  ||  P(i) = softmax(S(i))
-// A rescale of O that the softmax of tile i asks for is applied at the start of the next fused
-// block (before P(i) is accumulated), which keeps that block free of branches.
-// A wavefront works on the contiguous tile range [tw_lo, tw_hi] that its 32 queries can see
-// (inside the workgroup's range); both 32-key halves of a tile in that range are computed and
-// masked per element where needed.
+// Main kernel (keys already rotated, or no RoPE on keys).  32-key tiles, and nothing of a step is
+// overlapped inside a wavefront: scores, softmax and the product of one tile follow each other.  The
+// kernel is small instead -- 163 VGPRs and 32 KiB of LDS at D = 128 -- so that THREE workgroups fit a
+// CU, three wavefronts a SIMD, and the latencies of one wavefront's step (the issue of its tile
+// copies, the LDS operand reads, the softmax chain, the barrier) are covered by the other two: matrix
+// instructions of one wavefront and vector instructions of another do run side by side on a SIMD.
+//   step n:  copies K(n+1), V(n+1) -> the other buffer;  S = K(n) Q^T;  P = softmax(S);  O += V(n)^T P;
+//            wait for the copies, barrier.
+// A wavefront computes only the tiles its 32 queries can see; a tile at the window / document edge or
+// on the diagonal is masked per element.
+constexpr int kTBN = 32;   // key rows per tile of prefill_tile_kernel
 template <int D>
-__global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(PrefillParams p) {
+__global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(PrefillParams p) {
   constexpr int NS = D / 16, NDT = D / 32, HALF = D / 2, CPR = D / 8;
-  constexpr int RPL = 64 / CPR, NLD = kBN / RPL / 4, TILE = kBN * D;
+  constexpr int RPL = 64 / CPR, NLD = kTBN / RPL / 4, TILE = kTBN * D;
+  static_assert(NLD >= 1, "a tile is at least one copy per wavefront");
   auto swz_k = [](int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); };
   auto swz_v = [](int r) { return D == 128 ? 4 * (r & 3) : 4 * ((r >> 1) & 1); };
 
@@ -501,68 +503,64 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
   const int lo_w_min = __builtin_amdgcn_readlane(lo_q, 0);
   const int lo_w_max = __builtin_amdgcn_readlane(lo_q, 31);
   const int q_w_min = min(qw0, p.T - 1), q_w_max = min(qw0 + 31, p.T - 1);
-
-  const int t_lo = row_lo(p, q0) / kBN;
-  const int t_hi = min(q0 + kBM - 1, p.T - 1) / kBN;
-  // This wavefront's own tile range (empty when all of its rows are past the end).
-  const int tw_lo = lo_w_min / kBN;
-  const int tw_hi = (qw0 < p.T) ? q_w_max / kBN : -1;
+  const bool wave_live = qw0 < p.T;
 
   // Tiles are visited in rotated order: start at the tile whose index is a multiple of the
   // window's tile count (one exists in every full range), run up to t_hi, wrap to t_lo.  The
   // online softmax does not care about the order, and the query blocks of one (batch, head)
   // that run side by side then read the same K/V tile at the same step, so one fetch into the
   // L2 serves all of them.  With no window every range starts at tile 0 and nothing is rotated.
+  const int t_lo = row_lo(p, q0) / kTBN;
+  const int t_hi = min(q0 + kBM - 1, p.T - 1) / kTBN;
   const int n_tiles = t_hi - t_lo + 1;
   int t_first = t_lo;
   if (p.period > 0) {
     const int c = (t_lo + p.period - 1) / p.period * p.period;
     if (c <= t_hi) t_first = c;
   }
+  auto tile_of = [&](int n) { const int t = t_first + n; return t <= t_hi ? t : t - n_tiles; };
 
   const uint16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
   const uint16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
 
-  // ---- global -> LDS copies (layout as in prefill_mfma_kernel) ---------------------------
+  // ---- global -> LDS copies ------------------------------------------------------------------
+  // Wavefront copy j of a tile moves rows RPL*j .. RPL*j+RPL-1 (1 KiB); lane i lands at chunk
+  // position i % CPR of row i / CPR, so it fetches the chunk that belongs there (the swizzle is
+  // applied on the global side).  This wavefront issues the copies wave, wave + 4, ...: their rows
+  // are 16 apart, the swizzles of such rows coincide, so one per-lane offset serves all of them and
+  // the row step goes into the wavefront-uniform base.
   const int ld_row = lane / CPR, ld_pos = lane % CPR;
-  int k_src_off[NLD], v_src_off[NLD];
+  const int r0 = RPL * wave + ld_row;
+  const int k_off = 2 * (r0 * (int)p.k_st + 8 * (ld_pos ^ swz_k(r0)));   // bytes
+  const int v_off = 2 * (r0 * (int)p.v_st + 8 * (ld_pos ^ swz_v(r0)));
+  const uint32_t ks_lds = lds_address(&Ks[0][0]) + 1024 * wave, vs_lds = lds_address(&Vs[0][0]) + 1024 * wave;
+  auto copy_tiles = [&](int tile, int buf) {
+    const int kv0 = tile * kTBN;
+    const uint16_t* kt = kbase + (int64_t)kv0 * p.k_st;
+    const uint16_t* vt = vbase + (int64_t)kv0 * p.v_st;
+    if (kv0 + kTBN <= p.T) {
 #pragma unroll
-  for (int i = 0; i < NLD; ++i) {
-    const int r = RPL * (4 * i + wave) + ld_row;
-    k_src_off[i] = r * (int)p.k_st + 8 * (ld_pos ^ swz_k(r));
-    v_src_off[i] = r * (int)p.v_st + 8 * (ld_pos ^ swz_v(r));
-  }
-  const uint32_t ks_lds = lds_address(&Ks[0][0]), vs_lds = lds_address(&Vs[0][0]);
-
-  auto copy_tile = [&](const uint16_t* base, int stride, const int* src_off, bool is_k, uint32_t lds, int tile, int buf) {
-    const int kv0 = tile * kBN;
-    const uint16_t* tb = base + (int64_t)kv0 * stride;
-    const uint32_t dst = lds + 2 * (buf * TILE + wave * 512);
-    if (kv0 + kBN <= p.T) {
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) copy16_to_lds_async(tb, 2 * src_off[i], dst + 2 * (4 * i * 512));
+      for (int i = 0; i < NLD; ++i) {
+        copy16_to_lds_async(kt + (int64_t)(4 * RPL * i) * p.k_st, k_off, ks_lds + 2 * (buf * TILE) + 4096 * i);
+        copy16_to_lds_async(vt + (int64_t)(4 * RPL * i) * p.v_st, v_off, vs_lds + 2 * (buf * TILE) + 4096 * i);
+      }
     } else {
       // The tile reaches past the last row: clamp (the surplus rows are masked by causality).
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
-        const int r = RPL * (4 * i + wave) + ld_row;
+        const int r = r0 + 4 * RPL * i;
         const int row = min(r, p.T - 1 - kv0);
-        const int chunk = ld_pos ^ (is_k ? swz_k(r) : swz_v(r));
-        copy16_to_lds_async(tb, 2 * (row * stride + 8 * chunk), dst + 2 * (4 * i * 512));
+        copy16_to_lds_async(kt, 2 * (row * (int)p.k_st + 8 * (ld_pos ^ swz_k(r))), ks_lds + 2 * (buf * TILE) + 4096 * i);
+        copy16_to_lds_async(vt, 2 * (row * (int)p.v_st + 8 * (ld_pos ^ swz_v(r))), vs_lds + 2 * (buf * TILE) + 4096 * i);
       }
     }
   };
-  auto copy_k = [&](int tile, int buf) { copy_tile(kbase, (int)p.k_st, k_src_off, true, ks_lds, tile, buf); };
-  auto copy_v = [&](int tile, int buf) { copy_tile(vbase, (int)p.v_st, v_src_off, false, vs_lds, tile, buf); };
   auto copies_landed = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), visible to the compiler's wait-count model
     asm volatile("" ::: "memory");
   };
-
-  // The first two K tiles go out before anything else so that their latency overlaps the Q loads.
-  auto tile_of = [&](int n) { const int t = t_first + n; return t <= t_hi ? t : t - n_tiles; };
-  copy_k(t_first, 0);
-  if (n_tiles > 1) copy_k(tile_of(1), 1);
+  // The first tile goes out before anything else so that its latency overlaps the Q loads.
+  copy_tiles(t_first, 0);
 
   // ---- Q fragment (B operand), RoPE fused ----------------------------------
   bf16x8 qreg[NS];
@@ -593,18 +591,19 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
     for (int s = 0; s < NS; ++s) qreg[s] = __builtin_bit_cast(bf16x8, raw[s]);
   }
 
-  // Per-lane LDS read pointers into buffer 0 (32-bit LDS addresses).
-  lds_u16_ptr k_rd[NS];
-  lds_u16_ptr v_rd[NDT];
-#pragma unroll
-  for (int s = 0; s < NS; ++s) k_rd[s] = (lds_u16_ptr)&Ks[0][0] + lq * D + 8 * ((2 * s + lh) ^ swz_k(lq));
+  // Operand addresses inside a tile (LDS byte addresses of buffer 0).  The swizzles are XORs on the
+  // chunk index, so the K fragment of contraction slice s sits at k_a0 ^ (32 s) and the V fragment of
+  // output tile dt at v_a0 ^ (64 dt): one register each instead of one per fragment.
+  //   K (A operand of S^T): row = key lq, slice s wants chunk (2s + lh) ^ swz_k(lq).
+  //   V (A operand of O^T, LDS transpose read): the lane's block of 16 covers output channels
+  //   32dt + 16*(block & 1) + 0..15 and keys 4*lh + 0..3 (+8, +16 as immediates); lane i of the
+  //   block addresses key i/4, channels 4*(i%4)..+3 and receives channel i, four keys.
+  const uint32_t k_a0 = lds_address(&Ks[0][0]) + 2 * (lq * D + 8 * (lh ^ swz_k(lq)));
+  uint32_t v_a0;
   {
     const int i16 = lane & 15, vrow = 4 * lh + (i16 >> 2);
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      const int chunk = 4 * dt + 2 * ((lane >> 4) & 1) + ((i16 & 3) >> 1);
-      v_rd[dt] = (lds_u16_ptr)&Vs[0][0] + vrow * D + 8 * (chunk ^ swz_v(vrow)) + 4 * (i16 & 1);
-    }
+    const int chunk = 2 * ((lane >> 4) & 1) + ((i16 & 3) >> 1);
+    v_a0 = lds_address(&Vs[0][0]) + 2 * (vrow * D + 8 * (chunk ^ swz_v(vrow)) + 4 * (i16 & 1));
   }
 
   f32x16 oacc[NDT];
@@ -612,211 +611,97 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_pipe_kernel(Prefil
   for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
-  f32x16 sc[2];                    // S of the tile this step turns into P; refilled in place for the next tile
-  float m_run = -INFINITY, l_run = 0.f;
-  float alpha_pend = 1.f;          // rescale of O asked for by the last softmax, not applied yet
-  bool rescale_pend = false;       // wave-uniform
-  bool pending = false;            // wave-uniform: pfrag holds a P that has not been multiplied into O yet
-  bf16x8 pfrag[2][2];              // P of the previous tile (B operands of the delayed product)
-  {
-    const u32x4 z = {0, 0, 0, 0};
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-      for (int m = 0; m < 2; ++m) pfrag[sb][m] = __builtin_bit_cast(bf16x8, z);
-  }
+  float m_run = -INFINITY;  // reference maximum (scaled, log2 domain) of this lane's query
+  float l_run = 0.f;        // this lane's share of the running sum
 
-  auto apply_pending_rescale = [&]() {
-    if (rescale_pend) {
+  // One tile of 32 keys.  There is ONE code path for clean and masked tiles (the mask is a small
+  // conditional region): two instantiations of the products would make the compiler keep a second
+  // copy of the accumulators across the join.
+  auto process_tile = [&](auto buf_tag, int kv0, bool masked) {
+    constexpr int buf = decltype(buf_tag)::value;
+    f32x16 sacc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const bf16x8 a = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(size_t)((k_a0 ^ (32u * s)) + 2 * buf * TILE));
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[s], sacc, 0, 0, 0);
+    }
+    if (masked) {
+      // element r of this lane is key kv0 + 4lh + c_r with c_r = 8*(r/4) + r%4; visible iff lo <= c_r <= hi
+      const int hi = qrow - (kv0 + 4 * lh);
+      const int lo = lo_q - (kv0 + 4 * lh);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int c = 8 * (r >> 2) + (r & 3);
+        if (c > hi || c < lo) sacc[r] = -INFINITY;
+      }
+    }
+    // Online softmax (log2 domain, lazy rescale): the reference maximum m_run only moves when some
+    // query of the wavefront sees a score more than 8 (log2 units) above it; until then
+    // probabilities are at most 2^8, which bf16 and the fp32 sums hold without loss, and O is not
+    // touched.
+    float mt = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sacc[r]);
+    mt = pair_max(mt) * p.scale_log2e;
+    if (__builtin_amdgcn_ballot_w64(mt > m_run + 8.f) != 0) {
+      const float m_new = fmaxf(m_run, mt);
+      const float mu = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run - mu);
+      m_run = m_new;
+      l_run *= alpha;
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha_pend;
-      rescale_pend = false;
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
     }
-  };
-
-  // One 32-key half of S^T = K Q^T into sc[sb], K from buffer offset kofs (elements).
-  auto qk_half = [&](int kofs, int sb) {
-    constexpr int KPF = 3;   // K fragments are read KPF contraction slices ahead of their MFMAs
-    bf16x8 ka[KPF];
-    auto read_k = [&](int s) {
-      ka[s % KPF] = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(k_rd[s] + kofs + 32 * sb * D));
-    };
+    const float mu = (m_run == -INFINITY) ? 0.f : m_run;
+    bf16x8 pfrag[2];
+    float lsum = 0.f;
 #pragma unroll
-    for (int s = 0; s < KPF; ++s) read_k(s);
+    for (int m = 0; m < 2; ++m) {
+      float pv[8];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) sc[sb][r] = 0.f;
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      sc[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[s % KPF], qreg[s], sc[sb], 0, 0, 0);
-      if (s + KPF < NS) read_k(s + KPF);
+      for (int e = 0; e < 8; ++e) {
+        pv[e] = fast_exp2(fmaf(sacc[8 * m + e], p.scale_log2e, -mu));
+        lsum += pv[e];
+      }
+      pfrag[m] = __builtin_bit_cast(bf16x8, pack8(pv));
     }
-  };
-
-  // Half of O^T += V^T P^T: the 32 keys of block sb, V from buffer offset vofs (elements).
-  auto pv_half = [&](int vofs, int sb) {
+    l_run += lsum;
+    // O^T += V^T P^T
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) {
-        lds_u16_ptr vp = v_rd[dt] + vofs;
-        const u32x2 a0 = lds_read_tr16_as3(vp + (32 * sb + 16 * m) * D);
-        const u32x2 a1 = lds_read_tr16_as3(vp + (32 * sb + 16 * m + 8) * D);
+        lds_u16_ptr vp = (lds_u16_ptr)(size_t)((v_a0 ^ (64u * dt)) + 2 * (buf * TILE + 16 * m * D));
+        const u32x2 a0 = lds_read_tr16_as3(vp);            // keys 16m + 4lh + 0..3
+        const u32x2 a1 = lds_read_tr16_as3(vp + 8 * D);    // keys 16m + 8 + 4lh + 0..3
         const u32x4 av = {a0.x, a0.y, a1.x, a1.y};
-        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), pfrag[sb][m], oacc[dt], 0, 0, 0);
+        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), pfrag[m], oacc[dt], 0, 0, 0);
       }
     }
   };
 
-  // Online-softmax bookkeeping for the tile held in sc (after masking): returns the exponent offset.
-  // Lazy rescale: the reference maximum only moves when some query of the wavefront sees a score
-  // more than 8 (log2 units) above it; until then probabilities stay below 2^8, which bf16 and
-  // the fp32 sums hold without loss, and O is not touched.
-  auto update_maximum = [&]() {
-    float mt = -INFINITY;
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sc[sb][r]);
-    mt = pair_max(mt) * p.scale_log2e;
-    const bool move = __builtin_amdgcn_ballot_w64(mt > m_run + 8.f) != 0;
-    const float m_new = move ? fmaxf(m_run, mt) : m_run;
-    const float mu = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - mu);      // 1 when the maximum did not move, 0 on the first tile
-    m_run = m_new;
-    alpha_pend = alpha;
-    rescale_pend = move;
-    l_run *= alpha;
-    return mu;
-  };
-  // P of one 32-key half: exp2, row sums, bf16 B operands of the delayed product.
-  auto probabilities_half = [&](int sb, float mu) {
-    float pv[16];
-    float lsum = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      pv[r] = fast_exp2(fmaf(sc[sb][r], p.scale_log2e, -mu));
-      lsum += pv[r];
+  using Buf0 = std::integral_constant<int, 0>;
+  using Buf1 = std::integral_constant<int, 1>;
+  copies_landed();
+  __syncthreads();
+  auto iteration = [&](int n, auto buf_tag) {
+    constexpr int buf = decltype(buf_tag)::value;
+    if (n + 1 < n_tiles) copy_tiles(tile_of(n + 1), buf ^ 1);
+    const int kv0 = tile_of(n) * kTBN;
+    if (wave_live && kv0 <= q_w_max && kv0 + kTBN - 1 >= lo_w_min) {
+      const bool clean = kv0 + kTBN - 1 <= q_w_min && kv0 >= lo_w_max;
+      process_tile(buf_tag, kv0, !clean);
     }
-#pragma unroll
-    for (int m = 0; m < 2; ++m) {
-      u32x4 pk;
-      pk.x = pack_bf16x2(pv[8 * m + 0], pv[8 * m + 1]);
-      pk.y = pack_bf16x2(pv[8 * m + 2], pv[8 * m + 3]);
-      pk.z = pack_bf16x2(pv[8 * m + 4], pv[8 * m + 5]);
-      pk.w = pack_bf16x2(pv[8 * m + 6], pv[8 * m + 7]);
-      pfrag[sb][m] = __builtin_bit_cast(bf16x8, pk);
-    }
-    l_run += lsum;
-  };
-  auto mask_scores = [&](int kv0) {
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-      // element r of this lane is key kv0 + 32sb + 4lh + c_r with c_r = 8*(r/4) + r%4
-      const int hi = qrow - (kv0 + 32 * sb + 4 * lh);    // visible iff lo <= c_r <= hi
-      const int lo = lo_q - (kv0 + 32 * sb + 4 * lh);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int c = 8 * (r >> 2) + (r & 3);
-        if (c > hi || c < lo) sc[sb][r] = -INFINITY;
-      }
-    }
-  };
-
-  auto is_active = [&](int n) {
-    if (n < 0 || n >= n_tiles) return false;
-    const int t = tile_of(n);
-    return t >= tw_lo && t <= tw_hi;
-  };
-  // Step n: K(n+2) and V(n) start on their way; at the end they have landed and all wavefronts meet.
-  // K(n+1) was published by the previous step, V(n-1) too.
-  auto step_begin = [&](int n) {
-    if (n + 2 < n_tiles) copy_k(tile_of(n + 2), n & 1);
-    copy_v(tile_of(n), n & 1);
-  };
-  auto step_end = [&]() {
     copies_landed();
     __syncthreads();
   };
-
-  // Generic step (tiles at the edges of a wavefront's range, masked tiles, idle steps): the three
-  // pieces one after the other.
-  auto generic_steps = [&](int from, int to) {
-    for (int n = from; n <= to; ++n) {
-      const int par = n & 1;
-      step_begin(n);
-      if (pending) {
-        apply_pending_rescale();
-        pv_half((par ^ 1) * TILE, 0);
-        pv_half((par ^ 1) * TILE, 1);
-        pending = false;
-      }
-      if (is_active(n)) {
-        const int kv0 = tile_of(n) * kBN;
-        if (!(kv0 + kBN - 1 <= q_w_min && kv0 >= lo_w_max)) mask_scores(kv0);
-        const float mu = update_maximum();
-        probabilities_half(0, mu);
-        probabilities_half(1, mu);
-        pending = true;
-      }
-      if (is_active(n + 1)) {
-        qk_half((par ^ 1) * TILE, 0);
-        qk_half((par ^ 1) * TILE, 1);
-      }
-      step_end();
-    }
-  };
-  // Hot step: tile n fully visible, the previous and the next tile belong to this wavefront too.
-  // One basic block holds the delayed product of tile n-1, the softmax of tile n and S of tile
-  // n+1 (written into the registers of S(n) as soon as each half has been turned into P), so
-  // that the matrix pipe has work all along the vector work of the same wavefront.
-  auto hot_steps = [&](int from, int to) {
-    for (int n = from; n <= to; ++n) {
-      const int par = n & 1;
-      const int other = (par ^ 1) * TILE;   // V(n-1) and K(n+1) both sit in the other buffer
-      step_begin(n);
-      apply_pending_rescale();
-      const float mu = update_maximum();
-      pv_half(other, 0);
-      probabilities_half(0, mu);   // frees sc[0] ...
-      pv_half(other, 1);
-      qk_half(other, 0);           // ... for S(n+1), first half
-      probabilities_half(1, mu);
-      qk_half(other, 1);
-      step_end();
-    }
-  };
-
-  copies_landed();
-  __syncthreads();
-  if (is_active(0)) {
-    qk_half(0, 0);
-    qk_half(0, 1);
-  }
-
-  // Fully visible tiles of this wavefront: first key >= every row's lower bound, last key <=
-  // the first row.  A hot step needs such a tile with active neighbours in the same run of
-  // consecutive tiles (the rotated order has two runs: t_first..t_hi, then t_lo..t_first-1).
-  const int c_lo = max((lo_w_max + kBN - 1) / kBN, max(tw_lo, t_lo));
-  const int c_hi = min((q_w_min + 1) / kBN - 1, min(tw_hi, t_hi));
-#pragma nounroll
-  for (int run = 0; run < 2; ++run) {
-    const int a = run == 0 ? t_first : t_lo;
-    const int b = run == 0 ? t_hi : t_first - 1;
-    const int n0 = run == 0 ? 0 : t_hi - t_first + 1;     // step of tile a
-    if (b < a) continue;
-    int ha = max(max(c_lo, a + 1), tw_lo + 1);
-    int hb = min(min(c_hi, b - 1), tw_hi - 1);
-    if (hb < ha) { ha = b + 1; hb = b; }                   // no hot tile in this run
-    generic_steps(n0, n0 + ha - 1 - a);
-    hot_steps(n0 + ha - a, n0 + hb - a);
-    generic_steps(n0 + hb + 1 - a, n0 + b - a);
-  }
-  if (pending) {
-    apply_pending_rescale();
-    pv_half(((n_tiles - 1) & 1) * TILE, 0);
-    pv_half(((n_tiles - 1) & 1) * TILE, 1);
+  for (int n = 0; n < n_tiles; n += 2) {
+    iteration(n, Buf0{});
+    if (n + 1 < n_tiles) iteration(n + 1, Buf1{});
   }
 
   const float l_tot = pair_sum(l_run);
@@ -950,14 +835,14 @@ static int launch_mfma(PrefillParams p, bool rope_in_kernel, hipStream_t s) {
     hipLaunchKernelGGL(rope_k_kernel<D>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, p);
     DAISY_CHECK_LAUNCH("rope_k_kernel");
     p.k = p.k_out; p.k_sb = p.ko_sb; p.k_st = p.ko_st; p.k_sh = p.ko_sh;
-    hipLaunchKernelGGL((prefill_pipe_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
-    DAISY_CHECK_LAUNCH("prefill_pipe_kernel");
+    hipLaunchKernelGGL((prefill_tile_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
+    DAISY_CHECK_LAUNCH("prefill_tile_kernel");
   } else if (p.cos != nullptr) {
     hipLaunchKernelGGL((prefill_mfma_kernel<D, true>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
     DAISY_CHECK_LAUNCH("prefill_mfma_kernel");
   } else {
-    hipLaunchKernelGGL((prefill_pipe_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
-    DAISY_CHECK_LAUNCH("prefill_pipe_kernel");
+    hipLaunchKernelGGL((prefill_tile_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
+    DAISY_CHECK_LAUNCH("prefill_tile_kernel");
   }
   return DAISY_OK;
 }
@@ -985,7 +870,7 @@ static int fill_prefill_params(PrefillParams& p, const void* q, const int64_t* q
   p.ko_sb = k_out ? k_out_strides[0] : 0; p.ko_st = k_out ? k_out_strides[1] : 0; p.ko_sh = k_out ? k_out_strides[2] : 0;
   p.B = B; p.T = T; p.H = H; p.D = D; p.window = window;
   p.nqb = (T + kBM - 1) / kBM;
-  p.period = (window > 0 && window < T) ? (kBM - 1) / kBN + 1 + (window - 1 + kBN - 1) / kBN : 0;
+  p.period = (window > 0 && window < T) ? (kBM - 1) / kTBN + 1 + (window - 1 + kTBN - 1) / kTBN : 0;
   p.n_light = (window > 0 && window < T) ? min((window - 1 + kBM - 1) / kBM, p.nqb) : 0;
   p.scale_log2e = scale * kLog2e;
   return DAISY_OK;

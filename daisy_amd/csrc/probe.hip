@@ -54,7 +54,7 @@ __global__ __launch_bounds__(512) void matrix_rate_kernel(float* sink, unsigned 
 // of every MFMA comes from LDS with the kernel's own access patterns -- a 16-byte read of a swizzled
 // row-major tile (the K operand) for even MFMAs, two 8-byte transposing reads (the V operand) for
 // odd ones -- requested eight MFMAs before its use.  No global memory, no barriers, no masks: the
-// rate of this stream is what the two-wavefronts-per-SIMD layout of prefill_pipe_kernel can reach at
+// rate of this stream is what the layout of prefill_tile_kernel (two or three wavefronts per SIMD) can reach at
 // best with its instruction mix.
 typedef short probe_s16x4 __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(512) void attention_mix_kernel(float* sink, unsigned long long* ticks, int iters) {

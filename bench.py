@@ -155,20 +155,30 @@ def bench_prefill_c2(steps, warmup, cpu_baseline=True):
     def full():
         ops.prefill_attention(q, k, v, window=W, scale=SCALE, cos=cos, sin=sin, out=o, k_out=k_rot)
 
-    ms_full = time_gpu(full, steps, warmup)
-
-    # The dominant kernel alone: same launch, keys already rotated (k_rot from above).  Median of the
-    # launches' own durations (an event pair around every launch).
     o2 = torch.empty_like(o)
 
     def attn_only():
         ops.prefill_attention(q, k_rot, v, window=W, scale=SCALE, out=o2)
 
-    ms_kernel, ms_kernel_mean = time_gpu(attn_only, steps, warmup, per_launch=True)
-    # The same kernel under sustained load: back-to-back launches for at least a second (the clock the power
-    # management grants falls while matrix load lasts, so a burst of a few milliseconds flatters the kernel).
-    n_sustained = max(int(1100.0 / ms_kernel), steps)
+    # After a change of load the chip needs some hundred launches to settle (the power management moves the shader
+    # clock when the HBM traffic of the pre-pass appears: ~200 us per step for the first steps from an idle GPU or
+    # right after a run of the attention kernel alone, ~170 us from the third hundred on).  So the order is: (1) the
+    # first steps from an idle GPU, for the record; (2) half a second of the headline step back to back (the sustained
+    # figure); (3) the headline: `warmup` untimed and `steps` timed steps on the GPU as (2) left it; (4) the attention
+    # kernel alone for at least a second; (5) its per-launch median.
+    full()
+    torch.cuda.synchronize()
+    time.sleep(1.0)
+    ms_full_from_idle = time_gpu(full, steps, 0)
+    n_full_sustained = max(int(500.0 / ms_full_from_idle), steps)
+    ms_full_sustained = time_gpu(full, n_full_sustained, 0)
+    ms_full = time_gpu(full, steps, warmup)
+    ms_estimate = time_gpu(attn_only, 10, 2)
+    n_sustained = max(int(1100.0 / ms_estimate), steps)
     ms_sustained = time_gpu(attn_only, n_sustained, 0)
+    # The dominant kernel alone: same launch, keys already rotated (k_rot from above).  Median of the
+    # launches' own durations (an event pair around every launch), right behind the sustained run.
+    ms_kernel, ms_kernel_mean = time_gpu(attn_only, steps, warmup, per_launch=True)
     clock_after = probe_matrix_rate(False, 4000)["clock_mhz"] if SUSTAINED_CLOCK else None
 
     def fused():
@@ -179,7 +189,10 @@ def bench_prefill_c2(steps, warmup, cpu_baseline=True):
     flops = prefill_flops(B, T, H, D, W)
     res = {
         "workload": "prefill_c2_B8_T4096_H8_D128_W1024_rope",
-        "ms_full": ms_full, "ms_kernel": ms_kernel, "ms_kernel_mean": ms_kernel_mean, "ms_rotate_k_in_kernel": ms_fused,
+        "ms_full": ms_full, "ms_full_first_steps_from_idle": ms_full_from_idle,
+        "ms_full_sustained": ms_full_sustained, "full_sustained_launches": n_full_sustained,
+        "tflops_full_sustained": flops / ms_full_sustained / 1e9,
+        "ms_kernel": ms_kernel, "ms_kernel_mean": ms_kernel_mean, "ms_rotate_k_in_kernel": ms_fused,
         "flops": flops,
         "tflops_full": flops / ms_full / 1e9, "tflops_kernel": flops / ms_kernel / 1e9,
         "frac_of_peak_kernel": flops / ms_kernel / 1e9 / PEAK_BF16_TFLOPS,

@@ -68,6 +68,18 @@ def time_gpu(fn, steps, warmup, per_launch=False):
     return start.elapsed_time(end) / steps
 
 
+def time_settled(fn, steps, warmup, seconds=0.4):
+    """(ms per call settled, ms per call over the first `steps` calls from an idle GPU).  After a change of load the
+    chip runs the first launches slower and settles over some hundred milliseconds (power management), so the timed
+    steps follow `seconds` of the same call back to back."""
+    fn()
+    torch.cuda.synchronize()
+    time.sleep(0.5)
+    ms_first = time_gpu(fn, steps, 0)
+    time_gpu(fn, max(int(seconds * 1e3 / ms_first), 1), 0)
+    return time_gpu(fn, steps, warmup), ms_first
+
+
 # ---- diagnostic kernels of the benchmark (their own library, not part of the product ABI) ----------
 _probe_lib = None
 
@@ -306,7 +318,7 @@ def bench_module_c2(steps, warmup):
     with torch.no_grad():
         for name, fused in (("ms_fused_prep", True), ("ms_library_elementwise", False)):
             attn.fused_prep = fused
-            out[name] = time_gpu(lambda: attn.prefill(x, None, attn_mask=mask), steps, warmup)
+            out[name], out[name + "_first_steps_from_idle"] = time_settled(lambda: attn.prefill(x, None, attn_mask=mask), steps, warmup)
         qkv = torch.nn.functional.linear(x, attn.qkvo_w[:3].flatten(end_dim=1)).view(B, T, 3 * H, D)
         q, k, v = qkv.chunk(3, dim=-2)
         cos, sin = attn.rotary._get_cos_sin(T)
@@ -327,9 +339,10 @@ def bench_prefill_c3(steps, warmup):
     o = torch.empty_like(q)
     out = {}
     for name, W, n in (("window2048", 2048, steps), ("full_causal", None, max(steps // 4, 2))):
-        ms = time_gpu(lambda: ops.prefill_attention(q, k, v, window=W, scale=SCALE, out=o), n, max(warmup // 2, 1))
+        ms, ms_first = time_settled(lambda: ops.prefill_attention(q, k, v, window=W, scale=SCALE, out=o), n, max(warmup // 2, 1))
         fl = prefill_flops(B, T, H, D, W)
-        out[name] = {"ms": ms, "flops": fl, "tflops": fl / ms / 1e9, "frac_of_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS}
+        out[name] = {"ms": ms, "ms_first_steps_from_idle": ms_first, "flops": fl, "tflops": fl / ms / 1e9,
+                     "frac_of_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS}
     return out
 
 
@@ -424,12 +437,12 @@ def bench_kda_c5(steps, warmup, cpu_baseline=True):
     gl = torch.nn.functional.logsigmoid(rn(B, T, H, Dk))
     beta = torch.sigmoid(rn(B, T, H))
     ws = torch.empty(max(ops.kda_workspace_bytes(B, T, H, Dk, Dv), 1), dtype=torch.uint8, device=dev)
-    ms = time_gpu(lambda: ops.kda_chunk_fwd(q, k, v, gl, beta, output_final_state=True, workspace=ws), steps, warmup)
+    ms, ms_first = time_settled(lambda: ops.kda_chunk_fwd(q, k, v, gl, beta, output_final_state=True, workspace=ws), steps, warmup)
     gl16 = gl.bfloat16()     # the dtype the reference's layer hands over (the gate's output follows its bf16 input)
     ms_g16 = time_gpu(lambda: ops.kda_chunk_fwd(q, k, v, gl16, beta, output_final_state=True, workspace=ws), steps, warmup)
     min_bytes = 5 * B * T * H * Dk * 2
     flops = 7.0 * Dk * Dv * B * T * H
-    out = {"workload": "kda_c5_B4_T8192_H16_D128_chunk64", "ms": ms, "min_bytes": min_bytes,
+    out = {"workload": "kda_c5_B4_T8192_H16_D128_chunk64", "ms": ms, "ms_first_steps_from_idle": ms_first, "min_bytes": min_bytes,
            "gbs_min_io": min_bytes / ms / 1e6, "frac_of_hbm_peak": min_bytes / ms / 1e6 / PEAK_HBM_GBS,
            "naive_flops": flops, "tflops_naive": flops / ms / 1e9,
            "g_dtype": "fp32", "ms_with_bf16_g": ms_g16, "frac_of_hbm_peak_with_bf16_g": min_bytes / ms_g16 / 1e6 / PEAK_HBM_GBS}

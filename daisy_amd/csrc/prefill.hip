@@ -487,6 +487,10 @@ __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(Prefil
 
   __shared__ __attribute__((aligned(1024))) uint16_t Ks[2][TILE];
   __shared__ __attribute__((aligned(1024))) uint16_t Vs[2][TILE];
+  // Two more tile-sized areas: with Ks[1] and Vs[1] they give every wavefront 32 rows x D of its own for
+  // turning the row-major Q block into operand fragments at the start (while the first K/V tile lands in
+  // Ks[0] / Vs[0]) and the accumulators into row-major O at the end.
+  __shared__ __attribute__((aligned(1024))) uint16_t Xs[2][TILE];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -562,33 +566,58 @@ __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(Prefil
   // The first tile goes out before anything else so that its latency overlaps the Q loads.
   copy_tiles(t_first, 0);
 
-  // ---- Q fragment (B operand), RoPE fused ----------------------------------
+  // ---- Q fragments (B operand), RoPE fused -------------------------------------------------------
+  // Global loads with whole rows per group of lanes (lane -> row lane / CH, pair chunk lane % CH: the
+  // 16 bytes at channel 8 ch and the 16 bytes at HALF + 8 ch, with the matching 32 bytes of the cos and
+  // sin rows), rotated in that layout, written to this wavefront's own LDS area in the K tile layout
+  // and read back as fragments.  Fetching the fragments straight from global memory would touch 32
+  // rows with every instruction (32 bytes of each), and the CU's memory path, which the other
+  // workgroups' tile copies share, would be busy four times as long.
+  constexpr int CH = HALF / 8;          // pair chunks per row
+  constexpr int QRI = 64 / CH;          // rows per load instruction
+  constexpr int QT = 32 / QRI;          // loads of each kind per lane
+  const uint32_t x_lds = wave == 0 ? lds_address(&Ks[1][0]) : wave == 1 ? lds_address(&Vs[1][0])
+                                                                         : lds_address(&Xs[wave - 2][0]);
   bf16x8 qreg[NS];
   {
-    const uint16_t* qptr = p.q + b * p.q_sb + (int64_t)qrow * p.q_st + h * p.q_sh + 8 * lh;
-    u32x4 raw[NS];
+    const int qr = lane / CH, qc = lane % CH;
+    u32x4 x1[QT], x2[QT];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) raw[s] = *reinterpret_cast<const u32x4*>(qptr + 16 * s);
+    for (int j = 0; j < QT; ++j) {
+      const int row = min(qw0 + QRI * j + qr, p.T - 1);
+      const uint16_t* qptr = p.q + b * p.q_sb + (int64_t)row * p.q_st + h * p.q_sh + 8 * qc;
+      x1[j] = *reinterpret_cast<const u32x4*>(qptr);
+      x2[j] = *reinterpret_cast<const u32x4*>(qptr + HALF);
+    }
     if (p.cos != nullptr) {
-      const float* cr = p.cos + (int64_t)qrow * HALF + 8 * lh;
-      const float* sr = p.sin + (int64_t)qrow * HALF + 8 * lh;
 #pragma unroll
-      for (int s = 0; s < NS / 2; ++s) {
-        float x1[8], x2[8], y1[8], y2[8];
-        unpack8(raw[s], x1);
-        unpack8(raw[s + NS / 2], x2);
+      for (int j = 0; j < QT; ++j) {
+        const int row = min(qw0 + QRI * j + qr, p.T - 1);
+        const float* cr = p.cos + (int64_t)row * HALF + 8 * qc;
+        const float* sr = p.sin + (int64_t)row * HALF + 8 * qc;
+        float a1[8], a2[8], y1[8], y2[8];
+        unpack8(x1[j], a1);
+        unpack8(x2[j], a2);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const float c = cr[16 * s + e], sn = sr[16 * s + e];
-          y1[e] = rope_lo(x1[e], x2[e], c, sn);
-          y2[e] = rope_hi(x1[e], x2[e], c, sn);
+          const float c = cr[e], sn = sr[e];
+          y1[e] = rope_lo(a1[e], a2[e], c, sn);
+          y2[e] = rope_hi(a1[e], a2[e], c, sn);
         }
-        raw[s] = pack8(y1);
-        raw[s + NS / 2] = pack8(y2);
+        x1[j] = pack8(y1);
+        x2[j] = pack8(y2);
       }
     }
 #pragma unroll
-    for (int s = 0; s < NS; ++s) qreg[s] = __builtin_bit_cast(bf16x8, raw[s]);
+    for (int j = 0; j < QT; ++j) {
+      const int r = QRI * j + qr;
+      *(u32x4 __attribute__((address_space(3)))*)(size_t)(x_lds + 2 * (r * D + 8 * (qc ^ swz_k(r)))) = x1[j];
+      *(u32x4 __attribute__((address_space(3)))*)(size_t)(x_lds + 2 * (r * D + 8 * ((CH + qc) ^ swz_k(r)))) = x2[j];
+    }
+    const uint32_t q_a0 = x_lds + 2 * (lq * D + 8 * (lh ^ swz_k(lq)));
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+      qreg[s] = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(size_t)(q_a0 ^ (32u * s)));
   }
 
   // Operand addresses inside a tile (LDS byte addresses of buffer 0).  The swizzles are XORs on the
@@ -704,20 +733,28 @@ __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(Prefil
     if (n + 1 < n_tiles) iteration(n + 1, Buf1{});
   }
 
+  // Epilogue: normalise, turn the accumulators (a lane holds four channels of one query per register
+  // group) into row-major bf16 through this wavefront's LDS area, and store 16 bytes per lane with whole
+  // rows per group of lanes.  The tile buffers are free: the loop ends with a barrier.
   const float l_tot = pair_sum(l_run);
   const float inv = 1.f / l_tot;
-  if (qw0 + lq < p.T) {
-    uint16_t* op = p.o + b * p.o_sb + (int64_t)(qw0 + lq) * p.o_st + h * p.o_sh + 4 * lh;
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
+  for (int dt = 0; dt < NDT; ++dt) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w.x = pack_bf16x2(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
-        w.y = pack_bf16x2(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
-        *reinterpret_cast<u32x2*>(op + 32 * dt + 8 * g) = w;
-      }
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w;
+      w.x = pack_bf16x2(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
+      w.y = pack_bf16x2(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
+      // channels 32 dt + 8 g + 4 lh + 0..3 of query lq: chunk 4 dt + g, half lh
+      *(u32x2 __attribute__((address_space(3)))*)(size_t)(x_lds + 2 * (lq * D + 8 * ((4 * dt + g) ^ swz_k(lq)) + 4 * lh)) = w;
     }
+  }
+  uint16_t* obase = p.o + b * p.o_sb + h * p.o_sh + 8 * ld_pos;
+#pragma unroll
+  for (int i = 0; i < 32 / RPL; ++i) {
+    const int r = RPL * i + ld_row;
+    const u32x4 w = *(const u32x4 __attribute__((address_space(3)))*)(size_t)(x_lds + 2 * (r * D + 8 * (ld_pos ^ swz_k(r))));
+    if (qw0 + r < p.T) *reinterpret_cast<u32x4*>(obase + (int64_t)(qw0 + r) * p.o_st) = w;
   }
 }
 

@@ -522,7 +522,6 @@ __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(Prefil
     const int c = (t_lo + p.period - 1) / p.period * p.period;
     if (c <= t_hi) t_first = c;
   }
-  auto tile_of = [&](int n) { const int t = t_first + n; return t <= t_hi ? t : t - n_tiles; };
 
   const uint16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
   const uint16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
@@ -538,10 +537,17 @@ __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(Prefil
   const int k_off = 2 * (r0 * (int)p.k_st + 8 * (ld_pos ^ swz_k(r0)));   // bytes
   const int v_off = 2 * (r0 * (int)p.v_st + 8 * (ld_pos ^ swz_v(r0)));
   const uint32_t ks_lds = lds_address(&Ks[0][0]) + 1024 * wave, vs_lds = lds_address(&Vs[0][0]) + 1024 * wave;
-  auto copy_tiles = [&](int tile, int buf) {
-    const int kv0 = tile * kTBN;
-    const uint16_t* kt = kbase + (int64_t)kv0 * p.k_st;
-    const uint16_t* vt = vbase + (int64_t)kv0 * p.v_st;
+  // The copies walk the tiles in visiting order; the source pointers move by one tile per step and go
+  // back to the first tile of the range once (kept incrementally: the scalar unit would otherwise
+  // rebuild two 64-bit products per step).
+  const int64_t k_step = (int64_t)kTBN * p.k_st, v_step = (int64_t)kTBN * p.v_st;
+  const uint16_t* const k_lo = kbase + t_lo * k_step;
+  const uint16_t* const v_lo = vbase + t_lo * v_step;
+  int t_cp = t_first;                                   // tile the next copy_tiles() call fetches
+  const uint16_t* kt = kbase + t_first * k_step;
+  const uint16_t* vt = vbase + t_first * v_step;
+  auto copy_tiles = [&](int buf) {
+    const int kv0 = t_cp * kTBN;
     if (kv0 + kTBN <= p.T) {
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
@@ -558,13 +564,16 @@ __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(Prefil
         copy16_to_lds_async(vt, 2 * (row * (int)p.v_st + 8 * (ld_pos ^ swz_v(r))), vs_lds + 2 * (buf * TILE) + 4096 * i);
       }
     }
+    if (++t_cp > t_hi) { t_cp = t_lo; kt = k_lo; vt = v_lo; }
+    else { kt += k_step; vt += v_step; }
   };
   auto copies_landed = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), visible to the compiler's wait-count model
     asm volatile("" ::: "memory");
   };
   // The first tile goes out before anything else so that its latency overlaps the Q loads.
-  copy_tiles(t_first, 0);
+  copy_tiles(0);
+  int t_cur = t_first;                                  // tile the next iteration works on
 
   // ---- Q fragments (B operand), RoPE fused -------------------------------------------------------
   // Global loads with whole rows per group of lanes (lane -> row lane / CH, pair chunk lane % CH: the
@@ -651,10 +660,23 @@ __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(Prefil
     f32x16 sacc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+    // K fragments: four reads ahead of the products (an LDS read takes about as long as four MFMAs;
+    // left alone the compiler keeps one fragment register set and waits for every read in turn).
+    {
+      bf16x8 kf[NS];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      const bf16x8 a = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(size_t)((k_a0 ^ (32u * s)) + 2 * buf * TILE));
-      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[s], sacc, 0, 0, 0);
+      for (int s = 0; s < NS; ++s)
+        kf[s] = __builtin_bit_cast(bf16x8, *(const u32x4 __attribute__((address_space(3)))*)(size_t)((k_a0 ^ (32u * s)) + 2 * buf * TILE));
+#pragma unroll
+      for (int s = 0; s < NS; ++s) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[s], qreg[s], sacc, 0, 0, 0);
+      constexpr int AHEAD = NS < 4 ? NS : 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);          // DS reads
+#pragma unroll
+      for (int s = 0; s < NS - AHEAD; ++s) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
     }
     if (masked) {
       // element r of this lane is key kv0 + 4lh + c_r with c_r = 8*(r/4) + r%4; visible iff lo <= c_r <= hi
@@ -719,8 +741,9 @@ __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(Prefil
   __syncthreads();
   auto iteration = [&](int n, auto buf_tag) {
     constexpr int buf = decltype(buf_tag)::value;
-    if (n + 1 < n_tiles) copy_tiles(tile_of(n + 1), buf ^ 1);
-    const int kv0 = tile_of(n) * kTBN;
+    if (n + 1 < n_tiles) copy_tiles(buf ^ 1);
+    const int kv0 = t_cur * kTBN;
+    t_cur = t_cur < t_hi ? t_cur + 1 : t_lo;
     if (wave_live && kv0 <= q_w_max && kv0 + kTBN - 1 >= lo_w_min) {
       const bool clean = kv0 + kTBN - 1 <= q_w_min && kv0 >= lo_w_max;
       process_tile(buf_tag, kv0, !clean);

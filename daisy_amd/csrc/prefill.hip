@@ -777,39 +777,55 @@ __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(Prefil
   for (int i = 0; i < 32 / RPL; ++i) {
     const int r = RPL * i + ld_row;
     const u32x4 w = *(const u32x4 __attribute__((address_space(3)))*)(size_t)(x_lds + 2 * (r * D + 8 * (ld_pos ^ swz_k(r))));
-    if (qw0 + r < p.T) *reinterpret_cast<u32x4*>(obase + (int64_t)(qw0 + r) * p.o_st) = w;
+    // whole rows, written once and not read again by this kernel: streaming stores leave the last-level
+    // cache to q, k and v (the same store from the accumulator layout, 16 bytes per row, must not be
+    // streaming: such partial lines are then no longer merged on their way out)
+    if (qw0 + r < p.T) __builtin_nontemporal_store(w, reinterpret_cast<u32x4*>(obase + (int64_t)(qw0 + r) * p.o_st));
   }
 }
 
-// Rotates keys once and stores them with the caller's output strides.
-template <int D>
+// Rotates keys once and stores them with the caller's output strides.  A thread takes one pair chunk
+// (8 + 8 channels) of HPT heads of one position: the cos and sin values are fetched once for them.
+template <int D, int HPT>
 __global__ __launch_bounds__(256) void rope_k_kernel(PrefillParams p) {
   constexpr int HALF = D / 2;
   constexpr int CH = HALF / 8;  // pair chunks per row
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t total = (int64_t)p.B * p.T * p.H * CH;
+  const int HG = p.H / HPT;
+  const int64_t total = (int64_t)p.B * p.T * HG * CH;
   if (idx >= total) return;
   const int ch = idx % CH;
-  const int h = (idx / CH) % p.H;
-  const int t = (idx / ((int64_t)CH * p.H)) % p.T;
-  const int b = idx / ((int64_t)CH * p.H * p.T);
-  const uint16_t* kp = p.k + b * p.k_sb + (int64_t)t * p.k_st + h * p.k_sh + 8 * ch;
-  uint16_t* op = p.k_out + b * p.ko_sb + (int64_t)t * p.ko_st + h * p.ko_sh + 8 * ch;
-  float x1[8], x2[8], y1[8], y2[8];
+  const int hg = (idx / CH) % HG;
+  const int t = (idx / ((int64_t)CH * HG)) % p.T;
+  const int b = idx / ((int64_t)CH * HG * p.T);
+  u32x4 r1[HPT], r2[HPT];
   // The unrotated keys are not needed again: read them past the caches, so that q, v and the
   // rotated keys this pass writes are what the attention kernel finds there.
-  unpack8(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp)), x1);
-  unpack8(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp + HALF)), x2);
+#pragma unroll
+  for (int j = 0; j < HPT; ++j) {
+    const uint16_t* kp = p.k + b * p.k_sb + (int64_t)t * p.k_st + (hg + j * HG) * p.k_sh + 8 * ch;
+    r1[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp));
+    r2[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp + HALF));
+  }
   const float* cr = p.cos + (int64_t)t * HALF + 8 * ch;
   const float* sr = p.sin + (int64_t)t * HALF + 8 * ch;
+  float c[8], sn[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float c = cr[e], s = sr[e];
-    y1[e] = rope_lo(x1[e], x2[e], c, s);
-    y2[e] = rope_hi(x1[e], x2[e], c, s);
+  for (int e = 0; e < 8; ++e) { c[e] = cr[e]; sn[e] = sr[e]; }
+#pragma unroll
+  for (int j = 0; j < HPT; ++j) {
+    float x1[8], x2[8], y1[8], y2[8];
+    unpack8(r1[j], x1);
+    unpack8(r2[j], x2);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      y1[e] = rope_lo(x1[e], x2[e], c[e], sn[e]);
+      y2[e] = rope_hi(x1[e], x2[e], c[e], sn[e]);
+    }
+    uint16_t* op = p.k_out + b * p.ko_sb + (int64_t)t * p.ko_st + (hg + j * HG) * p.ko_sh + 8 * ch;
+    *reinterpret_cast<u32x4*>(op) = pack8(y1);
+    *reinterpret_cast<u32x4*>(op + HALF) = pack8(y2);
   }
-  *reinterpret_cast<u32x4*>(op) = pack8(y1);
-  *reinterpret_cast<u32x4*>(op + HALF) = pack8(y2);
 }
 
 // Scalar kernel for head dims the MFMA kernel does not cover (any even D <= 256) and for fp32
@@ -891,8 +907,10 @@ static int launch_mfma(PrefillParams p, bool rope_in_kernel, hipStream_t s) {
   }
   if (p.cos != nullptr && !rope_in_kernel) {
     // Pre-pass: rotate K once into k_out, then attend over k_out.
-    const int64_t total = (int64_t)p.B * p.T * p.H * (D / 16);
-    hipLaunchKernelGGL(rope_k_kernel<D>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, p);
+    const int hpt = p.H % 2 == 0 ? 2 : 1;
+    const int64_t total = (int64_t)p.B * p.T * (p.H / hpt) * (D / 16);
+    if (hpt == 2) hipLaunchKernelGGL((rope_k_kernel<D, 2>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((rope_k_kernel<D, 1>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, p);
     DAISY_CHECK_LAUNCH("rope_k_kernel");
     p.k = p.k_out; p.k_sb = p.ko_sb; p.k_st = p.ko_st; p.k_sh = p.ko_sh;
     hipLaunchKernelGGL((prefill_tile_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);

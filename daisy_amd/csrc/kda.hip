@@ -222,7 +222,19 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   }
   const int n_live = t_end - t0;                  // live rows of the chunk when < 64
   const int64_t ci = (int64_t)h * p.nc_total + gc;
-  auto row_off = [&](int r) -> int64_t { return (((int64_t)t0 + r) * p.H + h) * KD; };
+  // Addresses: a wavefront-uniform 64-bit base per array (the chunk's first token row of this head, or
+  // the chunk's slot in the workspace) plus a 32-bit offset per lane.  Written out once here: as one
+  // 64-bit expression per access the row products were rebuilt per lane and load (seven vector
+  // instructions each, three of them at a quarter of the rate).
+  const uint32_t row_stride = (uint32_t)p.H * KD;                 // elements between token rows of one head
+  const int64_t tok_base = ((int64_t)t0 * p.H + h) * KD;          // first element of the chunk's first row
+  const uint16_t* const q_c = p.q + tok_base;
+  const uint16_t* const k_c = p.k + tok_base;
+  const uint16_t* const v_c = p.v + tok_base;
+  const float* const beta_c = p.beta + ((int64_t)t0 * p.H + h);
+  uint16_t* const qg_c = p.Qg + ci * KC * KD;
+  uint16_t* const pm_c = p.Pm + ci * KC * KC;
+  float* const u0_c = p.U0T + ci * KD * KC;
 
   // ---- phase 0a: G = cumsum(g) -----------------------------------------------
   // Every global load of the chunk (g here, then q, k, v and beta of phase 0b) goes out before
@@ -234,7 +246,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   u32x4 qraw[4], vraw[4], kraw[4];
   float btv[4];
   {
-    const int d = tid & 127, half = tid >> 7;
+    const int d = tid & 127, half = __builtin_amdgcn_readfirstlane(tid >> 7);   // the row of a g load is wavefront-uniform
     float gv[32];
     // Rows past the end re-read the last row (always valid) and are zeroed afterwards, so that
     // the loads carry no branches and all go out together; the dtype is decided once, outside
@@ -244,14 +256,14 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
     if (p.g_bf16) {
 #pragma unroll
       for (int i = 0; i < 32; ++i) {
-        const int64_t off = row_off(min(32 * half + i, n_live - 1)) + d;
-        graw[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p.g) + (off >> 1));
+        const uint32_t* row = reinterpret_cast<const uint32_t*>(p.g) + ((tok_base + (uint32_t)min(32 * half + i, n_live - 1) * row_stride) >> 1);
+        graw[i] = __builtin_nontemporal_load(row + (uint32_t)(d >> 1));
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 32; ++i) {
-        const int64_t off = row_off(min(32 * half + i, n_live - 1)) + d;
-        graw[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p.g) + off);
+        const uint32_t* row = reinterpret_cast<const uint32_t*>(p.g) + (tok_base + (uint32_t)min(32 * half + i, n_live - 1) * row_stride);
+        graw[i] = __builtin_nontemporal_load(row + (uint32_t)d);
       }
     }
     const bool g16 = p.g_bf16 != 0, odd = (d & 1) != 0;
@@ -264,11 +276,11 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
     for (int i = 0; i < 4; ++i) {
       const int r = r4 + 16 * i;
       const int rc = min(r, n_live - 1);
-      const int64_t off = row_off(rc) + 8 * cc;
-      kraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.k + off));
-      vraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.v + off));
-      qraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.q + off));
-      btv[i] = p.beta[((int64_t)t0 + rc) * p.H + h];
+      const uint32_t off = (uint32_t)rc * row_stride + 8u * cc;
+      kraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(k_c + off));
+      vraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(v_c + off));
+      qraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q_c + off));
+      btv[i] = beta_c[(uint32_t)rc * (uint32_t)p.H];
     }
     __builtin_amdgcn_sched_barrier(0);
     // G holds the running sum in units of log 2 (g * log2(e)): every exponential below is a bare
@@ -345,7 +357,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
         o8[4 + e] = sc * __builtin_amdgcn_exp2f(g1[e]) * qf[4 + e];
       }
       const u32x4 pk = pack8(o8);
-      uint16_t* dst = p.Qg + (ci * KC + r) * KD + pos0;
+      uint16_t* dst = qg_c + (uint32_t)(r * KD + pos0);
       u32x2 lo2 = {pk.x, pk.y}, hi2 = {pk.z, pk.w};
       __builtin_nontemporal_store(lo2, reinterpret_cast<u32x2*>(dst));        // channels 8cc+0..3
       __builtin_nontemporal_store(hi2, reinterpret_cast<u32x2*>(dst + 8));    // channels 8cc+4..7
@@ -426,7 +438,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       const int i = 16 * I + 4 * q4 + r;
       av[r] = bt[i] * rk[i] * rkj * accA[r];
       const float pv = (j <= i) ? p.scale * rq[i] * rkj * accP[r] : 0.f;
-      p.Pm[(ci * KC + i) * KC + perm32(j)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
+      pm_c[(uint32_t)(i * KC + perm32(j))] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
     }
     if (I == J) {
       *reinterpret_cast<f32x4*>(&Ad[I][li][4 * q4]) = av;   // entries with i <= j are never read
@@ -486,7 +498,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
         const float rkj = rk[rj];
         if (j < il) Ad[I][j][il] = bi * rkj * av;
         pv = (j <= il) ? qs * rkj * pv : 0.f;
-        p.Pm[(ci * KC + ri) * KC + perm32(rj)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
+        pm_c[(uint32_t)(ri * KC + perm32(rj))] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
       }
     }
   };
@@ -562,7 +574,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       const int i = 16 * I + 4 * q4 + r;
       av[r] = bt[i] * rk[i] * rkj * accA[r];
       const float pv = (j <= i) ? p.scale * rq[i] * rkj * accP[r] : 0.f;
-      p.Pm[(ci * KC + i) * KC + perm32(j)] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
+      pm_c[(uint32_t)(i * KC + perm32(j))] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
     }
     *reinterpret_cast<f32x4*>(&Ad[I][li][4 * q4]) = av;   // entries with i <= j are never read
   };
@@ -593,7 +605,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
       for (int I = 0; I < 4; I += 2)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) p.Pm[(ci * KC + 16 * I + 4 * q4 + r) * KC + perm32(16 * (I + 1) + li)] = 0;
+        for (int r = 0; r < 4; ++r) pm_c[(uint32_t)((16 * I + 4 * q4 + r) * KC + perm32(16 * (I + 1) + li))] = 0;
     }
   }
   __syncthreads();
@@ -754,7 +766,7 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
           for (int r = 0; r < 4; ++r)
             Wst[(16 * I + 4 * q4 + r) * KD + pc] = (uint16_t)(pack_bf16x2(-X[I][r], 0.f) & 0xffffu);
       } else {
-        float* dst = p.U0T + (ci * KD + col) * KC + 4 * q4;
+        float* dst = u0_c + (uint32_t)(col * KC + 4 * q4);
 #pragma unroll
         for (int I = 0; I < 4; ++I) __builtin_nontemporal_store(X[I], reinterpret_cast<f32x4*>(dst + 16 * I));
       }

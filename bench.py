@@ -256,7 +256,7 @@ def cpu_prefill_baseline(q, k, v, cos, sin, W, sample):
 # HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # (profiles/prefill_tile_kernel_c2_hbm_traffic.txt), each scaled by the factor the same counter
 # shows for the 1 GiB copy of `--only copy` (2.000 for reads, 1.000 for writes).
-PREFILL_C2_TRAFFIC_BYTES = (122578 * 2 + 65536) * 1024
+PREFILL_C2_TRAFFIC_BYTES = (117121 * 2 + 65536) * 1024
 PREFILL_C2_TRAFFIC_SOURCE = ("recorded counter value from profiles/prefill_tile_kernel_c2_hbm_traffic.txt "
                              "(rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this kernel on this workload); not measured by this run")
 

@@ -468,14 +468,16 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(Prefil
 
 // Main kernel (keys already rotated, or no RoPE on keys).  32-key tiles, and nothing of a step is
 // overlapped inside a wavefront: scores, softmax and the product of one tile follow each other.  The
-// kernel is small instead -- 163 VGPRs and 32 KiB of LDS at D = 128 -- so that THREE workgroups fit a
+// kernel is small instead -- 167 VGPRs and 48 KiB of LDS at D = 128 -- so that THREE workgroups fit a
 // CU, three wavefronts a SIMD, and the latencies of one wavefront's step (the issue of its tile
 // copies, the LDS operand reads, the softmax chain, the barrier) are covered by the other two: matrix
 // instructions of one wavefront and vector instructions of another do run side by side on a SIMD.
 //   step n:  copies K(n+1), V(n+1) -> the other buffer;  S = K(n) Q^T;  P = softmax(S);  O += V(n)^T P;
 //            wait for the copies, barrier.
 // A wavefront computes only the tiles its 32 queries can see; a tile at the window / document edge or
-// on the diagonal is masked per element.
+// on the diagonal is masked per element.  The Q block at the start and the O block at the end pass
+// through an LDS area of the wavefront's own, so that every global access of the kernel covers whole
+// rows (a CU's memory path, shared by its three workgroups, is busy per cache line touched).
 constexpr int kTBN = 32;   // key rows per tile of prefill_tile_kernel
 template <int D>
 __global__ __launch_bounds__(kPrefillThreads, 3) void prefill_tile_kernel(PrefillParams p) {

@@ -92,6 +92,29 @@ def test_prefill_strided_views_of_merged_qkv():
     assert_close_bf16(o, ref, "o")
 
 
+@pytest.mark.parametrize("H,D,T", [(4, 128, 333), (3, 128, 200), (2, 64, 130)])
+def test_prefill_outputs_with_caller_strides(H, D, T):
+    """o and the rotated keys written into views with other strides ([B, H, T, D] storage, the ring's
+    layout; rows of a wider buffer) equal the contiguous results bit for bit, and nothing outside the
+    views is touched.  Odd H takes the one-head-per-thread pre-pass, even H the two-head one."""
+    B, W = 2, 70
+    q, k, v = (t.cuda() for t in _inputs(B, T, H, D, seed=21))
+    cos, sin = (t.cuda() for t in oracle.rope_tables(D, T))
+    o_ref, k_ref = ops.prefill_attention(q, k, v, window=W, cos=cos, sin=sin)
+    # [B, H, T, D] storage seen as [B, T, H, D]
+    o_bhtd = torch.full((B, H, T, D), 7.0, dtype=torch.bfloat16, device="cuda:0")
+    k_bhtd = torch.full((B, H, T, D), 7.0, dtype=torch.bfloat16, device="cuda:0")
+    ops.prefill_attention(q, k, v, window=W, cos=cos, sin=sin, out=o_bhtd.transpose(1, 2), k_out=k_bhtd.transpose(1, 2))
+    assert torch.equal(o_bhtd.transpose(1, 2), o_ref) and torch.equal(k_bhtd.transpose(1, 2), k_ref)
+    # rows of a wider buffer: [B, T, H, D + 16] with the last 16 channels of every row left alone
+    o_wide = torch.full((B, T, H, D + 16), 7.0, dtype=torch.bfloat16, device="cuda:0")
+    k_wide = torch.full((B, T, H, D + 16), 7.0, dtype=torch.bfloat16, device="cuda:0")
+    ops.prefill_attention(q, k, v, window=W, cos=cos, sin=sin, out=o_wide[..., :D], k_out=k_wide[..., :D])
+    assert torch.equal(o_wide[..., :D], o_ref) and torch.equal(k_wide[..., :D], k_ref)
+    assert bool((o_wide[..., D:] == 7.0).all()) and bool((k_wide[..., D:] == 7.0).all())
+    say(f"strided outputs H={H} D={D} T={T}: equal to the contiguous results")
+
+
 def test_prefill_long_sequence_sampled_rows():
     """T = 16384 with a 2048 window: spot-check rows against the blockwise oracle."""
     B, T, H, D, W = 1, 16384, 2, 128, 2048

@@ -807,7 +807,8 @@ constexpr int kStageWn = 0;                   // [64][128] bf16
 constexpr int kStageQg = 16384;               // [64][128] bf16
 constexpr int kStageKtH = 32768;              // [128][64] bf16
 constexpr int kStageKtL = 49152;              // [128][64] bf16
-constexpr int kStageBytes = 65536;
+constexpr int kStageDec = 65536;               // [128] fp32: the chunk's total decay per key channel
+constexpr int kStageBytes = 65536 + 1024;
 
 typedef __attribute__((address_space(3))) const char* lds_cptr;
 __device__ __forceinline__ bf16x8 lds_bf16x8(lds_cptr p) {
@@ -870,6 +871,10 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
         copy16_to_lds_async(kh + (j >> 1) * 1024, src128[j & 1], dst + kStageKtH + j * 1024);
         copy16_to_lds_async(kl + (j >> 1) * 1024, src128[j & 1], dst + kStageKtL + j * 1024);
       }
+      // the 512 bytes of the chunk's decay ride along (half a copy): fetched by the computing wavefronts
+      // themselves they were four more vector-memory instructions per wavefront and chunk, and the number
+      // of such instructions a CU issues per chunk is what the chunk time follows
+      if (pw == 0 && lane < 32) copy16_to_lds_async(reinterpret_cast<const uint16_t*>(p.dec + ci * KD), lane * 16, dst + kStageDec);
     };
     // The four workgroups of a (batch, head) copy the same 64 KB per chunk at about the same
     // time and would all wait out the full HBM latency.  Each touches a quarter of a later chunk
@@ -945,16 +950,13 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
       S[i][r] = p.s0 ? p.s0[((int64_t)bh * KD + 16 * (4 * hf + i) + 4 * q4 + r) * KD + vcol] : 0.f;
   }
 
-  // What depends on the value column or is small comes straight from global memory, one chunk
-  // ahead: U0 (accumulator initial value of U), the chunk's total decay of this wavefront's
-  // state rows, and this wavefront's rows of P as left operand.
-  auto load_direct = [&](int n, f32x4* u0, f32x4* dcy, bf16x8 (*pa)[2]) {
+  // What depends on the value column comes straight from global memory, one chunk ahead: U0
+  // (accumulator initial value of U) and this wavefront's rows of P as left operand.
+  auto load_direct = [&](int n, f32x4* u0, bf16x8 (*pa)[2]) {
     const int64_t ci = ci0 + n;
     const float* src = p.U0T + (ci * KD + vcol) * KC + 4 * q4;
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) u0[mt] = *reinterpret_cast<const f32x4*>(src + 16 * mt);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) dcy[i] = *reinterpret_cast<const f32x4*>(p.dec + ci * KD + 16 * (4 * hf + i) + 4 * q4);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -963,26 +965,26 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
   };
   // Two sets, used in turn by even and odd chunks (the chunk loop is unrolled by two so that no
   // register copy, which would have to wait for the loads, sits between them and their use).
-  f32x4 u0[2][4], dcy[2][4];
+  f32x4 u0[2][4];
   bf16x8 pa[2][2][2];
   bf16x8 Sb[4];   // the state as right operand, by local channel group
   Sb[0] = pack_acc2(S[0], S[1]);
   Sb[1] = pack_acc2(S[2], S[3]);
   xch[0][wave][0][lane] = __builtin_bit_cast(u32x4, Sb[0]);
   xch[0][wave][1][lane] = __builtin_bit_cast(u32x4, Sb[1]);
-  if (nc > 0) load_direct(0, u0[0], dcy[0], pa[0]);
+  if (nc > 0) load_direct(0, u0[0], pa[0]);
   __syncthreads();
 
   auto chunk_step = [&](int n, auto parity) {
     constexpr int st = decltype(parity)::value;
     f32x4 (&u0c)[4] = u0[st];
-    f32x4 (&dcc)[4] = dcy[st];
+    f32x4 dcc[4];
     bf16x8 (&pac)[2][2] = pa[st];
     // The direct loads of the next chunk go out first thing, ahead of the burst of copies of the
     // data-moving wavefronts (the memory pipeline of a CU is one queue: behind that burst they
     // would block this wavefront for thousands of cycles), and are waited for at the end of the
     // chunk, so that no wait for them can end up behind newer loads.
-    if (n + 1 < nc) load_direct(n + 1, u0[st ^ 1], dcy[st ^ 1], pa[st ^ 1]);
+    if (n + 1 < nc) load_direct(n + 1, u0[st ^ 1], pa[st ^ 1]);
     __builtin_amdgcn_sched_barrier(0);
     lds_cptr sb = stage0 + st * kStageBytes;
 
@@ -998,6 +1000,8 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
 #pragma unroll
       for (int i = 0; i < 2; ++i) qa[i][mm] = lds_bf16x8(sb + kStageQg + 4096 * (2 * hf + i) + rdk[mm]);
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dcc[i] = *(const f32x4 __attribute__((address_space(3)))*)(sb + kStageDec + 4 * (16 * (4 * hf + i) + 4 * q4));
     __builtin_amdgcn_sched_barrier(0);
 
     // U = U0 + (-W) S0 (all four row tiles) and O = Qg S0 (this wavefront's two row tiles).

@@ -427,9 +427,12 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
       }
       const bf16x8 vb = __builtin_bit_cast(bf16x8, pack8(bk));
       accA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[m], vb, accA, 0, 0, 0);
-      accP = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vq[m], vb, accP, 0, 0, 0);
+      // P comes out transposed (operands swapped: both operand layouts hold 8 contraction indices of
+      // one row / column per lane): a lane then owns four consecutive columns of one row of P, one
+      // 8-byte store instead of four 2-byte ones.
+      accP = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb, vq[m], accP, 0, 0, 0);
     }
-    // accumulator: lane holds column j = 16J + li, rows i = 16I + 4*q4 + r
+    // accA: lane holds column j = 16J + li, rows i = 16I + 4*q4 + r
     const int j = 16 * J + li;
     const float rkj = rk[j];
     f32x4 av;
@@ -437,8 +440,18 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
     for (int r = 0; r < 4; ++r) {
       const int i = 16 * I + 4 * q4 + r;
       av[r] = bt[i] * rk[i] * rkj * accA[r];
-      const float pv = (j <= i) ? p.scale * rq[i] * rkj * accP[r] : 0.f;
-      pm_c[(uint32_t)(i * KC + perm32(j))] = (uint16_t)(pack_bf16x2(pv, 0.f) & 0xffffu);
+    }
+    {
+      // accP: lane holds row i = 16I + li, columns j = 16J + 4*q4 + r (stored positions perm32(j): the
+      // four are consecutive, perm32 keeps the low two bits)
+      const int ip = 16 * I + li, jp = 16 * J + 4 * q4;
+      const f32x4 rk4 = lds_f4(&rk[jp]);
+      const float qs = p.scale * rq[ip];
+      float pv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) pv[r] = (jp + r <= ip) ? qs * rk4[r] * accP[r] : 0.f;
+      const u32x2 w = {pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3])};
+      *reinterpret_cast<u32x2*>(pm_c + (uint32_t)(ip * KC + perm32(jp))) = w;
     }
     if (I == J) {
       *reinterpret_cast<f32x4*>(&Ad[I][li][4 * q4]) = av;   // entries with i <= j are never read

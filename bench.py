@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME] [--no-cpu]
 
-NAME is one of prefill | ceiling | plumbing | module | long | decode | kda | next | copy; "copy" runs a plain 1 GiB
+NAME is one of prefill | ceiling | plumbing | module | long | decode | decode_b1 | kda | next | copy; "copy" runs a plain 1 GiB
 device copy and nothing else (the known-size kernel against which the HBM
 counters FETCH_SIZE / WRITE_SIZE are calibrated under rocprofv3 --pmc).
 
@@ -193,18 +193,13 @@ def bench_prefill_c2(steps, warmup, cpu_baseline=True):
     ms_kernel, ms_kernel_mean = time_gpu(attn_only, steps, warmup, per_launch=True)
     clock_after = probe_matrix_rate(False, 4000)["clock_mhz"] if SUSTAINED_CLOCK else None
 
-    def fused():
-        ops.prefill_attention(q, k, v, window=W, scale=SCALE, cos=cos, sin=sin, out=o2, k_out=k_rot, rotate_k_in_kernel=True)
-
-    ms_fused = time_gpu(fused, max(steps // 2, 1), max(warmup // 2, 1))
-
     flops = prefill_flops(B, T, H, D, W)
     res = {
         "workload": "prefill_c2_B8_T4096_H8_D128_W1024_rope",
         "ms_full": ms_full, "ms_full_first_steps_from_idle": ms_full_from_idle,
         "ms_full_sustained": ms_full_sustained, "full_sustained_launches": n_full_sustained,
         "tflops_full_sustained": flops / ms_full_sustained / 1e9,
-        "ms_kernel": ms_kernel, "ms_kernel_mean": ms_kernel_mean, "ms_rotate_k_in_kernel": ms_fused,
+        "ms_kernel": ms_kernel, "ms_kernel_mean": ms_kernel_mean,
         "flops": flops,
         "tflops_full": flops / ms_full / 1e9, "tflops_kernel": flops / ms_kernel / 1e9,
         "frac_of_peak_kernel": flops / ms_kernel / 1e9 / PEAK_BF16_TFLOPS,
@@ -253,12 +248,32 @@ def cpu_prefill_baseline(q, k, v, cos, sin, W, sample):
             "kind": "port", "sample": f"{sample}; {runs} passes in {dt * runs:.1f} s", "seconds": dt}
 
 
-# HBM bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (profiles/prefill_tile_kernel_c2_hbm_traffic.txt), each scaled by the factor the same counter
-# shows for the 1 GiB copy of `--only copy` (2.000 for reads, 1.000 for writes).
-PREFILL_C2_TRAFFIC_BYTES = (117121 * 2 + 65536) * 1024
-PREFILL_C2_TRAFFIC_SOURCE = ("recorded counter value from profiles/prefill_tile_kernel_c2_hbm_traffic.txt "
-                             "(rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this kernel on this workload); not measured by this run")
+# HBM bytes per launch of the headline kernel: a recorded counter value, not something this run measures.  It is read
+# from the committed rocprofv3 summary, whose line
+#   bench.py reads: kernel=<name> FETCH_SIZE_KiB=<n> WRITE_SIZE_KiB=<n> fetch_factor=<f> write_factor=<f>
+# names the kernel the counters were taken on (FETCH_SIZE / WRITE_SIZE per dispatch, each scaled by the factor the same
+# counter shows for the 1 GiB copy of `--only copy`).  A summary taken on another kernel than the one this run launches
+# is not used: the line then carries no traffic figure.
+PREFILL_C2_KERNEL = "prefill_tile_kernel<128>"
+PREFILL_C2_TRAFFIC_FILE = os.path.join("profiles", "prefill_tile_kernel_c2_hbm_traffic.txt")
+
+
+def recorded_traffic(path, kernel):
+    """(bytes per launch or None, a sentence on where the figure comes from)."""
+    import re
+    try:
+        with open(os.path.join(ROOT, path)) as f:
+            text = f.read()
+    except OSError:
+        return None, f"{path} is missing: no recorded counter value"
+    m = re.search(r"bench\.py reads: kernel=(\S+) FETCH_SIZE_KiB=(\d+) WRITE_SIZE_KiB=(\d+) fetch_factor=([\d.]+) write_factor=([\d.]+)", text)
+    if m is None:
+        return None, f"{path} has no 'bench.py reads:' line"
+    if m.group(1) != kernel:
+        return None, f"{path} was recorded on {m.group(1)}, this run launches {kernel}: figure not used"
+    nbytes = int((int(m.group(2)) * float(m.group(4)) + int(m.group(3)) * float(m.group(5))) * 1024)
+    return nbytes, (f"recorded counter value from {path} (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of {kernel} on this workload, "
+                    "scaled by the factors of a 1 GiB copy); not measured by this run")
 
 
 def bench_plumbing_c1(steps, warmup, cpu_baseline=True):
@@ -468,18 +483,14 @@ def bench_kda_c5(steps, warmup, cpu_baseline=True):
     return out
 
 
-def bench_next_rows(steps, warmup):
-    """The callers either side of the kernels: model-level prefill / step glue on an attention stack,
-    attention under training-time block masks, and the KDA layer."""
+def attention_stack(L, vocab, dim, H, D, window, max_len):
+    """A stack of attention layers with the attributes the model-level glue walks (embed, blocks, lm_head_w, window
+    sizes ...): the attention part of a Daisy model, no MLPs, random bf16 weights."""
     import torch.nn as nn
-    import torch.nn.functional as F
-    from daisy_amd import CausalSelfAttention, KVCache, KimiLinearSelfAttention, build_block_window_masks, core, ops
-    dev = "cuda:0"
-    out = {}
+    from daisy_amd import CausalSelfAttention
 
-    # ---- glue: 4 attention layers, 16 sequences, prompt 4100, ring of 4096 (wrapped) ----------------
     class Block(nn.Module):
-        def __init__(self, dim, H, D, max_len):
+        def __init__(self):
             super().__init__()
             self.attn = CausalSelfAttention(dim, H, D, max_seq_len=max_len)
             with torch.no_grad():
@@ -494,10 +505,10 @@ def bench_next_rows(steps, warmup):
             return x + y, k, v
 
     class Stack(nn.Module):
-        def __init__(self, L=4, vocab=1024, dim=1024, H=8, D=128, window=4096, max_len=8192):
+        def __init__(self):
             super().__init__()
             self.embed = nn.Embedding(vocab, dim)
-            self.blocks = nn.ModuleList([Block(dim, H, D, max_len) for _ in range(L)])
+            self.blocks = nn.ModuleList([Block() for _ in range(L)])
             self.skip_map, self.skip_weights, self.ve_module_map = {}, None, {}
             self.lm_head_w = nn.Parameter(torch.randn(vocab, dim) * 0.02)
             self.window_size = self.attn_window_size = window
@@ -505,9 +516,85 @@ def bench_next_rows(steps, warmup):
             self.attn_num_heads, self.attn_head_dim = H, D
             self.bfloat16()
 
+    return Stack()
+
+
+def bench_decode_b1(steps, warmup):
+    """The regime of the reference's generator (inference/generate.py:76: batch 1) at the shape of
+    model_specs/daisy_milli.yml (12 heads of 128, window 8192, model dim 1536), 12 attention layers, ring full:
+    per-token time of a model step, eager and as one recorded HIP graph, and of the attention launches alone
+    (the one-launch step over the 12 rings, back to back), against the bytes of ring a token reads."""
+    from daisy_amd import KVCache, core, ops
+    from daisy_amd.functional import NORM_EPS_BF16
+    dev = "cuda:0"
+    L, H, D, W, dim, vocab = 12, 12, 128, 8192, 1536, 8192
+    torch.manual_seed(0)
+    out = {"workload": f"decode_b1_L{L}_H{H}_D{D}_W{W}_dim{dim}", "batch": 1}
+    with torch.no_grad():
+        model = attention_stack(L, vocab, dim, H, D, W, 2 * W + 64).to(dev).eval()
+        cache = KVCache(L=L, B=1, H=H, W=W, D=D, device=dev, dtype=torch.bfloat16)
+        g = torch.Generator(device=dev).manual_seed(0)
+        cache.k.copy_(torch.randn(cache.k.shape, generator=g, device=dev, dtype=torch.float32))
+        cache.v.copy_(torch.randn(cache.v.shape, generator=g, device=dev, dtype=torch.float32))
+        cache.t = t_before = W + 100                  # the ring has wrapped: every step reads W rows per layer
+        tok = torch.randint(1, vocab, (1,), device=dev)
+
+        def step_eager():
+            cache.t = t_before
+            return core.step(model, tok, cache)
+
+        ms_eager = time_gpu(step_eager, max(steps, 32), max(warmup, 8))
+        recorded = core.GraphedStep(model, cache)
+
+        def step_recorded():
+            cache.t = t_before
+            return recorded(tok)
+
+        ms_graph = time_gpu(step_recorded, max(4 * steps, 128), max(warmup, 8))
+        # the attention launches alone: the one-launch step (norm, RoPE, append, attention) on each layer's ring
+        cos, sin = model.blocks[0].attn.rotary.cos, model.blocks[0].attn.rotary.sin
+        raw = torch.randn(1, 3 * H, D, generator=g, device=dev).bfloat16()
+        pos = torch.full((1,), t_before, dtype=torch.int32, device=dev)
+        o = torch.empty(1, H, D, dtype=torch.bfloat16, device=dev)
+        variants = {}
+        for nsplit in (0, 8, 16, 32, 64):
+            ws = torch.empty(max(ops.decode_workspace_bytes(1, H, D, W, nsplit), 1), dtype=torch.uint8, device=dev)
+
+            def attn_layers():
+                for i in range(L):
+                    ops.attn_step(raw[:, :H], raw[:, H:2 * H], raw[:, 2 * H:], cache.k[i], cache.v[i], pos, cos=cos, sin=sin,
+                                  eps=NORM_EPS_BF16, scale=SCALE, out=o, workspace=ws, nsplit=nsplit)
+
+            graph = torch.cuda.CUDAGraph()
+            attn_layers()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph):
+                attn_layers()
+            variants["library_choice" if nsplit == 0 else f"nsplit{nsplit}"] = time_gpu(graph.replay, max(4 * steps, 128), 8)
+            del graph
+    nbytes = L * 2 * W * H * D * 2
+    row = lambda ms: {"ms_per_token": ms, "gbs": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+    out.update({"kv_bytes_per_token": nbytes, "model_step_eager": row(ms_eager), "model_step_recorded_graph": row(ms_graph),
+                "attention_launches_only_recorded_graph": {k: row(v) for k, v in variants.items()},
+                "what": "model step = embed, 12 x (norm, QKV projection, one-launch attention step, output projection, residual), "
+                        "final norm, vocabulary projection; attention launches only = the 12 decode launches (+ their split "
+                        "combines) replayed as one graph"})
+    return out
+
+
+def bench_next_rows(steps, warmup):
+    """The callers either side of the kernels: model-level prefill / step glue on an attention stack,
+    attention under training-time block masks, and the KDA layer."""
+    import torch.nn as nn
+    import torch.nn.functional as F
+    from daisy_amd import CausalSelfAttention, KVCache, KimiLinearSelfAttention, build_block_window_masks, core, ops
+    dev = "cuda:0"
+    out = {}
+
+    # ---- glue: 4 attention layers, 16 sequences, prompt 4100, ring of 4096 (wrapped) ----------------
     torch.manual_seed(0)
     with torch.no_grad():
-        model = Stack().to(dev).eval()
+        model = attention_stack(L=4, vocab=1024, dim=1024, H=8, D=128, window=4096, max_len=8192).to(dev).eval()
         Bs, T0, W, L = 16, 4100, 4096, 4
         ids = torch.randint(1, 1024, (Bs, T0), device=dev)
         cache = KVCache(L=L, B=Bs, H=8, W=W, D=128, device=dev, dtype=torch.bfloat16)
@@ -610,7 +697,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--only", default=None, help="prefill | ceiling | plumbing | module | long | decode | kda | next | copy (default: all but copy)")
+    ap.add_argument("--only", default=None, help="prefill | ceiling | plumbing | module | long | decode | decode_b1 | kda | next | copy (default: all but copy)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -647,6 +734,8 @@ def main():
     if want("decode"):
         extra["decode_c4"] = bench_decode_c4(256, 16, cpu)
         extra["hbm_read_ceiling"] = dict(probe_read_rate(), what="read-only stream of 2 GiB, 8192 workgroups, 128 B in flight per lane")
+    if want("decode_b1"):
+        extra["decode_b1"] = bench_decode_b1(args.steps, args.warmup)
     if want("next"):
         extra["next_rows"] = bench_next_rows(args.steps, args.warmup)
     if want("kda"):
@@ -667,13 +756,22 @@ def main():
                    "timed": "K rotation pre-pass + attention kernel, inputs and outputs in HBM"},
     }
     if head is not None:
+        # What precedes the timed steps, at the top level: the GPU is brought to its settled clocks by a run of the same
+        # step (pre_timed_launches, then `warmup` more); the first `steps` steps from an idle GPU are reported beside it.
+        line["pre_timed_launches"] = head["full_sustained_launches"]
+        line["ms_per_step_first_steps_from_idle"] = head["ms_full_first_steps_from_idle"]
+        line["value_first_steps_from_idle"] = head["flops"] / head["ms_full_first_steps_from_idle"] / 1e9
+        line["config"]["timed"] += (f"; {args.steps} steps after {head['full_sustained_launches']} back-to-back launches of the same step "
+                                    f"and {args.warmup} warm-up steps (settled clocks); from an idle GPU the first {args.steps} steps "
+                                    f"take {head['ms_full_first_steps_from_idle']:.4f} ms each")
         # The roofline figure is the lower of the burst median and the sustained run (at least a second of launches).
         burst, sus = head["tflops_kernel"], head["sustained"]["tflops_kernel"]
         use_sus = sus < burst
+        traffic, traffic_source = recorded_traffic(PREFILL_C2_TRAFFIC_FILE, PREFILL_C2_KERNEL)
         line["roofline"] = {"bound": "mfma", "achieved": min(burst, sus), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                            "frac": min(burst, sus) / PEAK_BF16_TFLOPS, "traffic": PREFILL_C2_TRAFFIC_BYTES,
-                            "traffic_source": PREFILL_C2_TRAFFIC_SOURCE, "traffic_min_bytes": head["min_hbm_bytes"],
-                            "kernel": "prefill_tile_kernel<128>",
+                            "frac": min(burst, sus) / PEAK_BF16_TFLOPS, "traffic": traffic,
+                            "traffic_source": traffic_source, "traffic_min_bytes": head["min_hbm_bytes"],
+                            "kernel": PREFILL_C2_KERNEL,
                             "ms": head["sustained"]["ms_kernel"] if use_sus else head["ms_kernel"],
                             "timing": ("sustained: mean over %d back-to-back launches (%.2f s)" % (head["sustained"]["launches"], head["sustained"]["seconds"]))
                                       if use_sus else "median of per-launch HIP event pairs over the timed steps",

@@ -16,8 +16,7 @@ import torch
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libdaisy_hip.so")
 _lib: Optional[ctypes.CDLL] = None
 
-ABI_VERSION = 2
-PREFILL_ROTATE_K_IN_KERNEL = 1
+ABI_VERSION = 3
 STATUS_POSITION_PAST_TABLES = 1
 DECODE_STATIC_SCRATCH_BYTES = 4 << 20
 
@@ -57,6 +56,7 @@ SIGNATURES = {
         c_int, c_int, c_int,                                    # B, H, D
         c_int, c_int, c_int,                                    # n_rows, new_idx, write_back
         c_float, c_void_p]),                                    # scale, stream
+    "daisy_decode_noalloc_init": (c_int, []),
     "daisy_decode_fwd_noalloc": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,      # q, k_new, v_new (+strides)
         c_void_p, _I64P, c_void_p, _I64P,                       # k_cache, v_cache (+strides)

@@ -335,9 +335,6 @@ class CausalSelfAttention(nn.Module):
         else:
             self.g_ve = None
         self.debug_logging = False
-        # Set to True to rotate keys while they are staged into LDS instead of in a pre-pass
-        # (only used when fused_prep is off).
-        self.rotate_k_in_kernel = False
         # Norm + RoPE + ve mix in one streaming kernel ahead of attention (bf16 weights only);
         # False keeps norm / mix in PyTorch and rotates inside the attention call.
         self.fused_prep = True
@@ -392,8 +389,10 @@ class CausalSelfAttention(nn.Module):
         return ops.qkv_prep(q, k, v, eps=NORM_EPS_BF16, cos=cos, sin=sin, pos0=pos0, ve=ve, gate=gate,
                             k_out=k_out, v_out=v_out)
 
-    def _attend(self, x: Tensor, ve: Optional[Tensor], attn_mask, kv_out=None):
-        """Returns ``y [B, T, dim]`` and q (rotated), k (rotated), v as ``[B, T, H, D]``."""
+    def _attend(self, x: Tensor, ve: Optional[Tensor], attn_mask, kv_out=None, want_q: bool = False):
+        """Returns ``y [B, T, dim]`` and q (rotated), k (rotated), v as ``[B, T, H, D]``.  Where the kernels
+        rotate q themselves, the rotated q is computed for the caller only when ``want_q`` asks for it
+        (``prefill(debug=True)``), and is ``None`` otherwise."""
         B, T = x.size(0), x.size(1)
         mask = _as_window_mask(attn_mask)
         if mask.doc_start is not None and mask.doc_start.device != x.device:    # e.g. converted from a mask built on the CPU
@@ -412,18 +411,17 @@ class CausalSelfAttention(nn.Module):
         if dtype == torch.float32:
             # fp32 parameters (the reference's unit tests build the module so): fp32 tensors and fp32
             # arithmetic through the attention too, nothing is rounded to bf16 on the way.
-            q_rot = _apply_rope(q, cos[None, :, None, :], sin[None, :, None, :])
+            q_rot = _apply_rope(q, cos[None, :, None, :], sin[None, :, None, :]) if want_q else None
             o, k_rot = ops.prefill_attention_f32(q, k, v, window=mask.window, scale=self.attn_scale, cos=cos, sin=sin,
                                                  doc_start=mask.doc_start)
             y = F.linear(o.view(B, T, self.m_dim), self.qkvo_w[3])
             return y, q_rot, k_rot, v
         o, k_rot = ops.prefill_attention(
             self._kernel_dtype(q), self._kernel_dtype(k), self._kernel_dtype(v),
-            window=mask.window, scale=self.attn_scale, cos=cos, sin=sin, doc_start=mask.doc_start,
-            rotate_k_in_kernel=self.rotate_k_in_kernel)
+            window=mask.window, scale=self.attn_scale, cos=cos, sin=sin, doc_start=mask.doc_start)
         y = o.view(B, T, self.m_dim).to(dtype)
         y = F.linear(y, self.qkvo_w[3])
-        q_rot = _apply_rope(q, cos[None, :, None, :], sin[None, :, None, :])
+        q_rot = _apply_rope(q, cos[None, :, None, :], sin[None, :, None, :]) if want_q else None
         return y, q_rot, k_rot.to(dtype), v
 
     # -- reference interface -----------------------------------------------
@@ -444,7 +442,7 @@ class CausalSelfAttention(nn.Module):
         the way through a ``Block`` that passes only the reference's arguments on).
         ``debug`` keeps the rotated q and k as ``last_q`` / ``last_k`` like the reference
         (attention.py:176-178), as copies when they alias a destination that later steps overwrite."""
-        y, q, k, v = self._attend(x, ve, attn_mask, kv_out)
+        y, q, k, v = self._attend(x, ve, attn_mask, kv_out, want_q=debug)
         if debug:
             aliased = kv_out is not None or getattr(_as_window_mask(attn_mask), "kv_out", None) is not None
             self.last_q = q

@@ -644,8 +644,11 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 void* g_scratch_ptr[kMaxDevices] = {nullptr};
 
-// Device address of `scratch` on the current device (looked up on the first call there).
-int static_scratch(void** out) {
+// Device address of `scratch` on the current device.  The address is looked up once per device, by
+// daisy_decode_noalloc_init or by the first call on the device; the lookup may make the runtime load the
+// library's device image, which is not a thing to do while `capturing` (a stream of the caller is recording
+// a graph): then only an address found earlier is handed out.
+int static_scratch(void** out, bool capturing) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
@@ -654,6 +657,11 @@ int static_scratch(void** out) {
   }
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (g_scratch_ptr[dev] == nullptr) {
+    if (capturing) {
+      set_error("decode_noalloc: first use on device %d while the stream is capturing; call daisy_decode_noalloc_init() "
+                "on this device (or run one call) before the capture starts", dev);
+      return DAISY_ERR_INVALID_ARGUMENT;
+    }
     void* ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess || ptr == nullptr) {
@@ -666,6 +674,11 @@ int static_scratch(void** out) {
   return DAISY_OK;
 }
 }  // namespace
+
+extern "C" int daisy_decode_noalloc_init(void) {
+  void* ws = nullptr;
+  return static_scratch(&ws, /*capturing=*/false);
+}
 
 extern "C" int daisy_decode_fwd_noalloc(const void* q, const int64_t* q_strides,
                                         const void* k_new, const int64_t* k_new_strides,
@@ -686,7 +699,12 @@ extern "C" int daisy_decode_fwd_noalloc(const void* q, const int64_t* q_strides,
   }
   void* ws = nullptr;
   if (need > 0) {
-    const int rc = static_scratch(&ws);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &cap) != hipSuccess) {
+      (void)hipGetLastError();
+      cap = hipStreamCaptureStatusNone;
+    }
+    const int rc = static_scratch(&ws, cap != hipStreamCaptureStatusNone);
     if (rc != DAISY_OK) return rc;
   }
   // Every split writes its whole partial before the combine kernel reads it: nothing of the last

@@ -2,9 +2,8 @@
 //
 // Work decomposition
 //   workgroup = 4 wavefronts = 128 consecutive query rows of one (batch, head);
-//   wavefront = 32 query rows.  Key/value rows are visited in tiles (32 rows in
-//   prefill_tile_kernel, 64 in prefill_mfma_kernel), and only tiles that intersect
-//   [lo(q_first), q_last] are loaded at all, where
+//   wavefront = 32 query rows.  Key/value rows are visited in tiles of 32 rows, and
+//   only tiles that intersect [lo(q_first), q_last] are loaded at all, where
 //   lo(q) = max(q - window + 1, doc_start[q], 0) is non-decreasing in q.
 //
 // MFMA formulation (v_mfma_f32_32x32x16_bf16, wave64)
@@ -28,9 +27,8 @@
 // lanes L/4, L/4+4, L/4+8, L/4+12; with lane i of a block addressing key i/4,
 // channels 4*(i%4)..+3, lane i receives channel i of four consecutive keys.
 //
-// Two kernels share this structure: prefill_tile_kernel (keys need no rotation
-// here; three wavefronts per SIMD) and prefill_mfma_kernel<D, true> (keys are rotated
-// while they are staged into LDS).
+// Keys reach prefill_tile_kernel rotated: by the caller, or by rope_k_kernel, a
+// pre-pass that writes the rotated keys the reference's prefill returns anyway.
 //
 // Algorithmic work: 4*D flops per visible (query, key) pair.
 #include "common.h"
@@ -54,7 +52,6 @@ struct PrefillParams {
 };
 
 constexpr int kBM = 128;  // query rows per workgroup
-constexpr int kBN = 64;   // key rows per tile
 constexpr int kPrefillThreads = 256;
 
 __device__ __forceinline__ int row_lo(const PrefillParams& p, int q) {
@@ -97,373 +94,10 @@ __device__ __forceinline__ float pair_sum(float x) {
 
 // LDS transpose read (ds_read_b64_tr_b16); semantics in the header comment.
 typedef short s16x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ u32x2 lds_read_tr16(const uint16_t* p) {
-  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p);
-  return __builtin_bit_cast(u32x2, v);
-}
-
 typedef __attribute__((address_space(3))) const uint16_t* lds_u16_ptr;
 __device__ __forceinline__ u32x2 lds_read_tr16_as3(lds_u16_ptr p) {
   s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p);
   return __builtin_bit_cast(u32x2, v);
-}
-
-template <int D, bool ROPE_K>
-__global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(PrefillParams p) {
-  // LDS tiles are [64 rows][D] bf16 without padding; the 16-byte chunks of a row are stored
-  // XOR-swizzled (chunk c of row r sits at position c ^ f(r)) so that operand reads are free
-  // of bank conflicts.  The LDS has 64 banks of 4 bytes, i.e. 256 bytes per clock:
-  //   K: a 16-byte read serves 16 lanes per clock = 16 consecutive rows, same chunk
-  //      -> those rows must land in 16 different 16-byte slots of the 256-byte bank window;
-  //   V: an 8-byte transpose read serves 32 lanes per clock = 4 consecutive rows x 64 bytes
-  //      -> those rows must land in 4 different 64-byte slots.
-  constexpr int NS = D / 16;       // MFMA steps over the head dim for S^T
-  constexpr int NDT = D / 32;      // 32-row tiles of O^T
-  constexpr int HALF = D / 2;
-  constexpr int CPR = D / 8;       // 16-byte chunks per row
-  constexpr int RPL = 64 / CPR;    // rows covered by one wavefront copy (1 KiB)
-  constexpr int NLD = kBN / RPL / 4;   // wavefront copies per tensor, tile and wavefront
-  constexpr int TILE = kBN * D;    // elements per LDS tile
-  auto swz_k = [](int r) { return D == 128 ? (r & 15) : ((r >> 1) & 7); };
-  auto swz_v = [](int r) { return D == 128 ? 4 * (r & 3) : 4 * ((r >> 1) & 1); };
-
-  __shared__ __attribute__((aligned(1024))) uint16_t Ks[2][TILE];
-  __shared__ __attribute__((aligned(1024))) uint16_t Vs[2][TILE];
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int lq = lane & 31, lh = lane >> 5;
-
-  int bh, qb;
-  workgroup_to_block(p, bh, qb);
-  const int h = bh % p.H, b = bh / p.H;
-
-  const int q0 = qb * kBM;
-  const int qw0 = q0 + wave * 32;
-  const int qrow = min(qw0 + lq, p.T - 1);
-  const int lo_q = row_lo(p, qrow);
-  const int lo_w_min = __builtin_amdgcn_readlane(lo_q, 0);
-  const int lo_w_max = __builtin_amdgcn_readlane(lo_q, 31);
-  const int q_w_min = min(qw0, p.T - 1), q_w_max = min(qw0 + 31, p.T - 1);
-  const bool wave_live = qw0 < p.T;
-
-  const int t_lo = row_lo(p, q0) / kBN;
-  const int t_hi = min(q0 + kBM - 1, p.T - 1) / kBN;
-
-  // ---- Q fragment (B operand), RoPE fused ----------------------------------
-  bf16x8 qreg[NS];
-  {
-    const uint16_t* qptr = p.q + b * p.q_sb + (int64_t)qrow * p.q_st + h * p.q_sh + 8 * lh;
-    u32x4 raw[NS];
-#pragma unroll
-    for (int s = 0; s < NS; ++s) raw[s] = *reinterpret_cast<const u32x4*>(qptr + 16 * s);
-    if (p.cos != nullptr) {
-      const float* cr = p.cos + (int64_t)qrow * HALF + 8 * lh;
-      const float* sr = p.sin + (int64_t)qrow * HALF + 8 * lh;
-#pragma unroll
-      for (int s = 0; s < NS / 2; ++s) {
-        float x1[8], x2[8], y1[8], y2[8];
-        unpack8(raw[s], x1);
-        unpack8(raw[s + NS / 2], x2);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float c = cr[16 * s + e], sn = sr[16 * s + e];
-          y1[e] = rope_lo(x1[e], x2[e], c, sn);
-          y2[e] = rope_hi(x1[e], x2[e], c, sn);
-        }
-        raw[s] = pack8(y1);
-        raw[s + NS / 2] = pack8(y2);
-      }
-    }
-#pragma unroll
-    for (int s = 0; s < NS; ++s) qreg[s] = __builtin_bit_cast(bf16x8, raw[s]);
-  }
-
-  const uint16_t* kbase = p.k + b * p.k_sb + h * p.k_sh;
-  const uint16_t* vbase = p.v + b * p.v_sb + h * p.v_sh;
-
-  // ---- global -> LDS staging --------------------------------------------------
-  // Wavefront copy j (0 .. 64/RPL-1) of a tile moves rows RPL*j .. RPL*j+RPL-1; lane i lands
-  // at chunk position i % CPR of row i / CPR, so it fetches the chunk that belongs there.
-  const int ld_row = lane / CPR, ld_pos = lane % CPR;
-  int k_lane_off[NLD], v_lane_off[NLD];   // element offsets inside a tile's rows, per copy
-#pragma unroll
-  for (int i = 0; i < NLD; ++i) {
-    const int r = RPL * (4 * i + wave) + ld_row;
-    k_lane_off[i] = 8 * (ld_pos ^ swz_k(r));
-    v_lane_off[i] = 8 * (ld_pos ^ swz_v(r));
-  }
-
-  u32x4 kst[ROPE_K ? 2 * ((kBN * CPR / 2) / kPrefillThreads) : 1];
-  u32x4 cst[ROPE_K ? 2 * ((kBN * CPR / 2) / kPrefillThreads) : 1], sst[ROPE_K ? 2 * ((kBN * CPR / 2) / kPrefillThreads) : 1];
-  constexpr int NKC = (kBN * CPR / 2) / kPrefillThreads;   // (row, channel-pair chunk) items per thread when rotating K
-
-  // Per-lane source offsets of the wavefront copies relative to the first row of a tile
-  // (32-bit; the tile base is uniform, so the copy can use scalar-base addressing).
-  int k_src_off[NLD], v_src_off[NLD];
-#pragma unroll
-  for (int i = 0; i < NLD; ++i) {
-    const int row = RPL * (4 * i + wave) + ld_row;
-    k_src_off[i] = row * (int)p.k_st + k_lane_off[i];
-    v_src_off[i] = row * (int)p.v_st + v_lane_off[i];
-  }
-
-  const uint32_t ks_lds = lds_address(&Ks[0][0]), vs_lds = lds_address(&Vs[0][0]);
-
-  auto issue_copies = [&](int tile, auto buf_tag) {
-    constexpr int buf = decltype(buf_tag)::value;
-    const int kv0 = tile * kBN;
-    const uint16_t* kt = kbase + (int64_t)kv0 * p.k_st;
-    const uint16_t* vt = vbase + (int64_t)kv0 * p.v_st;
-    if (kv0 + kBN <= p.T) {
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        const uint32_t dst = 2 * (buf * TILE + (4 * i + wave) * 512);
-        if constexpr (!ROPE_K) copy16_to_lds_async(kt, 2 * k_src_off[i], ks_lds + dst);
-        copy16_to_lds_async(vt, 2 * v_src_off[i], vs_lds + dst);
-      }
-    } else {
-      // The tile reaches past the last row: clamp (the surplus rows are masked by causality).
-#pragma unroll
-      for (int i = 0; i < NLD; ++i) {
-        const uint32_t dst = 2 * (buf * TILE + (4 * i + wave) * 512);
-        const int row = min(RPL * (4 * i + wave) + ld_row, p.T - 1 - kv0);
-        if constexpr (!ROPE_K) copy16_to_lds_async(kt, 2 * (row * (int)p.k_st + k_lane_off[i]), ks_lds + dst);
-        copy16_to_lds_async(vt, 2 * (row * (int)p.v_st + v_lane_off[i]), vs_lds + dst);
-      }
-    }
-    if constexpr (ROPE_K) {
-#pragma unroll
-      for (int i = 0; i < NKC; ++i) {
-        const int c = tid + kPrefillThreads * i;
-        const int row = min(kv0 + c / (CPR / 2), p.T - 1);
-        const int dc = 8 * (c % (CPR / 2));
-        const uint16_t* kp = kbase + (int64_t)row * p.k_st + dc;
-        kst[2 * i] = *reinterpret_cast<const u32x4*>(kp);
-        kst[2 * i + 1] = *reinterpret_cast<const u32x4*>(kp + HALF);
-        const float* cp = p.cos + (int64_t)row * HALF + dc;
-        const float* sp = p.sin + (int64_t)row * HALF + dc;
-        cst[2 * i] = *reinterpret_cast<const u32x4*>(cp);
-        cst[2 * i + 1] = *reinterpret_cast<const u32x4*>(cp + 4);
-        sst[2 * i] = *reinterpret_cast<const u32x4*>(sp);
-        sst[2 * i + 1] = *reinterpret_cast<const u32x4*>(sp + 4);
-      }
-    }
-  };
-
-  // Completes the staging of a tile: waits for the asynchronous copies and, when K is rotated
-  // here, rotates the register-staged K rows into LDS (and publishes this workgroup's own rows).
-  auto finish_copies = [&](int tile, auto buf_tag) {
-    constexpr int buf = decltype(buf_tag)::value;
-    if constexpr (ROPE_K) {
-      const bool publish = p.k_out != nullptr && (tile * kBN) / kBM == qb;
-#pragma unroll
-      for (int i = 0; i < NKC; ++i) {
-        const int c = tid + kPrefillThreads * i;
-        const int r = c / (CPR / 2), cc = c % (CPR / 2), dc = 8 * cc;
-        float x1[8], x2[8], y1[8], y2[8];
-        unpack8(kst[2 * i], x1);
-        unpack8(kst[2 * i + 1], x2);
-        const float cs[8] = {__uint_as_float(cst[2 * i].x), __uint_as_float(cst[2 * i].y), __uint_as_float(cst[2 * i].z),
-                             __uint_as_float(cst[2 * i].w), __uint_as_float(cst[2 * i + 1].x), __uint_as_float(cst[2 * i + 1].y),
-                             __uint_as_float(cst[2 * i + 1].z), __uint_as_float(cst[2 * i + 1].w)};
-        const float sn[8] = {__uint_as_float(sst[2 * i].x), __uint_as_float(sst[2 * i].y), __uint_as_float(sst[2 * i].z),
-                             __uint_as_float(sst[2 * i].w), __uint_as_float(sst[2 * i + 1].x), __uint_as_float(sst[2 * i + 1].y),
-                             __uint_as_float(sst[2 * i + 1].z), __uint_as_float(sst[2 * i + 1].w)};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          y1[e] = rope_lo(x1[e], x2[e], cs[e], sn[e]);
-          y2[e] = rope_hi(x1[e], x2[e], cs[e], sn[e]);
-        }
-        const u32x4 a = pack8(y1), bb = pack8(y2);
-        *reinterpret_cast<u32x4*>(&Ks[buf][r * D + 8 * (cc ^ swz_k(r))]) = a;
-        *reinterpret_cast<u32x4*>(&Ks[buf][r * D + 8 * ((cc + CPR / 2) ^ swz_k(r))]) = bb;
-        const int grow = tile * kBN + r;
-        if (publish && grow < p.T) {
-          uint16_t* op = p.k_out + b * p.ko_sb + (int64_t)grow * p.ko_st + h * p.ko_sh + dc;
-          *reinterpret_cast<u32x4*>(op) = a;
-          *reinterpret_cast<u32x4*>(op + HALF) = bb;
-        }
-      }
-    }
-    // vmcnt(0) as a compiler-visible wait (encoding: vmcnt = 0, expcnt = 7, lgkmcnt = 15): the
-    // asynchronous copies have landed, and the compiler also learns that no earlier vector
-    // load is pending, so it places no conservative vmcnt waits inside the tile loop (those
-    // would wait for the copies of the NEXT tile, which it cannot see).
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    asm volatile("" ::: "memory");
-  };
-
-  // ---- accumulators -----------------------------------------------------------
-  f32x16 oacc[NDT];
-#pragma unroll
-  for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
-  float m_run = -INFINITY;  // reference maximum (scaled, log2 domain) of this lane's query
-  float l_run = 0.f;        // this lane's share of the running sum
-
-  // Per-lane LDS element offsets of the operand reads (inside one tile).
-  //   K (A operand of S^T): row = key lq of the 32-key sub-block, step s wants chunk 2s + lh.
-  //   V (A operand of O^T, LDS transpose read): the lane's block of 16 covers output channels
-  //   32dt + 16*(block & 1) + 0..15 and keys 4*lh + 0..3 (+8, +16, ... as immediates); lane i of
-  //   the block addresses key i/4, channels 4*(i%4)..+3 and receives channel i, four keys.
-  const uint16_t* k_rd[NS];
-  const uint16_t* v_rd[NDT];
-#pragma unroll
-  for (int s = 0; s < NS; ++s) k_rd[s] = &Ks[0][0] + lq * D + 8 * ((2 * s + lh) ^ swz_k(lq));
-  {
-    const int i16 = lane & 15, vrow = 4 * lh + (i16 >> 2);
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      const int chunk = 4 * dt + 2 * ((lane >> 4) & 1) + ((i16 & 3) >> 1);
-      v_rd[dt] = &Vs[0][0] + vrow * D + 8 * (chunk ^ swz_v(vrow)) + 4 * (i16 & 1);
-    }
-  }
-
-  // One tile of 64 keys.  MASKED = false: both 32-key sub-blocks are needed by this
-  // wavefront and fully visible to all of its queries (no mask, no skipping).
-  auto process_tile = [&](auto buf_tag, int kv0, auto masked_tag) {
-    constexpr int buf = decltype(buf_tag)::value;
-    constexpr bool MASKED = decltype(masked_tag)::value;
-    bool need[2] = {true, true};
-    if constexpr (MASKED) {
-#pragma unroll
-      for (int sb = 0; sb < 2; ++sb) {
-        const int kmin = kv0 + 32 * sb, kmax = kmin + 31;
-        need[sb] = kmin <= q_w_max && kmax >= lo_w_min;
-      }
-    }
-    f32x16 sacc[2];
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[sb][r] = 0.f;
-      if (!MASKED || need[sb]) {
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-          const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(k_rd[s] + (buf * TILE + 32 * sb * D)));
-          sacc[sb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[s], sacc[sb], 0, 0, 0);
-        }
-        if constexpr (MASKED) {
-          const int kmin = kv0 + 32 * sb;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int kv = kmin + 8 * (r >> 2) + 4 * lh + (r & 3);
-            if (kv > qrow || kv < lo_q) sacc[sb][r] = -INFINITY;
-          }
-        }
-      } else {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[sb][r] = -INFINITY;
-      }
-    }
-
-    // ---- online softmax (log2 domain, lazy rescale) ------------------------------
-    // The reference maximum m_run only moves when some query of the wavefront sees a
-    // score more than 8 (log2 units) above it; until then probabilities are at most 2^8,
-    // which bf16 and the fp32 sums hold without loss, and O is not touched.
-    float mt = -INFINITY;
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mt = fmaxf(mt, sacc[sb][r]);
-    mt = pair_max(mt) * p.scale_log2e;
-    if (__builtin_amdgcn_ballot_w64(mt > m_run + 8.f) != 0) {
-      const float m_new = fmaxf(m_run, mt);
-      const float mu = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fast_exp2(m_run - mu);
-      m_run = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-    }
-    const float mu = (m_run == -INFINITY) ? 0.f : m_run;
-    float lsum = 0.f;
-    bf16x8 pfrag[2][2];
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-      float pv[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        pv[r] = fast_exp2(fmaf(sacc[sb][r], p.scale_log2e, -mu));
-        lsum += pv[r];
-      }
-#pragma unroll
-      for (int m = 0; m < 2; ++m) {
-        u32x4 pk;
-        pk.x = pack_bf16x2(pv[8 * m + 0], pv[8 * m + 1]);
-        pk.y = pack_bf16x2(pv[8 * m + 2], pv[8 * m + 3]);
-        pk.z = pack_bf16x2(pv[8 * m + 4], pv[8 * m + 5]);
-        pk.w = pack_bf16x2(pv[8 * m + 6], pv[8 * m + 7]);
-        pfrag[sb][m] = __builtin_bit_cast(bf16x8, pk);
-      }
-    }
-    l_run += lsum;
-
-    // ---- O^T += V^T P^T ---------------------------------------------------------
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-      if (!MASKED || need[sb]) {
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-          const int voff = buf * TILE + (32 * sb + 16 * m) * D;
-#pragma unroll
-          for (int dt = 0; dt < NDT; ++dt) {
-            const u32x2 a0 = lds_read_tr16(v_rd[dt] + voff);            // keys 16m + 4lh + 0..3
-            const u32x2 a1 = lds_read_tr16(v_rd[dt] + voff + 8 * D);    // keys 16m + 8 + 4lh + 0..3
-            const u32x4 av = {a0.x, a0.y, a1.x, a1.y};
-            oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), pfrag[sb][m], oacc[dt], 0, 0, 0);
-          }
-        }
-      }
-    }
-  };
-
-  using Buf0 = std::integral_constant<int, 0>;
-  using Buf1 = std::integral_constant<int, 1>;
-  issue_copies(t_lo, Buf0{});
-  finish_copies(t_lo, Buf0{});
-  __syncthreads();
-
-  // One iteration: start the copies of the next tile into the other buffer, compute on this
-  // buffer, then wait for the copies and meet the other wavefronts.
-  auto iteration = [&](int tile, auto buf_tag) {
-    constexpr int buf = decltype(buf_tag)::value;
-    using Other = std::integral_constant<int, buf ^ 1>;
-    if (tile < t_hi) issue_copies(tile + 1, Other{});
-    const int kv0 = tile * kBN;
-    if (wave_live && kv0 <= q_w_max && kv0 + kBN - 1 >= lo_w_min) {
-      const bool clean = kv0 + kBN - 1 <= q_w_min && kv0 >= lo_w_max;
-      if (clean) process_tile(buf_tag, kv0, std::false_type{});
-      else process_tile(buf_tag, kv0, std::true_type{});
-    }
-    if (tile < t_hi) finish_copies(tile + 1, Other{});
-    __syncthreads();
-  };
-  for (int tile = t_lo; tile <= t_hi; tile += 2) {
-    iteration(tile, Buf0{});
-    if (tile + 1 <= t_hi) iteration(tile + 1, Buf1{});
-  }
-
-  // ---- epilogue ---------------------------------------------------------------
-  const float l_tot = pair_sum(l_run);
-  const float inv = 1.f / l_tot;
-  if (qw0 + lq < p.T) {
-    uint16_t* op = p.o + b * p.o_sb + (int64_t)(qw0 + lq) * p.o_st + h * p.o_sh + 4 * lh;
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w.x = pack_bf16x2(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
-        w.y = pack_bf16x2(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
-        *reinterpret_cast<u32x2*>(op + 32 * dt + 8 * g) = w;
-      }
-    }
-  }
 }
 
 // Main kernel (keys already rotated, or no RoPE on keys).  32-key tiles, and nothing of a step is
@@ -901,13 +535,13 @@ __global__ __launch_bounds__(64) void prefill_scalar_kernel(PrefillParams p) {
 }
 
 template <int D>
-static int launch_mfma(PrefillParams p, bool rope_in_kernel, hipStream_t s) {
+static int launch_mfma(PrefillParams p, hipStream_t s) {
   const int64_t nwg = (int64_t)p.nqb * p.H * p.B;
   if (nwg > 0x7fffffff) {
     set_error("prefill: too many workgroups (%lld)", (long long)nwg);
     return DAISY_ERR_INVALID_ARGUMENT;
   }
-  if (p.cos != nullptr && !rope_in_kernel) {
+  if (p.cos != nullptr) {
     // Pre-pass: rotate K once into k_out, then attend over k_out.
     const int hpt = p.H % 2 == 0 ? 2 : 1;
     const int64_t total = (int64_t)p.B * p.T * (p.H / hpt) * (D / 16);
@@ -915,15 +549,9 @@ static int launch_mfma(PrefillParams p, bool rope_in_kernel, hipStream_t s) {
     else hipLaunchKernelGGL((rope_k_kernel<D, 1>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, p);
     DAISY_CHECK_LAUNCH("rope_k_kernel");
     p.k = p.k_out; p.k_sb = p.ko_sb; p.k_st = p.ko_st; p.k_sh = p.ko_sh;
-    hipLaunchKernelGGL((prefill_tile_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
-    DAISY_CHECK_LAUNCH("prefill_tile_kernel");
-  } else if (p.cos != nullptr) {
-    hipLaunchKernelGGL((prefill_mfma_kernel<D, true>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
-    DAISY_CHECK_LAUNCH("prefill_mfma_kernel");
-  } else {
-    hipLaunchKernelGGL((prefill_tile_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
-    DAISY_CHECK_LAUNCH("prefill_tile_kernel");
   }
+  hipLaunchKernelGGL((prefill_tile_kernel<D>), dim3((unsigned)nwg), dim3(kPrefillThreads), 0, s, p);
+  DAISY_CHECK_LAUNCH("prefill_tile_kernel");
   return DAISY_OK;
 }
 
@@ -974,6 +602,7 @@ extern "C" int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
                                      k_out, k_out_strides, B, T, H, D, window, scale);
   if (rc != DAISY_OK) return rc;
   hipStream_t s = (hipStream_t)stream;
+  DAISY_CHECK_ARG(flags == 0, "prefill: flags must be 0 (got %d)", flags);
 
   if (D == 64 || D == 128) {
     auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
@@ -984,8 +613,11 @@ extern "C" int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
                           (!k_out || k_out_strides[i] % 8 == 0),
                       "prefill: strides must be multiples of 8 elements");
     }
-    const bool rope_in_kernel = (flags & DAISY_PREFILL_ROTATE_K_IN_KERNEL) != 0 || k_out == nullptr;
-    return D == 128 ? launch_mfma<128>(p, rope_in_kernel, s) : launch_mfma<64>(p, rope_in_kernel, s);
+    // The keys are rotated once, into k_out, and attended from there: without that buffer every query
+    // block would have to rotate every key tile again (measured 3.7 times slower), so it is required.
+    DAISY_CHECK_ARG(cos == nullptr || k_out != nullptr,
+                    "prefill: cos/sin with head_dim %d need k_out (the rotated keys are written there and attended from there)", D);
+    return D == 128 ? launch_mfma<128>(p, s) : launch_mfma<64>(p, s);
   }
 
   DAISY_CHECK_ARG(B <= 65535 && H <= 65535, "prefill: B and H must each be <= 65535 for the scalar kernel");

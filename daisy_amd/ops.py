@@ -27,8 +27,7 @@ def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *,
                       window: Optional[int], scale: float = ATTN_SCALE,
                       cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
                       doc_start: Optional[torch.Tensor] = None,
-                      out: Optional[torch.Tensor] = None, k_out: Optional[torch.Tensor] = None,
-                      rotate_k_in_kernel: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+                      out: Optional[torch.Tensor] = None, k_out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """Sliding-window causal attention over ``[B, T, H, D]`` bf16 tensors.
 
     ``cos``/``sin`` (fp32 ``[>=T, D/2]``) rotate q and k inside the call;
@@ -68,7 +67,7 @@ def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *,
         if cos is None:
             raise ValueError("k_out is only produced when cos/sin are given")
     w = 0 if window is None else int(window)
-    flags = _lib.PREFILL_ROTATE_K_IN_KERNEL if rotate_k_in_kernel else 0
+    flags = 0
     lib = _lib.load()
     with _lib.on_device(dev):
         rc = lib.daisy_prefill_fwd(

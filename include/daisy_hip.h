@@ -67,18 +67,16 @@ int daisy_abi_version(void);
  *              128 queries from the block's first row; a bound that decreases
  *              inside a block silently drops keys, a bound beyond t gives NaN).
  *              Shared by all batches, like the reference's [1,1,T,T] mask.
- * k_out      : bf16 [B, T, H, D] with its own strides, or NULL.  When cos/sin
- *              are given, receives the rotated keys (what the reference's
- *              prefill returns for the KV cache, attention.py:179); the
- *              attention kernel then reads keys from k_out instead of rotating
- *              them again for every query block.
+ * k_out      : bf16 [B, T, H, D] with its own strides.  REQUIRED when cos/sin are
+ *              given and D is 64 or 128 (DAISY_ERR_INVALID_ARGUMENT otherwise):
+ *              a pre-pass writes the rotated keys there once (what the
+ *              reference's prefill returns for the KV cache, attention.py:179)
+ *              and the attention kernel reads them from there instead of
+ *              rotating every key tile again for every query block.  NULL
+ *              when cos/sin are NULL; optional for the scalar kernel.
  * window     : keys visible per query INCLUDING itself; <= 0 means full causal.
- * flags      : 0, or DAISY_PREFILL_ROTATE_K_IN_KERNEL to rotate the keys while
- *              they are staged into LDS instead of in a pre-pass (k_out, when
- *              given, is still written).  That is also what happens when
- *              cos/sin are given and k_out is NULL.
+ * flags      : reserved, must be 0.
  */
-#define DAISY_PREFILL_ROTATE_K_IN_KERNEL 1
 int daisy_prefill_fwd(const void* q, const int64_t* q_strides,
                       const void* k, const int64_t* k_strides,
                       const void* v, const int64_t* v_strides,
@@ -169,8 +167,16 @@ int daisy_decode_fwd_f32(const float* q, const int64_t* q_strides,
  * daisy_decode_workspace_bytes(B, H, D, n_rows, nsplit) exceeds that size.  All calls on one GPU
  * share the buffer: calls that overlap on one GPU (different streams) race and must be ordered by
  * the caller.  Same results as daisy_decode_fwd.
+ *
+ * The buffer's device address is looked up once per device, by daisy_decode_noalloc_init() or by the
+ * first call on that device.  The lookup is not done while `stream` is capturing: a caller that records
+ * the entry point into a HIP graph calls daisy_decode_noalloc_init() (or runs one call) on that device
+ * before the capture starts, else the call fails with DAISY_ERR_INVALID_ARGUMENT.
+ * daisy_decode_noalloc_init: set-up for the current device; launches nothing, allocates nothing, may be
+ * called any number of times.  No counterpart in the reference either.
  */
 #define DAISY_DECODE_STATIC_SCRATCH_BYTES (4u << 20)
+int daisy_decode_noalloc_init(void);
 int daisy_decode_fwd_noalloc(const void* q, const int64_t* q_strides,
                              const void* k_new, const int64_t* k_new_strides,
                              const void* v_new, const int64_t* v_new_strides,
@@ -267,8 +273,13 @@ int daisy_kda_chunk_fwd(const void* q, const void* k, const void* v,
  * (models/daisy/attention_kimi.py:133-134,150-154).  q, k, g: [T, H, Dk]; v, o: [T, H, Dv];
  * beta: [T, H]; cu_seqlens: int32 [n_seq + 1] in device memory, sequence i = rows
  * cu_seqlens[i] .. cu_seqlens[i+1] - 1, cu_seqlens[0] = 0, cu_seqlens[n_seq] = T, non-decreasing
- * (empty sequences allowed).  The bounds are read by the kernels, never by the host; bounds that
- * break the contract are forced into 0..T and rows that belong to no sequence are left unwritten.
+ * (empty sequences allowed).  The bounds are read by the kernels, never by the host.  Every packed-
+ * sequence kernel of this library (this one, daisy_kda_recurrent_varlen_fwd, daisy_short_conv_varlen_fwd)
+ * forces each bound into 0..T, so that no bound can lead outside the tensors; rows that belong to no
+ * sequence are left unwritten.  Bounds that DECREASE break the contract: every kernel stays inside the
+ * tensors, but how tokens are then assigned to sequences differs between the kernels (this one takes
+ * the running maximum of the bounds, the recurrent one clamps each pair, the convolution bisects over
+ * them as they are) -- the three kernels of one layer agree only on bounds that honour the contract.
  * initial_state / final_state: fp32 [n_seq, H, Dk, Dv].
  */
 size_t daisy_kda_varlen_workspace_bytes(int T, int n_seq, int H, int Dk, int Dv, int chunk);

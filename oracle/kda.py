@@ -55,7 +55,8 @@ def kda_recurrent(q, k, v, g, beta, scale: Optional[float] = None,
                   l2_eps: float = 1e-6, dtype=torch.float32):
     """Token-by-token recurrence; q, k, g ``[B, T, H, Dk]``, v ``[B, T, H, Dv]``,
     beta ``[B, T, H]``; returns ``o [B, T, H, Dv]`` and the final state
-    ``[B, H, Dk, Dv]`` (both in ``dtype``, fp32 by default, fp64 for pinning).
+    ``[B, H, Dk, Dv]`` (both in ``dtype``, fp32 by default, fp64 for pinning), on the inputs' device
+    (the same library calls either way; full-size checks run the loop on the GPU's fp32 units).
     """
     B, T, H, Dk = q.shape
     Dv = v.shape[-1]
@@ -66,8 +67,8 @@ def kda_recurrent(q, k, v, g, beta, scale: Optional[float] = None,
         qf = qf * torch.rsqrt(qf.pow(2).sum(-1, keepdim=True) + l2_eps)
         kf = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + l2_eps)
     vf, gf, bf = v.to(dtype), g.to(dtype), beta.to(dtype)
-    S = torch.zeros(B, H, Dk, Dv, dtype=dtype) if initial_state is None else initial_state.to(dtype).clone()
-    o = torch.empty(B, T, H, Dv, dtype=dtype)
+    S = torch.zeros(B, H, Dk, Dv, dtype=dtype, device=q.device) if initial_state is None else initial_state.to(dtype).clone()
+    o = torch.empty(B, T, H, Dv, dtype=dtype, device=q.device)
     for t in range(T):
         S = S * torch.exp(gf[:, t])[..., None]                      # decay rows of S
         pred = torch.einsum("bhkv,bhk->bhv", S, kf[:, t])            # S^T k_t

@@ -58,6 +58,15 @@ def test_prefill_argument_errors():
     assert rc == -1 and "cos and sin" in _err()
     rc = lib.daisy_prefill_fwd(p, s3, p, s3, p, s3, None, None, None, p, s3, None, None, 0, 8, 1, 64, 4, 0.12, 0, None)
     assert rc == -1 and "positive" in _err()
+    # Rotation tables without a buffer for the rotated keys: refused (head dims of the matrix-core kernel),
+    # as are flag bits (none is defined).
+    big = ctypes.create_string_buffer(4096)
+    a = (ctypes.addressof(big) + 15) & ~15
+    for D in (64, 128):
+        rc = lib.daisy_prefill_fwd(a, s3, a, s3, a, s3, a, a, None, a, s3, None, None, 1, 8, 1, D, 4, 0.12, 0, None)
+        assert rc == -1 and "k_out" in _err()
+    rc = lib.daisy_prefill_fwd(a, s3, a, s3, a, s3, None, None, None, a, s3, None, None, 1, 8, 1, 64, 4, 0.12, 1, None)
+    assert rc == -1 and "flags" in _err()
 
 
 def test_decode_argument_errors():

@@ -199,3 +199,38 @@ def test_config5_kda_full_size():
         rel = ((S[b, h].cpu() - S_ref[0, 0]).norm() / S_ref[0, 0].norm()).item()
         say(f"config 5 (b={b}, h={h}): o max-abs {mx:.2e} mean-abs {mn:.2e}, state rel err {rel:.2e}")
         assert rel <= 1e-3
+    _check_every_pair(q, k, v, gl, beta, o, S, "config 5")
+
+
+def _check_every_pair(q, k, v, gl, beta, o, S, what):
+    """Every (batch, head) pair, every token: the naive recurrence evaluated in fp32 on the same device tensors
+    (the oracle's loop, library fp32 einsums) against the kernel's outputs and final states."""
+    o_ref, S_ref = oracle.kda_recurrent(q, k, v, gl, beta)
+    err = (o.float() - o_ref).abs()
+    per_pair_max = err.amax(dim=(1, 3))                              # [B, H]
+    per_pair_mean = err.mean(dim=(1, 3))
+    rel = (S - S_ref).flatten(2).norm(dim=-1) / S_ref.flatten(2).norm(dim=-1)
+    say(f"{what}, all {rel.numel()} (batch, head) pairs: o max-abs {per_pair_max.max().item():.2e}, worst mean-abs "
+        f"{per_pair_mean.max().item():.2e}, worst state rel err {rel.max().item():.2e}")
+    assert per_pair_max.max().item() <= 2e-2 and per_pair_mean.max().item() <= 2e-3
+    assert rel.max().item() <= 1e-3
+
+
+def test_config5_kda_full_size_with_the_layer_gate():
+    """The configuration-5 shape with log-decays from the layer's own gate at its initial parameters
+    (A_log = log U(1, 16), dt_bias = 0, models/daisy/attention_kimi.py:95-99,132): decays of e^-1 .. e^-20 per token,
+    the steep path of the chunk kernel.  Every (batch, head) pair and token against the recurrence."""
+    B, T, H, Dk = 4, 8192, 16, 128
+    gd = torch.Generator(device=DEV).manual_seed(5)
+    rn = lambda *s: torch.randn(*s, generator=gd, device=DEV)
+    q = F.normalize(rn(B, T, H, Dk), dim=-1).bfloat16()
+    k = F.normalize(rn(B, T, H, Dk), dim=-1).bfloat16()
+    v = rn(B, T, H, Dk).bfloat16()
+    A_log = torch.log(torch.empty(H, device=DEV).uniform_(1, 16, generator=gd))
+    gl = oracle.kda_gate(rn(B, T, H * Dk), A_log, Dk)               # fp32 [B, T, H, Dk]
+    beta = torch.sigmoid(rn(B, T, H))
+    o, S = chunk_kda(q, k, v, gl, beta, scale=Dk ** -0.5, output_final_state=True, use_qk_l2norm_in_kernel=True)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(S).all()
+    say(f"gate log-decays: mean {gl.mean().item():.2f}, min {gl.min().item():.1f}")
+    _check_every_pair(q, k, v, gl, beta, o, S, "config 5 shape, layer gate")

@@ -54,12 +54,18 @@ class OneHotModel(nn.Module):
 V = 16
 
 
-@pytest.fixture()
-def env():
+DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
+
+
+@pytest.fixture(params=DEVICES)
+def env(request):
+    """(model, generator, device): the scenarios run on CPU tensors and, under the ``gpu`` mark, with model,
+    cache and prompts on ``cuda:0``, where the generator is used."""
     torch.manual_seed(0)
-    model = OneHotModel(V).eval()
-    gen = Generator(model, window=8, seed=1337, device=torch.device("cpu"), dtype=torch.bfloat16, temperature=0.0)
-    return model, gen
+    dev = torch.device(request.param)
+    model = OneHotModel(V).to(dev).eval()
+    gen = Generator(model, window=8, seed=1337, device=dev, dtype=torch.bfloat16, temperature=0.0)
+    return model, gen, dev
 
 
 def onehot(i):
@@ -68,50 +74,54 @@ def onehot(i):
     return v
 
 
+def eq(got, want):
+    return torch.equal(got.float().cpu(), want.float().cpu())
+
+
 def test_prefill_updates_cache_and_returns_logits(env):
-    model, gen = env
-    prompt = torch.tensor([3, 5, 7, 9])
+    model, gen, dev = env
+    prompt = torch.tensor([3, 5, 7, 9], device=dev)
     logits = gen._prefill(prompt)
-    assert logits.shape == (1, V) and torch.equal(logits[0].float(), onehot(9))
+    assert logits.shape == (1, V) and eq(logits[0], onehot(9))
     assert gen.cache.t == 4
     for layer in range(2):
         k, v = gen.cache.view(layer)
         assert k.shape == (1, 4, 1, V)
         for t, tok in enumerate(prompt.tolist()):
-            assert torch.equal(k[0, t, 0].float(), onehot(tok)) and torch.equal(v[0, t, 0].float(), onehot(tok))
-    assert torch.equal(gen.history, prompt)
+            assert eq(k[0, t, 0], onehot(tok)) and eq(v[0, t, 0], onehot(tok))
+    assert torch.equal(gen.history, prompt) and gen.cache.k.device == dev and logits.device == dev
     assert gen.use_ring_context is False   # a foreign model gets chronological tensors
 
 
 def test_step_writes_kv_and_advances_cache(env):
-    model, gen = env
-    gen._prefill(torch.tensor([2, 4, 6]))
+    model, gen, dev = env
+    gen._prefill(torch.tensor([2, 4, 6], device=dev))
     t0 = gen.cache.t
-    logits = gen._step(torch.tensor(11))
-    assert torch.equal(logits[0].float(), onehot(11))
+    logits = gen._step(torch.tensor(11, device=dev))
+    assert eq(logits[0], onehot(11))
     assert gen.cache.t == t0 + 1
     for layer in range(2):
         k, v = gen.cache.view(layer)
-        assert torch.equal(k[0, -1, 0].float(), onehot(11)) and torch.equal(v[0, -1, 0].float(), onehot(11))
+        assert eq(k[0, -1, 0], onehot(11)) and eq(v[0, -1, 0], onehot(11))
         # the model saw the cache as it was BEFORE this token's row was written
-        assert torch.equal(model.seen_k[layer].float(), k[:, :-1].float())
-        assert torch.equal(model.seen_v[layer].float(), v[:, :-1].float())
+        assert eq(model.seen_k[layer], k[:, :-1])
+        assert eq(model.seen_v[layer], v[:, :-1])
     assert gen.history[-1].item() == 11
 
 
 def test_window_limits_what_prefill_stores(env):
-    model, gen = env
-    prompt = torch.arange(12) % V
+    model, gen, dev = env
+    prompt = torch.arange(12, device=dev) % V
     gen._prefill(prompt)
     k, _ = gen.cache.view(0)          # W = 8: a view shows 8 rows, bulk write stored the last W - 1 = 7
     assert k.shape[1] == 8
     for j, tok in enumerate(prompt[-7:].tolist()):
-        assert torch.equal(k[0, 1 + j, 0].float(), onehot(tok))
+        assert eq(k[0, 1 + j, 0], onehot(tok))
 
 
 def test_generate_end_to_end(env):
-    model, gen = env
-    prompt = torch.tensor([4, 1, 4])
+    model, gen, dev = env
+    prompt = torch.tensor([4, 1, 4], device=dev)
     assert [int(t) for t in gen.generate(prompt, max_new_tokens=3)] == [4, 4, 4]
     g = gen.generate(prompt, max_new_tokens=2)
     toks = []

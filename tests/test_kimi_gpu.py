@@ -301,3 +301,41 @@ def test_packed_bounds_that_break_the_contract_stay_inside_the_tensors():
     o2, S2 = chunk_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), output_final_state=True, use_qk_l2norm_in_kernel=True,
                        cu_seqlens=good.to(DEV))
     assert torch.equal(o, o2) and torch.equal(S, S2) and bool(torch.isfinite(o.float()).all())
+
+
+def test_bounds_outside_the_token_range_are_clamped_the_same_way_by_every_packed_kernel():
+    """Every packed-sequence kernel forces each bound into 0..T (the one rule they share): bounds that are ordered
+    but reach outside the token range give exactly what the clamped bounds give -- in the chunked and the
+    token-by-token delta rule and in the short convolution.  Bounds that are out of order break the contract; each
+    kernel then stays inside the tensors and leaves finite states, but which tokens it assigns to which sequence is
+    left open (the header says so)."""
+    from daisy_amd import chunk_kda, fused_recurrent_kda, ops
+    T, C, K = 150, 64, 4
+    q, k, v, gl, beta, _ = _kda_pack([T], seed=8)
+    dev = lambda t: t.to(DEV)
+    wide = torch.tensor([-7, 5, 90, 10 ** 6], dtype=torch.int32).to(DEV)
+    clamped = torch.tensor([0, 5, 90, T], dtype=torch.int32).to(DEV)
+    broken = torch.tensor([5, -3, 90, 40, 10 ** 6], dtype=torch.int32).to(DEV)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1, T, C, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(C, K, generator=g) * 0.5).bfloat16().to(DEV)
+    win = torch.randn(3, C, K, generator=g).bfloat16().to(DEV)
+
+    def run_all(cu, n):
+        out = {}
+        out["chunk"] = chunk_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), output_final_state=True,
+                                 use_qk_l2norm_in_kernel=True, cu_seqlens=cu)
+        out["recurrent"] = fused_recurrent_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), output_final_state=True,
+                                               use_qk_l2norm_in_kernel=True, cu_seqlens=cu)
+        cache = win if n == 3 else torch.zeros(n, C, K, dtype=torch.bfloat16, device=DEV)
+        out["conv"] = ops.short_conv(x, w, cache=cache, output_final_state=True, cu_seqlens=cu)
+        torch.cuda.synchronize()
+        return out
+
+    a, b = run_all(wide, 3), run_all(clamped, 3)
+    for name in a:
+        assert torch.equal(a[name][0], b[name][0]), f"{name}: outputs differ between wide and clamped bounds"
+        assert torch.equal(a[name][1], b[name][1]), f"{name}: states / windows differ between wide and clamped bounds"
+    c = run_all(broken, 4)
+    for name, (y, st) in c.items():      # (rows that end up in no sequence are left unwritten, so only the states are looked at)
+        assert bool(torch.isfinite(st.float()).all()), f"{name}: state with out-of-order bounds"

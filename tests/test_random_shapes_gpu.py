@@ -25,9 +25,10 @@ def test_prefill_random_shapes(seed):
         T = rng.choice([1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 191, 255, 256, 257, 300, 383, 385, 511, 513, 640])
         window = rng.choice([None, 1, 2, 16, 17, 64, 100, 127, 128, 129, 200, 256, 300, 512, 1000])
         rope, docs, strided = rng.random() < 0.6, rng.random() < 0.5, rng.random() < 0.4
-        rotate_in_kernel = rope and rng.random() < 0.3
+        if rope:
+            rng.random()   # one draw more for rotated cases (keeps the case sequence of this seed unchanged)
         say(f"prefill sweep seed {seed} case {it}: B{B} H{H} D{D} T{T} window {window} rope {rope} docs {docs} "
-            f"strided {strided} rotate_in_kernel {rotate_in_kernel}")
+            f"strided {strided}")
         g = torch.Generator().manual_seed(seed * 100003 + it)
         if strided:   # three views of one [B, T, 3H, D] tensor, the layout of the QKV projection output
             qkv = torch.randn(B, T, 3 * H, D, generator=g).bfloat16()
@@ -50,8 +51,7 @@ def test_prefill_random_shapes(seed):
                                         doc_start).transpose(1, 2)
         o, k_rot = ops.prefill_attention(qd, kd, vd, window=window, scale=SCALE,
                                          cos=None if cos is None else cos.cuda(), sin=None if sin is None else sin.cuda(),
-                                         doc_start=None if doc_start is None else doc_start.cuda(),
-                                         rotate_k_in_kernel=rotate_in_kernel)
+                                         doc_start=None if doc_start is None else doc_start.cuda())
         assert_close_bf16(o, ref, f"o (case {it})")
         if rope:
             assert_close_bf16(k_rot, kr, f"rotated keys (case {it})")

@@ -40,10 +40,17 @@ def _case(B, H, D, W, n_rows, new_idx, nsplit, seed):
     o2 = torch.zeros_like(o1)
     rc = _call("workspace", q, kn, vn, kc1, vc1, o1, n_rows, new_idx, nsplit, ws)
     assert rc == 0, lib.daisy_last_error()
+    assert lib.daisy_decode_noalloc_init() == 0, lib.daisy_last_error()
+    torch.cuda.synchronize()
+    # Free device memory as the HIP runtime reports it (hipMemGetInfo), not torch's allocator statistics: an
+    # allocation made by the library itself would show here.
+    free_before, _ = torch.cuda.mem_get_info(DEV)
     before = torch.cuda.memory_allocated(DEV)
     rc = _call("noalloc", q, kn, vn, kc2, vc2, o2, n_rows, new_idx, nsplit)
     assert rc == 0, lib.daisy_last_error()
     torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(DEV)
+    assert free_after >= free_before, f"free device memory fell by {free_before - free_after} bytes during the call"
     assert torch.cuda.memory_allocated(DEV) == before
     assert torch.isfinite(o2.float()).all()
     assert torch.equal(o1, o2), f"outputs differ: {(o1.float() - o2.float()).abs().max().item()}"
@@ -57,6 +64,38 @@ def test_no_alloc_decode_equals_the_workspace_entry_point_twice_in_a_row():
     _case(B=1, H=2, D=64, W=1024, n_rows=700, new_idx=699, nsplit=2, seed=2)
     print("no-alloc decode: the split count chosen by the library", flush=True)
     _case(B=3, H=8, D=128, W=2048, n_rows=2048, new_idx=0, nsplit=0, seed=3)
+
+
+def test_no_alloc_decode_recorded_into_a_graph():
+    """The entry point under HIP graph capture (one of the callers it exists for): set up outside the capture,
+    recorded once, replayed with new inputs and with eager work and synchronisations between the replays; every
+    replay equals daisy_decode_fwd on the same inputs bit for bit."""
+    lib = _lib.load()
+    B, H, D, W, nsplit = 2, 4, 128, 2048, 4
+    g = torch.Generator(device=DEV).manual_seed(9)
+    rn = lambda *s: torch.randn(*s, generator=g, device=DEV).bfloat16()
+    q, kn, vn = rn(B, H, D), rn(B, H, D), rn(B, H, D)
+    kc, vc = rn(B, H, W, D), rn(B, H, W, D)
+    o = torch.zeros(B, H, D, dtype=torch.bfloat16, device=DEV)
+    assert lib.daisy_decode_noalloc_init() == 0, lib.daisy_last_error()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = _call("noalloc", q, kn, vn, kc, vc, o, W, 5, nsplit)
+    assert rc == 0, lib.daisy_last_error()
+    need = int(lib.daisy_decode_workspace_bytes(B, H, D, W, nsplit))
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    for it in range(4):
+        print(f"no-alloc decode in a graph: replay {it}", flush=True)
+        q.copy_(rn(B, H, D)); kn.copy_(rn(B, H, D)); vn.copy_(rn(B, H, D))      # eager work between the replays
+        kc_ref, vc_ref = kc.clone(), vc.clone()
+        o_ref = torch.zeros_like(o)
+        assert _call("workspace", q, kn, vn, kc_ref, vc_ref, o_ref, W, 5, nsplit, ws) == 0
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_ref), f"replay {it}: outputs differ by {(o.float() - o_ref.float()).abs().max().item()}"
+        assert torch.equal(kc, kc_ref) and torch.equal(vc, vc_ref), f"replay {it}: the appended rows differ"
 
 
 def test_no_alloc_decode_refuses_sizes_beyond_its_buffer():

@@ -286,9 +286,10 @@ class Rotary(nn.Module):
                 if name == "inv_freq":
                     fresh = self._inv_freq_fp32.to(dev)
                 else:
-                    theta = torch.outer(torch.arange(self._max_seq_len, dtype=torch.float32, device=dev),
-                                        self._inv_freq_fp32.to(dev))
-                    fresh = theta.cos() if name == "cos" else theta.sin()
+                    # rebuilt where the constructor built them, on the CPU: the GPU's cos / sin differ from the
+                    # CPU's in the last bit, and the tables are to stay what the reference's constructor computes
+                    theta = torch.outer(torch.arange(self._max_seq_len, dtype=torch.float32), self._inv_freq_fp32.cpu())
+                    fresh = (theta.cos() if name == "cos" else theta.sin()).to(dev)
                 setattr(self, name, nn.Buffer(fresh, persistent=False))
         return self
 

@@ -337,5 +337,7 @@ def test_bounds_outside_the_token_range_are_clamped_the_same_way_by_every_packed
         assert torch.equal(a[name][0], b[name][0]), f"{name}: outputs differ between wide and clamped bounds"
         assert torch.equal(a[name][1], b[name][1]), f"{name}: states / windows differ between wide and clamped bounds"
     c = run_all(broken, 4)
-    for name, (y, st) in c.items():      # (rows that end up in no sequence are left unwritten, so only the states are looked at)
-        assert bool(torch.isfinite(st.float()).all()), f"{name}: state with out-of-order bounds"
+    # Rows (and convolution windows) that end up in no sequence are left unwritten, so only the delta-rule states are
+    # looked at; for the convolution the point is that the launch completes (run_all synchronises).
+    for name in ("chunk", "recurrent"):
+        assert bool(torch.isfinite(c[name][1].float()).all()), f"{name}: state with out-of-order bounds"

@@ -34,8 +34,11 @@ def _structured(B, T, H, D, rise_per_32_keys, seed, noise=0.3):
 
 
 def _random_large(B, T, H, D, seed):
+    """q, k ~ 3 N(0,1) (scores hundreds of log2 units apart), v ~ N(0,1) (outputs of a size at which the rounding of
+    the bf16 result itself stays well inside the tolerance)."""
     g = torch.Generator().manual_seed(seed)
-    return tuple((3.0 * torch.randn(B, T, H, D, generator=g)).bfloat16() for _ in range(3))
+    q, k = ((3.0 * torch.randn(B, T, H, D, generator=g)).bfloat16() for _ in range(2))
+    return q, k, torch.randn(B, T, H, D, generator=g).bfloat16()
 
 
 @pytest.mark.parametrize("D", [64, 128])

@@ -95,6 +95,9 @@ def probe_lib():
         lib.daisy_probe_matrix_rate.restype = ctypes.c_int
         lib.daisy_probe_matrix_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
                                                 ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
+        lib.daisy_probe_matrix_rate_data.restype = ctypes.c_int
+        lib.daisy_probe_matrix_rate_data.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                                     ctypes.c_void_p, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
         lib.daisy_probe_read_rate.restype = ctypes.c_int
         lib.daisy_probe_read_rate.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
         _probe_lib = lib
@@ -123,6 +126,35 @@ def probe_matrix_rate(with_vector_mix, iters=50000, workgroups=256, device="cuda
     ms = start.elapsed_time(end)
     t = ticks.view(workgroups, 2).double().sum(0)
     return {"ms": ms, "tflops": flop.value / ms / 1e9, "clock_mhz": float(t[0] / t[1] * 100.0)}
+
+
+def probe_matrix_rate_data(kind, seconds=1.0, iters=80000, workgroups=256, device="cuda:0"):
+    """Sustained rate of register-only bf16 MFMAs whose operands change with every instruction and hold `kind` data
+    ("zeros" or "normal": N(0,1) rounded to bf16), launches back to back for `seconds`; the rate and clock of the last
+    quarter of the run.  The instruction stream is the same for both kinds: the difference is what the chip's power
+    management takes for the toggling of the operand bits."""
+    import ctypes
+    dev = torch.device(device)
+    n_el = 16 * 512 * 8
+    data = (torch.zeros(n_el, device=dev) if kind == "zeros"
+            else torch.randn(n_el, device=dev, generator=torch.Generator(device=dev).manual_seed(0))).bfloat16()
+    sink = torch.empty(4096, dtype=torch.float32, device=dev)
+    ticks = torch.zeros(2 * workgroups, dtype=torch.int64, device=dev)
+    lib = probe_lib()
+    flop = ctypes.c_double(0.0)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def run():
+        rc = lib.daisy_probe_matrix_rate_data(data.data_ptr(), n_el * 2, 0, workgroups, iters, sink.data_ptr(), ticks.data_ptr(),
+                                              ctypes.byref(flop), stream)
+        assert rc == 0, rc
+
+    ms_one = time_gpu(run, 2, 1)
+    n = max(int(seconds * 1e3 / ms_one), 4)
+    time_gpu(run, 3 * n // 4, 0)
+    ms = time_gpu(run, n - 3 * n // 4, 0)
+    t = ticks.view(workgroups, 2).double().sum(0)
+    return {"tflops": flop.value / ms / 1e9, "clock_mhz": float(t[0] / t[1] * 100.0), "seconds": n * ms_one / 1e3, "operands": kind}
 
 
 def probe_read_rate(gib=2, workgroups=8192, repeats=5, device="cuda:0"):
@@ -358,6 +390,13 @@ def bench_prefill_c3(steps, warmup):
         fl = prefill_flops(B, T, H, D, W)
         out[name] = {"ms": ms, "ms_first_steps_from_idle": ms_first, "flops": fl, "tflops": fl / ms / 1e9,
                      "frac_of_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS}
+    # The same launch on tensors of zeros: the same instructions, addresses and memory traffic, but operand bits that
+    # never toggle.  Timing only (the result is meaningless); what it shows is how much of the rate on N(0,1) data the
+    # chip's power management takes away (see extra.matrix_pipe_ceiling.mfma_only_*_operands for the matrix pipe alone).
+    q.zero_(); k.zero_(); v.zero_()
+    ms, _ = time_settled(lambda: ops.prefill_attention(q, k, v, window=None, scale=SCALE, out=o), max(steps // 4, 2), 1)
+    fl = prefill_flops(B, T, H, D, None)
+    out["full_causal_on_zero_tensors_timing_only"] = {"ms": ms, "tflops": fl / ms / 1e9, "frac_of_peak": fl / ms / 1e9 / PEAK_BF16_TFLOPS}
     return out
 
 
@@ -719,6 +758,11 @@ def main():
         extra["matrix_pipe_ceiling"] = {
             "what": "register-only v_mfma_f32_32x32x16_bf16 on every SIMD, 2 wavefronts each, ~25 ms per run",
             "mfma_only": probe_matrix_rate(False, 80000),
+            "mfma_only_zero_operands": probe_matrix_rate_data("zeros"),
+            "mfma_only_normal_operands": dict(
+                probe_matrix_rate_data("normal"),
+                what="the same instruction stream on N(0,1) bf16 operands: the sustained rate of the matrix pipe ALONE on data like "
+                     "the benchmark's; the power management lowers the clock until the chip stays inside its power limit"),
             "mfma_with_attention_vector_mix": probe_matrix_rate(True, 60000),
             "mfma_with_attention_mix_and_lds_operands": dict(
                 probe_matrix_rate(2, 50000),

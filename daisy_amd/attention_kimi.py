@@ -98,7 +98,16 @@ class KimiLinearSelfAttention(nn.Module):
         super().__init__()
         self.hidden_size, self.num_heads, self.head_dim = dim, num_heads, head_dim
         self.head_k_dim, self.head_v_dim = head_dim, int(head_dim * expand_v)
-        torch._assert(self.head_k_dim == 128 and self.head_v_dim == 128, "the KDA kernels need head_dim 128 and expand_v 1")
+        # What the kernels under this layer serve, checked here rather than at the first call: key heads of up to
+        # 128 channels (a multiple of 8), value heads of 32, 64, 128 or 256 columns (the delta-rule kernels take any
+        # multiple of 8; the gated norm takes these four), convolutions of 2 to 4 taps, bf16 parameters (this
+        # constructor makes them so).
+        if not (8 <= self.head_k_dim <= 128 and self.head_k_dim % 8 == 0):
+            raise ValueError(f"KimiLinearSelfAttention: head_dim {head_dim} not supported by the KDA kernels (a multiple of 8 up to 128)")
+        if self.head_v_dim not in (32, 64, 128, 256):
+            raise ValueError(f"KimiLinearSelfAttention: head_dim * expand_v = {self.head_v_dim} not supported (32, 64, 128 or 256)")
+        if use_short_conv and not 2 <= conv_size <= 4:
+            raise ValueError(f"KimiLinearSelfAttention: conv_size {conv_size} not supported by the convolution kernel (2 to 4)")
         self.key_dim, self.value_dim = num_heads * self.head_k_dim, num_heads * self.head_v_dim
         self.use_short_conv, self.conv_size, self.layer_idx = use_short_conv, conv_size, layer_idx
         bf = torch.bfloat16

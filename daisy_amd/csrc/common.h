@@ -101,6 +101,7 @@ __device__ __forceinline__ float group_sum(float x) {
   x = dpp_add<0x4E>(x);                     // quad_perm [2,3,0,1]   (xor 2)
   if (LPR >= 8) x = dpp_add<0x141>(x);      // row_half_mirror       (joins the two quads of 8 lanes)
   if (LPR >= 16) x = dpp_add<0x128>(x);     // row_ror 8             (joins the two halves of 16 lanes)
+  if (LPR >= 32) x += __shfl_xor(x, 16);    // the neighbouring row of 16 lanes
   return x;
 }
 

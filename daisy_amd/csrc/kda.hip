@@ -65,7 +65,11 @@ __global__ __launch_bounds__(256) void kda_gate_kernel(const void* g, const floa
 
 
 // ===========================================================================
-// Chunked forward.  Per (batch, head), chunk of C = 64 positions, Dk = Dv = 128.
+// Chunked forward.  Per (batch, head), chunk of C = 64 positions.  The kernels work on 128 key
+// channels and 128 value columns; a smaller Dk (a multiple of 8) is served by reading the missing
+// channels as zeros (zero channels of q, k and g change nothing: they add nothing to any dot product
+// or norm, and their state rows stay zero), and value columns are independent of each other, so any
+// Dv (a multiple of 8) is served in passes of up to 128 columns, a short last pass reading zeros.
 //
 // With G_i the inclusive running sum of the log-decay g inside the chunk (per
 // channel), S0 the state at the chunk start, and (per channel products written
@@ -116,6 +120,8 @@ struct KdaParams {
   const void* g; int g_bf16; const float* beta;
   const float* s0; uint16_t* o; float* s_out;
   int B, T, H, NC; float scale; int l2norm; float l2eps;
+  int Dk, Dv;     // the tensors' own widths: Dk <= 128 key channels, Dv value columns
+  int v0, nv;     // this pass covers value columns v0 .. v0 + nv - 1 (nv <= 128)
   uint16_t* Wn; uint16_t* Qg; uint16_t* Pm; uint16_t* KtH; uint16_t* KtL; float* U0T; float* dec;
   // Sequences packed along the token axis of a batch of one (B == 1, T = all tokens): n_seq > 0,
   // bounds [n_seq + 1] = sanitised running lengths, seq_chunk0 [n_seq + 1] = first chunk slot of
@@ -226,11 +232,12 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   // the chunk's slot in the workspace) plus a 32-bit offset per lane.  Written out once here: as one
   // 64-bit expression per access the row products were rebuilt per lane and load (seven vector
   // instructions each, three of them at a quarter of the rate).
-  const uint32_t row_stride = (uint32_t)p.H * KD;                 // elements between token rows of one head
-  const int64_t tok_base = ((int64_t)t0 * p.H + h) * KD;          // first element of the chunk's first row
+  const uint32_t row_stride = (uint32_t)p.H * (uint32_t)p.Dk;     // elements between token rows of one head (q, k, g)
+  const uint32_t row_stride_v = (uint32_t)p.H * (uint32_t)p.Dv;   //   ... of v
+  const int64_t tok_base = ((int64_t)t0 * p.H + h) * p.Dk;        // first element of the chunk's first row
   const uint16_t* const q_c = p.q + tok_base;
   const uint16_t* const k_c = p.k + tok_base;
-  const uint16_t* const v_c = p.v + tok_base;
+  const uint16_t* const v_c = p.v + ((int64_t)t0 * p.H + h) * p.Dv + p.v0;
   const float* const beta_c = p.beta + ((int64_t)t0 * p.H + h);
   uint16_t* const qg_c = p.Qg + ci * KC * KD;
   uint16_t* const pm_c = p.Pm + ci * KC * KC;
@@ -247,6 +254,8 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
   float btv[4];
   {
     const int d = tid & 127, half = __builtin_amdgcn_readfirstlane(tid >> 7);   // the row of a g load is wavefront-uniform
+    const bool d_live = d < p.Dk;                 // channels beyond Dk read as zero (their loads re-read the last channel)
+    const int dl = min(d, p.Dk - 1);
     float gv[32];
     // Rows past the end re-read the last row (always valid) and are zeroed afterwards, so that
     // the loads carry no branches and all go out together; the dtype is decided once, outside
@@ -257,28 +266,29 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
 #pragma unroll
       for (int i = 0; i < 32; ++i) {
         const uint32_t* row = reinterpret_cast<const uint32_t*>(p.g) + ((tok_base + (uint32_t)min(32 * half + i, n_live - 1) * row_stride) >> 1);
-        graw[i] = __builtin_nontemporal_load(row + (uint32_t)(d >> 1));
+        graw[i] = __builtin_nontemporal_load(row + (uint32_t)(dl >> 1));
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 32; ++i) {
         const uint32_t* row = reinterpret_cast<const uint32_t*>(p.g) + (tok_base + (uint32_t)min(32 * half + i, n_live - 1) * row_stride);
-        graw[i] = __builtin_nontemporal_load(row + (uint32_t)d);
+        graw[i] = __builtin_nontemporal_load(row + (uint32_t)dl);
       }
     }
     const bool g16 = p.g_bf16 != 0, odd = (d & 1) != 0;
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       const float x = g16 ? (odd ? bf16hi_to_f32(graw[i]) : bf16lo_to_f32(graw[i])) : __uint_as_float(graw[i]);
-      gv[i] = (32 * half + i < n_live) ? x : 0.f;
+      gv[i] = (32 * half + i < n_live && d_live) ? x : 0.f;
     }
+    const int ccl = min(cc, p.Dk / 8 - 1), ccv = min(cc, p.nv / 8 - 1);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = r4 + 16 * i;
       const int rc = min(r, n_live - 1);
-      const uint32_t off = (uint32_t)rc * row_stride + 8u * cc;
+      const uint32_t off = (uint32_t)rc * row_stride + 8u * ccl;
       kraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(k_c + off));
-      vraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(v_c + off));
+      vraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(v_c + (uint32_t)rc * row_stride_v + 8u * ccv));
       qraw[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q_c + off));
       btv[i] = beta_c[(uint32_t)rc * (uint32_t)p.H];
     }
@@ -320,7 +330,8 @@ __global__ __launch_bounds__(256, 2) void kda_prep_kernel(KdaParams p) {
     const int r = r4 + 16 * i;
     const bool live = r < n_live;
     const u32x4 zero4 = {0, 0, 0, 0};
-    if (!live) { kraw[i] = zero4; vraw[i] = zero4; qraw[i] = zero4; }
+    if (!live || 8 * cc >= p.Dk) { kraw[i] = zero4; qraw[i] = zero4; }
+    if (!live || 8 * cc >= p.nv) vraw[i] = zero4;
     float kf[8], qf[8];
     unpack8(kraw[i], kf);
     unpack8(qraw[i], qf);
@@ -847,7 +858,7 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
   // Keep the column groups of one (batch, head) on one XCD: they read the same chunk data.
   int vid = blockIdx.x;
   if ((gridDim.x & 7) == 0) vid = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-  constexpr int NGRP = KD / (KVS * KCT);
+  const int NGRP = (p.nv + KVS * KCT - 1) / (KVS * KCT);   // groups of 32 value columns in this pass
   const int grp = vid % NGRP, bh = vid / NGRP;
   const int h = bh % p.H, b = bh / p.H;     // b: batch element, or sequence of a packed batch
   const SeqSpan sp = seq_span(p, b);
@@ -910,8 +921,8 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
         const int idx = 64 * k + lane, row = idx >> 2, piece = idx & 3;
         const u32x4 v = *reinterpret_cast<const u32x4*>(&ost[n & 1][row][8 * piece]);
         const int tok = sp.tok0 + n * KC + row;
-        if (tok < sp.tok_end)
-          *reinterpret_cast<u32x4*>(p.o + ((int64_t)tok * p.H + h) * KD + KVS * KCT * grp + 8 * piece) = v;
+        if (tok < sp.tok_end && KVS * KCT * grp + 8 * piece < p.nv)
+          *reinterpret_cast<u32x4*>(p.o + ((int64_t)tok * p.H + h) * p.Dv + p.v0 + KVS * KCT * grp + 8 * piece) = v;
       }
     };
     if (nc > 0) issue_copies(0, 0);
@@ -954,13 +965,17 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
   for (int m = 0; m < 2; ++m) rd128[m] = ln * 128 + 16 * ((4 * m + q4) ^ ((ln >> 1) & 7));
   lds_cptr stage0 = (lds_cptr)&stage[0][0];
 
-  // State tile i: rows (key channels) 16*(4 hf + i) + 4*q4 + r, column vcol.
+  // State tile i: rows (key channels) 16*(4 hf + i) + 4*q4 + r, column vcol of this pass; rows beyond Dk and
+  // columns beyond Dv do not exist in the caller's [Dk, Dv] state: they are zero and stay zero.
+  const bool col_live = vcol < p.nv;
   f32x4 S[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      S[i][r] = p.s0 ? p.s0[((int64_t)bh * KD + 16 * (4 * hf + i) + 4 * q4 + r) * KD + vcol] : 0.f;
+    for (int r = 0; r < 4; ++r) {
+      const int row = 16 * (4 * hf + i) + 4 * q4 + r;
+      S[i][r] = (p.s0 && col_live && row < p.Dk) ? p.s0[((int64_t)bh * p.Dk + row) * p.Dv + p.v0 + vcol] : 0.f;
+    }
   }
 
   // What depends on the value column comes straight from global memory, one chunk ahead: U0
@@ -1097,11 +1112,14 @@ __global__ __launch_bounds__(64 * (KSW + KPW), 1) void kda_state_kernel(KdaParam
     chunk_step(n, std::integral_constant<int, 0>{});
     if (n + 1 < nc) chunk_step(n + 1, std::integral_constant<int, 1>{});
   }
-  if (p.s_out != nullptr) {
+  if (p.s_out != nullptr && col_live) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) p.s_out[((int64_t)bh * KD + 16 * (4 * hf + i) + 4 * q4 + r) * KD + vcol] = S[i][r];
+      for (int r = 0; r < 4; ++r) {
+        const int row = 16 * (4 * hf + i) + 4 * q4 + r;
+        if (row < p.Dk) p.s_out[((int64_t)bh * p.Dk + row) * p.Dv + p.v0 + vcol] = S[i][r];
+      }
   }
 }
 
@@ -1142,13 +1160,16 @@ static size_t kda_table_bytes(int T, int n_seq) {
   return (ints * sizeof(int32_t) + 255) & ~(size_t)255;
 }
 
+// Head widths the kernels serve: Dk a multiple of 8 up to 128, Dv any multiple of 8.
+static bool kda_dims_ok(int Dk, int Dv) { return Dk >= 8 && Dk <= KD && Dk % 8 == 0 && Dv >= 8 && Dv % 8 == 0; }
+
 extern "C" size_t daisy_kda_workspace_bytes(int B, int T, int H, int Dk, int Dv, int chunk) {
-  if (B <= 0 || T <= 0 || H <= 0 || Dk != KD || Dv != KD || chunk != KC) return 0;
+  if (B <= 0 || T <= 0 || H <= 0 || !kda_dims_ok(Dk, Dv) || chunk != KC) return 0;
   return kda_chunk_slots(B, T, 0) * H * kChunkBytes;
 }
 
 extern "C" size_t daisy_kda_varlen_workspace_bytes(int T, int n_seq, int H, int Dk, int Dv, int chunk) {
-  if (T <= 0 || n_seq <= 0 || H <= 0 || Dk != KD || Dv != KD || chunk != KC) return 0;
+  if (T <= 0 || n_seq <= 0 || H <= 0 || !kda_dims_ok(Dk, Dv) || chunk != KC) return 0;
   return kda_chunk_slots(1, T, n_seq) * H * kChunkBytes + kda_table_bytes(T, n_seq);
 }
 
@@ -1160,7 +1181,7 @@ static int kda_chunk_launch(const void* q, const void* k, const void* v,
                             int B, int T, int H, int Dk, int Dv, int chunk,
                             float scale, int l2norm_qk, float l2_eps,
                             void* workspace, size_t workspace_bytes, void* stream) {
-  DAISY_CHECK_SUPPORTED(Dk == KD && Dv == KD, "kda: Dk=%d, Dv=%d not supported (both must be %d)", Dk, Dv, KD);
+  DAISY_CHECK_SUPPORTED(kda_dims_ok(Dk, Dv), "kda: Dk=%d, Dv=%d not supported (Dk: a multiple of 8 up to %d; Dv: a multiple of 8)", Dk, Dv, KD);
   DAISY_CHECK_SUPPORTED(chunk == KC, "kda: chunk=%d not supported (must be %d)", chunk, KC);
   DAISY_CHECK_ARG(q && k && v && g && beta && o, "kda: q, k, v, g, beta and o must be non-NULL");
   DAISY_CHECK_ARG(B > 0 && T > 0 && H > 0, "kda: B=%d, T=%d, H=%d must be positive", B, T, H);
@@ -1204,10 +1225,17 @@ static int kda_chunk_launch(const void* q, const void* k, const void* v,
     p.bounds = bounds; p.seq_chunk0 = seq_chunk0; p.chunk_seq = chunk_seq;
   }
   const int n_streams = n_seq > 0 ? n_seq : B;    // independent recurrences per head
-  hipLaunchKernelGGL(kda_prep_kernel, dim3(p.NC, H, n_seq > 0 ? 1 : B), dim3(256), 0, s, p);
-  DAISY_CHECK_LAUNCH("kda_prep_kernel");
-  hipLaunchKernelGGL(kda_state_kernel, dim3((unsigned)(n_streams * H * (KD / (KVS * KCT)))), dim3(64 * (KSW + KPW)), 0, s, p);
-  DAISY_CHECK_LAUNCH("kda_state_kernel");
+  p.Dk = Dk; p.Dv = Dv;
+  // Value columns are independent: passes of up to 128 columns, each through the same workspace (the
+  // launches of one stream run in order).
+  for (int v0 = 0; v0 < Dv; v0 += KD) {
+    p.v0 = v0; p.nv = Dv - v0 < KD ? Dv - v0 : KD;
+    const int groups = (p.nv + KVS * KCT - 1) / (KVS * KCT);
+    hipLaunchKernelGGL(kda_prep_kernel, dim3(p.NC, H, n_seq > 0 ? 1 : B), dim3(256), 0, s, p);
+    DAISY_CHECK_LAUNCH("kda_prep_kernel");
+    hipLaunchKernelGGL(kda_state_kernel, dim3((unsigned)(n_streams * H * groups)), dim3(64 * (KSW + KPW)), 0, s, p);
+    DAISY_CHECK_LAUNCH("kda_state_kernel");
+  }
   return DAISY_OK;
 }
 

@@ -7,7 +7,9 @@
 // not support; a generation loop calls it with T = 1 per step.  At T = 1 the call is bound by
 // HBM: it reads and writes the [Dk, Dv] fp32 state of every (batch, head) once (128 KiB each).
 //
-// Workgroup = one (batch, head), 4 wavefronts; wavefront w owns value columns [32w, 32w+32).
+// Workgroup = one (batch, head) and one slab of 128 value columns (value columns are independent of each
+// other; key channels beyond Dk read as zeros, whose state rows stay zero), 4 wavefronts; wavefront w
+// owns value columns [32w, 32w+32) of the slab.
 // Lane (dq = lane/8, jc = lane%8) holds S[16dq .. 16dq+15][32w+4jc .. +3] as 16 float4: state
 // loads and stores are 128-byte row segments, the per-token vectors k, q, exp(g) are 16
 // consecutive floats per lane read from LDS, and the two matrix-vector products reduce over the
@@ -16,7 +18,7 @@
 
 namespace daisy {
 
-constexpr int RD = 128;   // Dk = Dv
+constexpr int RD = 128;   // key channels and value columns a workgroup works on
 
 struct KdaStepParams {
   const uint16_t* q; const uint16_t* k; const uint16_t* v;
@@ -25,6 +27,7 @@ struct KdaStepParams {
   const float* s_in; float* s_out;
   uint16_t* o;
   int B, T, H;
+  int Dk, Dv;   // the tensors' own widths (Dk <= 128)
   float scale; int l2norm; float l2eps;
   // Packed sequences (B == 1, T = all tokens): workgroup (s, h) walks rows cu[s] .. cu[s+1]-1.
   const int32_t* cu; int n_seq;
@@ -47,16 +50,16 @@ __global__ __launch_bounds__(256) void kda_recurrent_kernel(KdaStepParams p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int dq = lane >> 3, jc = lane & 7;
   const int h = blockIdx.x % p.H, b = blockIdx.x / p.H;
-  const int col = 32 * wave + 4 * jc;
-  const int64_t sbase = ((int64_t)(b * p.H + h) * RD + 16 * dq) * RD + col;
+  const int col = RD * blockIdx.y + 32 * wave + 4 * jc;     // first of this lane's four value columns
+  const bool col_live = col < p.Dv;                         // (Dv is a multiple of 8: four columns are live or dead together)
+  const int64_t sbase = ((int64_t)(b * p.H + h) * p.Dk + 16 * dq) * p.Dv + col;
 
   f32x4 S[16];
-  if (p.s_in != nullptr) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) S[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p.s_in + sbase + (int64_t)i * RD));
-  } else {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) S[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < 16; ++i) {
+    S[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (p.s_in != nullptr && col_live && 16 * dq + i < p.Dk)
+      S[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p.s_in + sbase + (int64_t)i * p.Dv));
   }
 
   // Token rows of this recurrence on the flattened token axis; bounds read from the device are
@@ -71,10 +74,13 @@ __global__ __launch_bounds__(256) void kda_recurrent_kernel(KdaStepParams p) {
     // ---- stage k, q (L2-normalised) and exp(g) of this token in LDS ---------
     float kx = 0.f, qx = 0.f;
     if (tid < RD) {
-      kx = bf16lo_to_f32(p.k[row * RD + tid]);
-      qx = bf16lo_to_f32(p.q[row * RD + tid]);
-      const float gx = p.g_bf16 ? bf16lo_to_f32(reinterpret_cast<const uint16_t*>(p.g)[row * RD + tid])
-                                : reinterpret_cast<const float*>(p.g)[row * RD + tid];
+      float gx = 0.f;
+      if (tid < p.Dk) {
+        kx = bf16lo_to_f32(p.k[row * p.Dk + tid]);
+        qx = bf16lo_to_f32(p.q[row * p.Dk + tid]);
+        gx = p.g_bf16 ? bf16lo_to_f32(reinterpret_cast<const uint16_t*>(p.g)[row * p.Dk + tid])
+                      : reinterpret_cast<const float*>(p.g)[row * p.Dk + tid];
+      }
       eg[tid] = __expf(gx);
     }
     if (p.l2norm) {
@@ -89,7 +95,8 @@ __global__ __launch_bounds__(256) void kda_recurrent_kernel(KdaStepParams p) {
       qx *= qn;
     }
     if (tid < RD) { kf[tid] = kx; qf[tid] = qx; }
-    const u32x2 vraw = *reinterpret_cast<const u32x2*>(p.v + row * RD + col);
+    u32x2 vraw = {0u, 0u};
+    if (col_live) vraw = *reinterpret_cast<const u32x2*>(p.v + row * p.Dv + col);
     const f32x4 v4 = {bf16lo_to_f32(vraw.x), bf16hi_to_f32(vraw.x), bf16lo_to_f32(vraw.y), bf16hi_to_f32(vraw.y)};
     const float beta = p.beta[row];
     __syncthreads();
@@ -127,16 +134,17 @@ __global__ __launch_bounds__(256) void kda_recurrent_kernel(KdaStepParams p) {
     }
 #pragma unroll
     for (int c = 0; c < 4; ++c) out[c] = sum_over_dq(out[c]) * p.scale;
-    if (dq == 0) {
+    if (dq == 0 && col_live) {
       u32x2 w = {pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3])};
-      *reinterpret_cast<u32x2*>(p.o + row * RD + col) = w;
+      *reinterpret_cast<u32x2*>(p.o + row * p.Dv + col) = w;
     }
     __syncthreads();   // kf / qf / eg are rewritten by the next token
   }
 
-  if (p.s_out != nullptr) {
+  if (p.s_out != nullptr && col_live) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) __builtin_nontemporal_store(S[i], reinterpret_cast<f32x4*>(p.s_out + sbase + (int64_t)i * RD));
+    for (int i = 0; i < 16; ++i)
+      if (16 * dq + i < p.Dk) __builtin_nontemporal_store(S[i], reinterpret_cast<f32x4*>(p.s_out + sbase + (int64_t)i * p.Dv));
   }
 }
 
@@ -151,7 +159,8 @@ static int recurrent_launch(const void* q, const void* k, const void* v,
                             const float* initial_state, void* o, float* final_state,
                             int B, int T, int H, int Dk, int Dv,
                             float scale, int l2norm_qk, float l2_eps, void* stream) {
-  DAISY_CHECK_SUPPORTED(Dk == RD && Dv == RD, "kda_recurrent: Dk=%d, Dv=%d not supported (both must be %d)", Dk, Dv, RD);
+  DAISY_CHECK_SUPPORTED(Dk >= 8 && Dk <= RD && Dk % 8 == 0 && Dv >= 8 && Dv % 8 == 0,
+                        "kda_recurrent: Dk=%d, Dv=%d not supported (Dk: a multiple of 8 up to %d; Dv: a multiple of 8)", Dk, Dv, RD);
   DAISY_CHECK_ARG(q && k && v && g && beta && o, "kda_recurrent: q, k, v, g, beta and o must be non-NULL");
   DAISY_CHECK_ARG(B > 0 && T > 0 && H > 0, "kda_recurrent: B=%d, T=%d, H=%d must be positive", B, T, H);
   DAISY_CHECK_ARG((int64_t)B * H <= 0x7fffffff && (int64_t)B * T <= 0x7fffffff, "kda_recurrent: B*H or B*T too large");
@@ -161,10 +170,11 @@ static int recurrent_launch(const void* q, const void* k, const void* v,
   p.q = (const uint16_t*)q; p.k = (const uint16_t*)k; p.v = (const uint16_t*)v;
   p.g = g; p.g_bf16 = g_is_bf16; p.beta = beta;
   p.s_in = initial_state; p.s_out = final_state; p.o = (uint16_t*)o;
-  p.B = B; p.T = T; p.H = H;
+  p.B = B; p.T = T; p.H = H; p.Dk = Dk; p.Dv = Dv;
   p.scale = scale; p.l2norm = l2norm_qk; p.l2eps = l2_eps;
   p.cu = cu_seqlens; p.n_seq = cu_seqlens ? B : 0;
-  hipLaunchKernelGGL(kda_recurrent_kernel, dim3((unsigned)(B * H)), dim3(256), 0, (hipStream_t)stream, p);
+  DAISY_CHECK_ARG((Dv + RD - 1) / RD <= 65535, "kda_recurrent: Dv=%d too wide", Dv);
+  hipLaunchKernelGGL(kda_recurrent_kernel, dim3((unsigned)(B * H), (unsigned)((Dv + RD - 1) / RD)), dim3(256), 0, (hipStream_t)stream, p);
   DAISY_CHECK_LAUNCH("kda_recurrent_kernel");
   return DAISY_OK;
 }

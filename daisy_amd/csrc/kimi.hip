@@ -331,7 +331,7 @@ extern "C" int daisy_gated_rmsnorm_fwd(const void* x, const void* gate, const vo
                                        int64_t rows, int D, float eps, void* stream) {
   DAISY_CHECK_ARG(x && gate && weight && out, "gated_rmsnorm: x, gate, weight and out must be non-NULL");
   DAISY_CHECK_ARG(rows > 0, "gated_rmsnorm: rows=%lld must be positive", (long long)rows);
-  DAISY_CHECK_SUPPORTED(D == 64 || D == 128, "gated_rmsnorm: last dim %d not supported (64 or 128)", D);
+  DAISY_CHECK_SUPPORTED(D == 32 || D == 64 || D == 128 || D == 256, "gated_rmsnorm: last dim %d not supported (32, 64, 128 or 256)", D);
   auto al16 = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
   DAISY_CHECK_ARG(al16(x) && al16(gate) && al16(weight) && al16(out), "gated_rmsnorm: tensors must be 16-byte aligned");
   GatedNormParams p;
@@ -341,6 +341,8 @@ extern "C" int daisy_gated_rmsnorm_fwd(const void* x, const void* gate, const vo
   DAISY_CHECK_ARG(nwg <= 0x7fffffff, "gated_rmsnorm: too many rows (%lld)", (long long)rows);
   hipStream_t s = (hipStream_t)stream;
   if (D == 128) hipLaunchKernelGGL(gated_rmsnorm_kernel<128>, dim3((unsigned)nwg), dim3(256), 0, s, p);
+  else if (D == 256) hipLaunchKernelGGL(gated_rmsnorm_kernel<256>, dim3((unsigned)nwg), dim3(256), 0, s, p);
+  else if (D == 32) hipLaunchKernelGGL(gated_rmsnorm_kernel<32>, dim3((unsigned)nwg), dim3(256), 0, s, p);
   else hipLaunchKernelGGL(gated_rmsnorm_kernel<64>, dim3((unsigned)nwg), dim3(256), 0, s, p);
   DAISY_CHECK_LAUNCH("gated_rmsnorm_kernel");
   return DAISY_OK;

@@ -50,6 +50,47 @@ __global__ __launch_bounds__(512) void matrix_rate_kernel(float* sink, unsigned 
   }
 }
 
+// Register-only MFMAs whose operands CHANGE from one instruction to the next and hold the caller's data (eight A and
+// eight B fragments per lane, loaded once from `data`).  With operands of random bits the multiplier arrays toggle as
+// they do on real tensors; with a buffer of zeros or of one repeated value they do not.  The difference between the
+// two sustained rates is what the chip's power management takes for the data alone.
+template <int VARIANT>   // 0: A and B change with every instruction; 1: B stays the same (A changes); 2: A stays the same (B changes)
+__global__ __launch_bounds__(512) void matrix_rate_data_kernel(const u32x4* data, float* sink, unsigned long long* ticks, int iters) {
+  bf16x8 xs[8], ys[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    xs[j] = __builtin_bit_cast(bf16x8, data[(size_t)(2 * j) * 512 + threadIdx.x]);
+    ys[j] = __builtin_bit_cast(bf16x8, data[(size_t)(2 * j + 1) * 512 + threadIdx.x]);
+  }
+  f32x16 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+  const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xs[VARIANT == 2 ? 0 : j], ys[VARIANT == 1 ? 0 : j], acc[j & 3], 0, 0, 0);
+    // keep the sums bounded: the accumulators are cleared every 64 iterations (a handful of vector moves per 512 MFMAs)
+    if ((it & 63) == 63) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] *= 0.f;
+    }
+  }
+  const unsigned long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) s += acc[j][0];
+  sink[(blockIdx.x * 512 + threadIdx.x) & 4095] = s;
+  if (threadIdx.x == 0) {
+    ticks[2 * blockIdx.x] = c1 - c0;
+    ticks[2 * blockIdx.x + 1] = r1 - r0;
+  }
+}
+
 // The same with the attention loop's LDS operand traffic: per MFMA 3 fma and 1 exp2, and the A operand
 // of every MFMA comes from LDS with the kernel's own access patterns -- a 16-byte read of a swizzled
 // row-major tile (the K operand) for even MFMAs, two 8-byte transposing reads (the V operand) for
@@ -153,6 +194,22 @@ extern "C" int daisy_probe_read_rate(const void* buf, size_t bytes, int workgrou
   hipLaunchKernelGGL(read_rate_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream,
                      reinterpret_cast<const u32x4*>(buf), bytes / 16 / (size_t)workgroups, reinterpret_cast<uint32_t*>(sink));
   DAISY_CHECK_LAUNCH("read_rate_kernel");
+  return DAISY_OK;
+}
+
+extern "C" int daisy_probe_matrix_rate_data(const void* data, size_t data_bytes, int variant, int workgroups, int iters,
+                                            float* sink, unsigned long long* ticks, double* flop_out, void* stream) {
+  DAISY_CHECK_ARG(data && sink && ticks, "probe: data, sink (4096 floats) and ticks (2 per workgroup) must be non-NULL");
+  DAISY_CHECK_ARG(data_bytes >= 16 * 512 * 16 && (reinterpret_cast<uintptr_t>(data) & 15) == 0,
+                  "probe: data must hold 16 x 512 x 16 bytes, 16-byte aligned");
+  DAISY_CHECK_ARG(workgroups > 0 && iters > 0, "probe: workgroups=%d, iters=%d must be positive", workgroups, iters);
+  const u32x4* d = reinterpret_cast<const u32x4*>(data);
+  hipStream_t s = (hipStream_t)stream;
+  if (variant == 1) hipLaunchKernelGGL(matrix_rate_data_kernel<1>, dim3(workgroups), dim3(512), 0, s, d, sink, ticks, iters);
+  else if (variant == 2) hipLaunchKernelGGL(matrix_rate_data_kernel<2>, dim3(workgroups), dim3(512), 0, s, d, sink, ticks, iters);
+  else hipLaunchKernelGGL(matrix_rate_data_kernel<0>, dim3(workgroups), dim3(512), 0, s, d, sink, ticks, iters);
+  DAISY_CHECK_LAUNCH("matrix_rate_data_kernel");
+  if (flop_out) *flop_out = (double)workgroups * 8.0 * iters * 8.0 * 32768.0;
   return DAISY_OK;
 }
 

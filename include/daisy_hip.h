@@ -255,7 +255,9 @@ int daisy_attn_step_fwd(const void* q, const int64_t* q_strides,
  * beta  : fp32 [B, T, H] contiguous.
  * initial_state : fp32 [B, H, Dk, Dv] or NULL (zeros).
  * final_state   : fp32 [B, H, Dk, Dv] or NULL (not wanted).
- * Dk = Dv = 128 and chunk = 64 are the supported shapes.  T is arbitrary.
+ * Dk: a multiple of 8 up to 128.  Dv: any multiple of 8 (value columns are independent; they are
+ * processed in passes of up to 128 through the same workspace).  chunk = 64.  T is arbitrary.  The
+ * kernels are laid out for 128 x 128; narrower heads cost what 128 costs.
  * l2norm_qk : normalise q and k rows as x / sqrt(sum(x^2) + l2_eps) first.
  * workspace : >= daisy_kda_workspace_bytes(...) bytes, 256-byte aligned.
  */
@@ -298,7 +300,7 @@ int daisy_kda_chunk_varlen_fwd(const void* q, const void* k, const void* v,
  * models/daisy/attention_kimi.py:70,144 names and leaves unsupported; a
  * generation loop calls it with T = 1 per step, carrying the state.
  *
- * Tensors as in daisy_kda_chunk_fwd (contiguous [B, T, H, D]; Dk = Dv = 128).
+ * Tensors and head widths as in daisy_kda_chunk_fwd (contiguous [B, T, H, D]).
  * initial_state NULL = zeros; final_state NULL = not wanted; the two may alias.
  */
 int daisy_kda_recurrent_fwd(const void* q, const void* k, const void* v,
@@ -406,7 +408,7 @@ int daisy_short_conv_varlen_fwd(const void* x, int64_t x_row_stride, const void*
 
 /* daisy_gated_rmsnorm_fwd: out = x * rsqrt(mean(x^2) + eps) * weight * sigmoid(gate) over the last
  * dim, statistics in fp32, one rounding.  x, gate, out: [rows, D] bf16 contiguous; weight: [D] bf16;
- * D = 64 or 128.
+ * D = 32, 64, 128 or 256.
  */
 int daisy_gated_rmsnorm_fwd(const void* x, const void* gate, const void* weight, void* out,
                             int64_t rows, int D, float eps, void* stream);

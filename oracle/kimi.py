@@ -93,16 +93,19 @@ def kimi_layer_forward(x: torch.Tensor, p: dict, num_heads: int, head_dim: int, 
     ``p`` maps the reference's parameter names (``q_proj.weight``, ``q_conv1d.weight``, ``f_proj.0.weight``,
     ``f_proj.1.weight``, ``b_proj.weight``, ``A_log``, ``dt_bias``, ``g_proj.0.weight``, ``g_proj.1.weight``,
     ``g_proj.1.bias``, ``o_norm.weight``, ``o_proj.weight`` ...) to tensors.  The projections run in the
-    parameters' dtype, as in the reference (bf16 there); everything between them in fp32.
+    parameters' dtype, as in the reference (bf16 there); everything between them in fp32.  Value heads may
+    be wider than key heads (``head_v_dim = head_dim * expand_v``, attention_kimi.py:80): their width is read
+    off the value projection.
     """
     lin = torch.nn.functional.linear
     B, T, _ = x.shape
     H, D = num_heads, head_dim
+    Dv = p["v_proj.weight"].shape[0] // H
     x = x.to(p["q_proj.weight"].dtype)
     q, _ = short_conv(lin(x, p["q_proj.weight"]), p["q_conv1d.weight"], cu_seqlens=cu_seqlens)
     k, _ = short_conv(lin(x, p["k_proj.weight"]), p["k_conv1d.weight"], cu_seqlens=cu_seqlens)
     v, _ = short_conv(lin(x, p["v_proj.weight"]), p["v_conv1d.weight"], cu_seqlens=cu_seqlens)
-    q, k, v = (t.view(B, T, H, D) for t in (q, k, v))
+    q, k, v = q.view(B, T, H, D), k.view(B, T, H, D), v.view(B, T, H, Dv)
     if g_ve is not None:
         gx = torch.sigmoid(torch.as_tensor(g_ve, dtype=torch.float32))
         v = gx * v + (1.0 - gx) * ve.float().view_as(v)
@@ -112,10 +115,10 @@ def kimi_layer_forward(x: torch.Tensor, p: dict, num_heads: int, head_dim: int, 
         o, _ = kda_recurrent(q, k, v, g, beta, use_qk_l2norm=True)
     else:
         cu = [int(c) for c in cu_seqlens.tolist()]
-        o = torch.zeros(B, T, H, D)
+        o = torch.zeros(B, T, H, Dv)
         for s, e in zip(cu[:-1], cu[1:]):
             if e > s:
                 o[:, s:e], _ = kda_recurrent(q[:, s:e], k[:, s:e], v[:, s:e], g[:, s:e], beta[:, s:e], use_qk_l2norm=True)
-    gate = lin(lin(x, p["g_proj.0.weight"]), p["g_proj.1.weight"], p["g_proj.1.bias"]).view(B, T, H, D)
+    gate = lin(lin(x, p["g_proj.0.weight"]), p["g_proj.1.weight"], p["g_proj.1.bias"]).view(B, T, H, Dv)
     o = gated_rms_norm(o, gate, p["o_norm.weight"])
-    return lin(o.reshape(B, T, H * D).to(p["o_proj.weight"].dtype), p["o_proj.weight"])
+    return lin(o.reshape(B, T, H * Dv).to(p["o_proj.weight"].dtype), p["o_proj.weight"])

@@ -91,8 +91,16 @@ def test_kda_argument_errors():
     lib = _lib.load()
     buf = ctypes.create_string_buffer(64)
     p = ctypes.addressof(buf)
-    rc = lib.daisy_kda_chunk_fwd(p, p, p, p, 0, p, None, p, None, 1, 64, 1, 64, 128, 64, 0.1, 1, 1e-6, None, 0, None)
-    assert rc == -2 and "Dk" in _err()
+    for Dk, Dv in ((136, 128), (60, 128), (128, 20), (0, 128)):      # Dk: a multiple of 8 up to 128; Dv: a multiple of 8
+        rc = lib.daisy_kda_chunk_fwd(p, p, p, p, 0, p, None, p, None, 1, 64, 1, Dk, Dv, 64, 0.1, 1, 1e-6, None, 0, None)
+        assert rc == -2 and "Dk" in _err(), (Dk, Dv)
+        assert lib.daisy_kda_workspace_bytes(1, 64, 1, Dk, Dv, 64) == 0
+        rc = lib.daisy_kda_recurrent_fwd(p, p, p, p, 0, p, None, p, None, 1, 1, 1, Dk, Dv, 0.1, 1, 1e-6, None)
+        assert rc == -2 and "Dk" in _err(), (Dk, Dv)
+    # narrower and wider heads share the workspace of the 128 x 128 layout (value columns go through it in passes)
+    assert lib.daisy_kda_workspace_bytes(1, 64, 1, 64, 64, 64) == lib.daisy_kda_workspace_bytes(1, 64, 1, 128, 256, 64) > 0
+    rc = lib.daisy_kda_chunk_fwd(p, p, p, p, 0, p, None, p, None, 1, 64, 1, 64, 256, 64, 0.1, 1, 1e-6, None, 0, None)
+    assert rc == -3 and "workspace" in _err()
     rc = lib.daisy_kda_chunk_fwd(None, p, p, p, 0, p, None, p, None, 1, 64, 1, 128, 128, 64, 0.1, 1, 1e-6, None, 0, None)
     assert rc == -1
     rc = lib.daisy_kda_chunk_fwd(p, p, p, p, 0, p, None, p, None, 1, 64, 1, 128, 128, 64, 0.1, 1, 1e-6, None, 0, None)

@@ -25,6 +25,9 @@ def _ref_decode(q, k_rows, v_rows, scale=0.12):
     (3, 2, 64, 200, 777, 3),
     (1, 1, 128, 1, 9, 0),        # W = 1: only the new row
     (4, 8, 128, 4096, 8192, 0),  # the benchmark's ring shape at small batch
+    (1, 12, 128, 8192, 8292, 0),   # one sequence, 12 heads, ring of 8192 (model_specs/daisy_milli.yml; the generator's batch of one)
+    (1, 12, 128, 8192, 8292, 16),
+    (1, 12, 128, 8192, 300, 0),    # the same ring early in a generation: 301 live rows
 ])
 def test_decode_ring_matches_oracle(B, H, D, W, t, nsplit):
     say(f"decode ring case B{B} H{H} D{D} W{W} t{t} nsplit{nsplit}")

@@ -113,9 +113,83 @@ def test_kda_gate_matches_oracle():
 
 
 def test_kda_rejects_unsupported_shapes():
-    z = torch.zeros(1, 64, 1, 64, dtype=torch.bfloat16, device="cuda:0")
+    z = torch.zeros(1, 64, 1, 136, dtype=torch.bfloat16, device="cuda:0")
     with pytest.raises(RuntimeError, match="Dk"):
         ops.kda_chunk_fwd(z, z, z, z.float(), torch.zeros(1, 64, 1, device="cuda:0"))
+
+
+def _inputs_dims(B, T, H, Dk, Dv, seed, g_scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = F.normalize(torch.randn(B, T, H, Dk, generator=g), dim=-1).bfloat16()
+    k = F.normalize(torch.randn(B, T, H, Dk, generator=g), dim=-1).bfloat16()
+    v = torch.randn(B, T, H, Dv, generator=g).bfloat16()
+    gl = F.logsigmoid(torch.randn(B, T, H, Dk, generator=g)) * g_scale
+    beta = torch.sigmoid(torch.randn(B, T, H, generator=g))
+    S0 = torch.randn(B, H, Dk, Dv, generator=g) * 0.1
+    return q, k, v, gl, beta, S0
+
+
+# Head widths other than 128 x 128: the reference's own KDA spec has head_dim 64 (model_specs/old/daisy_pico_linear.yml:5-13)
+# and the layer has expand_v (models/daisy/attention_kimi.py:68,80: head_v_dim = head_dim * expand_v).
+HEAD_DIMS = [(64, 64), (64, 128), (128, 256), (128, 64), (32, 40), (96, 136), (8, 8), (128, 392)]
+
+
+@pytest.mark.parametrize("Dk,Dv", HEAD_DIMS)
+@pytest.mark.parametrize("T,g_scale,g_bf16", [(200, 1.0, False), (70, 8.0, True)])
+def test_kda_other_head_widths_match_recurrence(Dk, Dv, T, g_scale, g_bf16):
+    """Chunked and token-by-token kernels, with an initial state, default scale Dk**-0.5, against the recurrence."""
+    B, H = 2, 3
+    say(f"kda widths Dk{Dk} Dv{Dv} T{T} g_scale{g_scale} g_bf16={g_bf16}")
+    q, k, v, gl, beta, S0 = _inputs_dims(B, T, H, Dk, Dv, seed=Dk + Dv + T, g_scale=g_scale)
+    if g_bf16:
+        gl = gl.bfloat16()
+    o_ref, S_ref = oracle.kda_recurrent(q, k, v, gl.float(), beta, initial_state=S0)
+    dev = lambda t: t.cuda()
+    o, S = chunk_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), initial_state=dev(S0), output_final_state=True,
+                     use_qk_l2norm_in_kernel=True)
+    assert o.shape == (B, T, H, Dv) and S.shape == (B, H, Dk, Dv)
+    _check(o, S, o_ref, S_ref, f"chunked Dk{Dk} Dv{Dv}")
+    o_r, S_r = fused_recurrent_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), initial_state=dev(S0), output_final_state=True,
+                                   use_qk_l2norm_in_kernel=True)
+    _check(o_r, S_r, o_ref, S_ref, f"recurrent Dk{Dk} Dv{Dv}")
+    # no initial state, no L2 norm, explicit scale
+    o_ref2, S_ref2 = oracle.kda_recurrent(q, k, v, gl.float(), beta, scale=0.3, use_qk_l2norm=False)
+    o2, S2 = chunk_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), scale=0.3, output_final_state=True, use_qk_l2norm_in_kernel=False)
+    _check(o2, S2, o_ref2, S_ref2, f"chunked, no norm, Dk{Dk} Dv{Dv}")
+
+
+def test_kda_narrow_heads_decode_steps_and_packed_sequences():
+    """Dk = Dv = 64: a chunked prefill continued by in-place decode steps equals one run; packed sequences
+    (cu_seqlens) run each from its own state, in both kernels."""
+    B, T0, n_steps, H, D = 2, 130, 12, 2, 64
+    T = T0 + n_steps
+    q, k, v, gl, beta, _ = (t.cuda() for t in _inputs_dims(B, T, H, D, D, seed=5))
+    o_ref, S_ref = oracle.kda_recurrent(q.cpu(), k.cpu(), v.cpu(), gl.cpu(), beta.cpu())
+    o0, S = chunk_kda(q[:, :T0], k[:, :T0], v[:, :T0], gl[:, :T0], beta[:, :T0], output_final_state=True, use_qk_l2norm_in_kernel=True)
+    outs = [o0]
+    for t in range(T0, T):
+        o_t, S_t = fused_recurrent_kda(q[:, t:t + 1], k[:, t:t + 1], v[:, t:t + 1], gl[:, t:t + 1], beta[:, t:t + 1],
+                                       initial_state=S, use_qk_l2norm_in_kernel=True, inplace_state=True)
+        assert S_t.data_ptr() == S.data_ptr()
+        outs.append(o_t)
+    _check(torch.cat(outs, 1), S, o_ref, S_ref, "narrow heads: prefill + decode steps")
+    lens = [70, 0, 64, 9]
+    cu = torch.tensor([0, 70, 70, 134, 143], dtype=torch.int32)
+    q, k, v, gl, beta, _ = _inputs_dims(1, 143, H, D, 2 * D, seed=6)
+    S0 = torch.randn(len(lens), H, D, 2 * D, generator=torch.Generator().manual_seed(7)) * 0.1
+    dev = lambda t: t.cuda()
+    o, S = chunk_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), initial_state=dev(S0), output_final_state=True,
+                     use_qk_l2norm_in_kernel=True, cu_seqlens=cu.cuda())
+    o_r, S_r = fused_recurrent_kda(dev(q), dev(k), dev(v), dev(gl), dev(beta), initial_state=dev(S0), output_final_state=True,
+                                   use_qk_l2norm_in_kernel=True, cu_seqlens=cu.cuda())
+    for i, n in enumerate(lens):
+        s, e = int(cu[i]), int(cu[i + 1])
+        if n == 0:
+            assert torch.equal(S[i].cpu(), S0[i]) and torch.equal(S_r[i].cpu(), S0[i])
+            continue
+        o_ref, S_ref = oracle.kda_recurrent(q[:, s:e], k[:, s:e], v[:, s:e], gl[:, s:e], beta[:, s:e], initial_state=S0[i:i + 1])
+        _check(o[:, s:e], S[i:i + 1], o_ref, S_ref, f"narrow heads, chunked, sequence {i}")
+        _check(o_r[:, s:e], S_r[i:i + 1], o_ref, S_ref, f"narrow heads, recurrent, sequence {i}")
 
 
 # ---- token-by-token kernel (decode steps, short prompts) ------------------------------------
@@ -169,7 +243,7 @@ def test_kda_decode_steps_continue_a_chunked_prefill():
 def test_kda_recurrent_rejects_bad_arguments():
     q, k, v, gl, beta = (t.cuda() for t in _inputs(1, 4, 1, seed=3))
     with pytest.raises(RuntimeError, match="not supported"):
-        ops.kda_recurrent_fwd(q[..., :64].contiguous(), k[..., :64].contiguous(), v, gl[..., :64].contiguous(), beta)
+        ops.kda_recurrent_fwd(q[..., :60].contiguous(), k[..., :60].contiguous(), v, gl[..., :60].contiguous(), beta)
     with pytest.raises(ValueError):
         ops.kda_recurrent_fwd(q, k, v, gl, beta, inplace_state=True)
 

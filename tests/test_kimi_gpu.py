@@ -19,9 +19,10 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _layer(dim=256, H=2, seed=0, receives_ve=False):
+def _layer(dim=256, H=2, seed=0, receives_ve=False, head_dim=128, expand_v=1.0, conv_size=4):
     torch.manual_seed(seed)
-    m = KimiLinearSelfAttention(dim, H, max_seq_len=1024, head_dim=128, receives_ve=receives_ve)
+    m = KimiLinearSelfAttention(dim, H, max_seq_len=1024, head_dim=head_dim, expand_v=expand_v, conv_size=conv_size,
+                                receives_ve=receives_ve)
     with torch.no_grad():
         for p in m.parameters():
             if p.dim() >= 2 and p.dtype == torch.bfloat16:
@@ -57,6 +58,39 @@ def test_forward_matches_cpu_layer(B, T, receives_ve):
         y = md(x.to(DEV), None if ve is None else ve.to(DEV))
         assert y.shape == (B, T, 256) and y.dtype == torch.bfloat16
         _close(y, y_ref, "forward vs CPU layer", 3e-2)
+
+
+@pytest.mark.parametrize("H,head_dim,expand_v,conv_size", [
+    (4, 64, 1.0, 4),      # the reference's own KDA spec: head_dim 64 (model_specs/old/daisy_pico_linear.yml:5-13)
+    (4, 64, 2.0, 3),      # value heads twice as wide as key heads (attention_kimi.py:68,80)
+    (2, 128, 2.0, 4),     # 256 value columns per head: two passes of the delta-rule kernels
+    (8, 32, 1.0, 2),
+])
+def test_other_head_widths_match_cpu_layer_and_stream(H, head_dim, expand_v, conv_size):
+    """Forward against the oracle's layer, and prompt + decode steps against the full forward, at head widths
+    other than 128."""
+    with torch.no_grad():
+        kw = dict(H=H, head_dim=head_dim, expand_v=expand_v, conv_size=conv_size, seed=7)
+        m = _layer(**kw)
+        assert m.head_v_dim == int(head_dim * expand_v) and m.value_dim == H * m.head_v_dim
+        g = torch.Generator().manual_seed(8)
+        x = torch.randn(2, 150, 256, generator=g).bfloat16()
+        params = {k: v.detach() for k, v in m.state_dict().items()}
+        y_ref = oracle.kimi_layer_forward(x, params, H, head_dim, conv_size=conv_size)
+        md = _layer(**kw).to(DEV)
+        md.load_state_dict(m.state_dict())
+        xd = x.to(DEV)
+        y = md(xd, None)
+        _close(y, y_ref, f"forward vs CPU layer, head_dim {head_dim} expand_v {expand_v}", 3e-2)
+        y0, _, _ = md.prefill(xd[:, :130], None)
+        ys = [y0] + [md.step(xd[:, t:t + 1], None, None, t, None, None)[0] for t in range(130, 150)]
+        _close(torch.cat(ys, 1), y, "prefill + steps vs full forward", 2e-2)
+
+
+def test_constructor_refuses_what_the_kernels_do_not_serve():
+    for kw in (dict(head_dim=160), dict(head_dim=36), dict(head_dim=128, expand_v=0.75), dict(head_dim=128, conv_size=5)):
+        with pytest.raises(ValueError, match="not supported"):
+            KimiLinearSelfAttention(256, 2, max_seq_len=64, **kw)
 
 
 def test_prefill_then_steps_equals_full_forward():
@@ -211,7 +245,7 @@ def test_short_convolution_window_updated_in_place():
         ops.short_conv(torch.zeros(B, 40, C, device=DEV, dtype=torch.bfloat16), w, bias, window.clone(), True, inplace_cache=True)
 
 
-@pytest.mark.parametrize("rows,D", [(5, 128), (1000, 128), (77, 64)])
+@pytest.mark.parametrize("rows,D", [(5, 128), (1000, 128), (77, 64), (33, 32), (130, 256)])
 def test_gated_rmsnorm_kernel_matches_oracle(rows, D):
     from daisy_amd import ops
     g = torch.Generator().manual_seed(rows)

@@ -128,11 +128,12 @@ def probe_matrix_rate(with_vector_mix, iters=50000, workgroups=256, device="cuda
     return {"ms": ms, "tflops": flop.value / ms / 1e9, "clock_mhz": float(t[0] / t[1] * 100.0)}
 
 
-def probe_matrix_rate_data(kind, seconds=1.0, iters=80000, workgroups=256, device="cuda:0"):
+def probe_matrix_rate_data(kind, seconds=1.0, iters=80000, workgroups=256, device="cuda:0", variant=0):
     """Sustained rate of register-only bf16 MFMAs whose operands change with every instruction and hold `kind` data
     ("zeros" or "normal": N(0,1) rounded to bf16), launches back to back for `seconds`; the rate and clock of the last
     quarter of the run.  The instruction stream is the same for both kinds: the difference is what the chip's power
-    management takes for the toggling of the operand bits."""
+    management takes for the toggling of the operand bits.  variant 3: the attention loop's mix (per MFMA 3 fma + 1 exp2,
+    A operands read from LDS) instead of MFMAs alone, LDS tile and B operands filled with the data."""
     import ctypes
     dev = torch.device(device)
     n_el = 16 * 512 * 8
@@ -145,7 +146,7 @@ def probe_matrix_rate_data(kind, seconds=1.0, iters=80000, workgroups=256, devic
     stream = torch.cuda.current_stream(dev).cuda_stream
 
     def run():
-        rc = lib.daisy_probe_matrix_rate_data(data.data_ptr(), n_el * 2, 0, workgroups, iters, sink.data_ptr(), ticks.data_ptr(),
+        rc = lib.daisy_probe_matrix_rate_data(data.data_ptr(), n_el * 2, variant, workgroups, iters, sink.data_ptr(), ticks.data_ptr(),
                                               ctypes.byref(flop), stream)
         assert rc == 0, rc
 
@@ -763,6 +764,10 @@ def main():
                 probe_matrix_rate_data("normal"),
                 what="the same instruction stream on N(0,1) bf16 operands: the sustained rate of the matrix pipe ALONE on data like "
                      "the benchmark's; the power management lowers the clock until the chip stays inside its power limit"),
+            "mfma_with_attention_mix_and_lds_operands_on_normal_data": dict(
+                probe_matrix_rate_data("normal", iters=50000, variant=3),
+                what="the stream of mfma_with_attention_mix_and_lds_operands below, sustained for a second, with the LDS tile and "
+                     "the B operands holding N(0,1) values: what the attention loop's instruction mix can reach on such data"),
             "mfma_with_attention_vector_mix": probe_matrix_rate(True, 60000),
             "mfma_with_attention_mix_and_lds_operands": dict(
                 probe_matrix_rate(2, 50000),

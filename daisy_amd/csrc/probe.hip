@@ -98,9 +98,11 @@ __global__ __launch_bounds__(512) void matrix_rate_data_kernel(const u32x4* data
 // rate of this stream is what the layout of prefill_tile_kernel (two or three wavefronts per SIMD) can reach at
 // best with its instruction mix.
 typedef short probe_s16x4 __attribute__((ext_vector_type(4)));
-__global__ __launch_bounds__(512) void attention_mix_kernel(float* sink, unsigned long long* ticks, int iters) {
+// data: NULL, or 64 x 128 + 512 x 8 bf16 values that fill the LDS tile and the B operands (N(0,1) values make the
+// operand bits toggle as they do on real tensors; without it the tile holds a few repeated values).
+__global__ __launch_bounds__(512) void attention_mix_kernel(const uint16_t* data, float* sink, unsigned long long* ticks, int iters) {
   __shared__ __attribute__((aligned(1024))) uint16_t tile[64 * 128];
-  for (int i = threadIdx.x; i < 64 * 128; i += 512) tile[i] = (uint16_t)(0x3c00 + (i & 63));
+  for (int i = threadIdx.x; i < 64 * 128; i += 512) tile[i] = data ? data[i] : (uint16_t)(0x3c00 + (i & 63));
   __syncthreads();
   const int lane = threadIdx.x & 63, lq = lane & 31, lh = lane >> 5;
   typedef __attribute__((address_space(3))) const uint16_t* lptr;
@@ -133,6 +135,7 @@ __global__ __launch_bounds__(512) void attention_mix_kernel(float* sink, unsigne
   bf16x8 y;
 #pragma unroll
   for (int e = 0; e < 8; ++e) y[e] = (__bf16)(0.11f * ((threadIdx.x * 3 + e) % 17) - 1.f);
+  if (data) y = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(data + 64 * 128 + 8 * threadIdx.x));
   bf16x8 opa[8], opb[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) opa[j] = read_operand(j);
@@ -205,7 +208,10 @@ extern "C" int daisy_probe_matrix_rate_data(const void* data, size_t data_bytes,
   DAISY_CHECK_ARG(workgroups > 0 && iters > 0, "probe: workgroups=%d, iters=%d must be positive", workgroups, iters);
   const u32x4* d = reinterpret_cast<const u32x4*>(data);
   hipStream_t s = (hipStream_t)stream;
-  if (variant == 1) hipLaunchKernelGGL(matrix_rate_data_kernel<1>, dim3(workgroups), dim3(512), 0, s, d, sink, ticks, iters);
+  if (variant == 3) {   // the attention loop's mix: vector work and LDS operand reads next to the MFMAs, on the caller's data
+    iters = (iters + 1) & ~1;
+    hipLaunchKernelGGL(attention_mix_kernel, dim3(workgroups), dim3(512), 0, s, reinterpret_cast<const uint16_t*>(data), sink, ticks, iters);
+  } else if (variant == 1) hipLaunchKernelGGL(matrix_rate_data_kernel<1>, dim3(workgroups), dim3(512), 0, s, d, sink, ticks, iters);
   else if (variant == 2) hipLaunchKernelGGL(matrix_rate_data_kernel<2>, dim3(workgroups), dim3(512), 0, s, d, sink, ticks, iters);
   else hipLaunchKernelGGL(matrix_rate_data_kernel<0>, dim3(workgroups), dim3(512), 0, s, d, sink, ticks, iters);
   DAISY_CHECK_LAUNCH("matrix_rate_data_kernel");
@@ -218,7 +224,7 @@ extern "C" int daisy_probe_matrix_rate(int with_vector_mix, int workgroups, int 
   DAISY_CHECK_ARG(sink && ticks, "probe: sink (4096 floats) and ticks (2 per workgroup) must be non-NULL");
   DAISY_CHECK_ARG(workgroups > 0 && iters > 0, "probe: workgroups=%d, iters=%d must be positive", workgroups, iters);
   hipStream_t s = (hipStream_t)stream;
-  if (with_vector_mix == 2) hipLaunchKernelGGL(attention_mix_kernel, dim3(workgroups), dim3(512), 0, s, sink, ticks, (iters + 1) & ~1);
+  if (with_vector_mix == 2) hipLaunchKernelGGL(attention_mix_kernel, dim3(workgroups), dim3(512), 0, s, (const uint16_t*)nullptr, sink, ticks, (iters + 1) & ~1);
   else if (with_vector_mix) hipLaunchKernelGGL(matrix_rate_kernel<1>, dim3(workgroups), dim3(512), 0, s, sink, ticks, iters);
   else hipLaunchKernelGGL(matrix_rate_kernel<0>, dim3(workgroups), dim3(512), 0, s, sink, ticks, iters);
   DAISY_CHECK_LAUNCH("matrix_rate_kernel");

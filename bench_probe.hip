@@ -5,7 +5,7 @@
 // (per MFMA: 5 fma and 1 exp2).  No LDS, no memory traffic: the rate is bounded by instruction
 // issue and by the clock the power management grants, and is the ceiling against which the
 // attention kernel's own rate can be read (the published 2.5 PFLOP/s assumes 2.4 GHz).
-#include "common.h"
+#include "daisy_amd/csrc/common.h"
 
 namespace daisy {
 

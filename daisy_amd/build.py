@@ -16,11 +16,12 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_NAME = "libdaisy_hip.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
 SOURCES = ["abi.hip", "decode.hip", "prefill.hip", "kda.hip", "kda_step.hip", "prep.hip", "kimi.hip"]
-# Diagnostic kernels for the benchmark (matrix-pipe and read-stream ceilings, a copy kernel of known
-# size): their own library, not part of the product ABI.
-PROBE_LIB_NAME = "libdaisy_probe.so"
-PROBE_LIB_PATH = os.path.join(CSRC, PROBE_LIB_NAME)
-PROBE_SOURCES = ["abi.hip", "probe.hip"]
+# Diagnostic kernels of the benchmark (matrix-pipe and read-stream ceilings): not part of the product.  Their source
+# sits next to bench.py at the repository root and is built into a library of its own there, which only bench.py loads.
+ROOT = os.path.dirname(os.path.dirname(CSRC))
+PROBE_LIB_NAME = "libdaisy_bench_probe.so"
+PROBE_LIB_PATH = os.path.join(ROOT, PROBE_LIB_NAME)
+PROBE_SOURCE = os.path.join(ROOT, "bench_probe.hip")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -43,8 +44,9 @@ def _hipcc() -> str:
 
 
 def _compile(src: str, verbose: bool) -> str:
-    obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    path = src if os.path.isabs(src) else os.path.join(CSRC, src)
+    obj = os.path.splitext(path)[0] + ".o"
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-I", ROOT, "-c", path, "-o", obj]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -71,11 +73,14 @@ def build(verbose: bool = True, sources=None) -> str:
     """Compiles every source and links the product library (and the benchmark's probe library);
     returns the product library's path."""
     srcs = list(sources or SOURCES)
-    every = srcs + [s for s in PROBE_SOURCES if s not in srcs]
+    every = srcs + ([PROBE_SOURCE] if os.path.exists(PROBE_SOURCE) else [])
+    if "abi.hip" not in every:
+        every.append("abi.hip")
     with ThreadPoolExecutor(max_workers=min(4, len(every))) as ex:
         objs = dict(zip(every, ex.map(lambda s: _compile(s, verbose), every)))
     _link([objs[s] for s in srcs], LIB_PATH, verbose)
-    _link([objs[s] for s in PROBE_SOURCES], PROBE_LIB_PATH, verbose)
+    if PROBE_SOURCE in objs:
+        _link([objs["abi.hip"], objs[PROBE_SOURCE]], PROBE_LIB_PATH, verbose)
     return LIB_PATH
 
 

@@ -400,12 +400,19 @@ __global__ __launch_bounds__(D) void decode_combine_kernel(DecodeParams p) {
 }
 
 static int choose_nsplit(int B, int H, int n_rows) {
-  // Aim for about 1024 workgroups on the 256 compute units (more, shorter ones measured no
-  // faster), keep at least 256 rows per workgroup so every wavefront has two full iterations.
+  // About 512 rows per workgroup (two full iterations of every wavefront and some), as long as that does not make
+  // more than about 1024 workgroups; when it leaves fewer than 192 workgroups on the 256 compute units (a few
+  // (batch, head) pairs: the generator's batch of one), shorter splits down to 128 rows.  From a sweep over
+  // B*H = 6..1024, 1024..8192 rows and 1..64 splits; within a few per cent of the best count everywhere.
   const int bh = B * H;
-  int ns = (1024 + bh - 1) / bh;
-  const int max_by_rows = n_rows / 256 > 0 ? n_rows / 256 : 1;
-  if (ns > max_by_rows) ns = max_by_rows;
+  int by_rows = n_rows / 512 > 0 ? n_rows / 512 : 1;
+  const int by_grid = (1024 + bh - 1) / bh;
+  int ns = by_rows < by_grid ? by_rows : by_grid;
+  if (bh * ns < 192) {
+    by_rows = n_rows / 128 > 0 ? n_rows / 128 : 1;
+    const int fill = (192 + bh - 1) / bh;
+    ns = by_rows < fill ? by_rows : fill;
+  }
   if (ns < 1) ns = 1;
   if (ns > 64) ns = 64;
   return ns;

@@ -7,9 +7,11 @@ from torch import Tensor
 
 
 def norm(x: Tensor) -> Tensor:
-    """Weightless RMS norm over the last dim, eps = finfo(dtype).eps.
+    """Weightless RMS norm over the last dim with the library's default eps.
 
-    Same call as the reference's ``norm`` (models/daisy/functional.py:6-7).
+    Same call as the reference's ``norm`` (models/daisy/functional.py:6-7): no eps is passed, and torch 2.10
+    then adds the machine epsilon of its accumulation type -- fp32's for bf16 and fp32 inputs alike, on the
+    CPU and on the GPU -- not ``finfo(x.dtype).eps`` (see ``NORM_EPS_BF16`` below).
     """
     return F.rms_norm(x, (x.size(-1),))
 

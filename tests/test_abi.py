@@ -40,6 +40,27 @@ def test_workspace_queries_need_no_gpu():
     assert lib.daisy_kda_workspace_bytes(4, 8192, 16, 128, 128, 64) > 0
 
 
+def test_split_count_the_library_picks():
+    """nsplit = 0 lets the library choose; the workspace size shows the choice (B * H * splits * (D + 2) floats).
+    About 512 rows per workgroup, at most about 1024 workgroups, and shorter splits (down to 128 rows) when a few
+    (batch, head) pairs would otherwise leave most compute units idle."""
+    lib = _lib.load()
+
+    def splits(B, H, n_rows, D=128):
+        nbytes = lib.daisy_decode_workspace_bytes(B, H, D, n_rows, 0)
+        return 1 if nbytes == 0 else nbytes // (B * H * (D + 2) * 4)
+
+    assert splits(64, 16, 4096) == 1          # BASELINE config 4: one workgroup per (batch, head) already fills the chip
+    assert splits(16, 8, 4096) == 8           # 512 rows each
+    assert splits(1, 12, 8192) == 16          # the generator's batch of one (model_specs/daisy_milli.yml): 512 rows each
+    assert splits(1, 12, 1024) == 8           # few pairs, short ring: 128 rows each
+    assert splits(1, 6, 8192) == 32
+    assert splits(4, 12, 300) == 2
+    assert splits(1, 1, 100) == 1
+    for B, H, n in ((1, 1, 10 ** 6), (3, 5, 70000)):
+        assert 1 <= splits(B, H, n) <= 64
+
+
 def _err():
     return _lib.load().daisy_last_error().decode()
 

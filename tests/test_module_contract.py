@@ -56,3 +56,22 @@ def test_a_reference_state_dict_loads(device):
     assert torch.equal(attn.qkvo_w.detach().cpu(), src["qkvo_w"]) and float(attn.g_ve.detach()) == 0.25
     with pytest.raises((RuntimeError, AssertionError)):
         CausalSelfAttention(dim, 3, 64, max_seq_len=16)                 # attention.py:76: dim % num_heads
+
+
+def test_kimi_layer_constructor_contract():
+    """KimiLinearSelfAttention (models/daisy/attention_kimi.py:64-110): the reference's parameter names, shapes and
+    dtypes at head widths other than 128, and a clear refusal of what the kernels under the layer do not serve."""
+    from daisy_amd import KimiLinearSelfAttention
+    m = KimiLinearSelfAttention(256, 4, max_seq_len=64, head_dim=64, expand_v=2.0, conv_size=3)
+    assert (m.head_k_dim, m.head_v_dim, m.key_dim, m.value_dim) == (64, 128, 256, 512)      # attention_kimi.py:79-82
+    sd = m.state_dict()
+    assert sd["q_proj.weight"].shape == (256, 256) and sd["v_proj.weight"].shape == (512, 256)
+    assert sd["q_conv1d.weight"].shape == (256, 1, 3) and sd["v_conv1d.weight"].shape == (512, 1, 3)
+    assert sd["f_proj.0.weight"].shape == (128, 256) and sd["f_proj.1.weight"].shape == (256, 128)
+    assert sd["g_proj.1.weight"].shape == (512, 128) and sd["g_proj.1.bias"].shape == (512,)
+    assert sd["o_norm.weight"].shape == (128,) and sd["o_proj.weight"].shape == (256, 512)
+    assert sd["A_log"].shape == (1, 1, 4, 1) and sd["A_log"].dtype == torch.float32 and sd["dt_bias"].shape == (256,)
+    assert sd["b_proj.weight"].shape == (4, 256) and sd["q_proj.weight"].dtype == torch.bfloat16
+    for kw in (dict(head_dim=160), dict(head_dim=36), dict(head_dim=128, expand_v=0.75), dict(head_dim=128, conv_size=5)):
+        with pytest.raises(ValueError, match="not supported"):
+            KimiLinearSelfAttention(256, 2, max_seq_len=64, **kw)

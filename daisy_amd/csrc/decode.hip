@@ -61,30 +61,44 @@ __device__ __forceinline__ DecodeRange decode_range(const DecodeParams& p) {
 
 constexpr int kDecodeThreads = 256;
 constexpr int kDecodeWaves = kDecodeThreads / 64;
-constexpr int kDecodeUnroll = 8;  // 16-byte loads in flight per lane and tensor
+constexpr int kDecodeUnroll = 4;  // 16-byte loads per lane, tensor and register set (two sets)
 
-// Loads this lane's 8 channels of a [D] bf16 vector, optionally rotates them
-// with the position's cos/sin row (pairs (i, i + D/2)), rounds to bf16 like the
-// reference does after RoPE, and returns them as floats.
+// The new token's rows are fetched in two steps -- raw loads first, arithmetic later -- so that the
+// kernel can put the first cache-row loads between the two: the rows and the rotation table take a
+// memory round trip that the stream of cache rows then does not wait for.
+struct RawRow { u32x4 own, par; };   // this lane's 8 channels and the 8 they are rotated with
+struct TrigRow { float c[8], s[8]; };
+
 template <int D>
-__device__ __forceinline__ void load_vec_rot(const uint16_t* vec, int dl, const float* cos_row, const float* sin_row,
-                                             float* out) {
-  u32x4 own = *reinterpret_cast<const u32x4*>(vec + dl);
-  unpack8(own, out);
-  if (cos_row != nullptr) {
-    constexpr int HALF = D / 2;
-    const bool lower = dl < HALF;
-    const int pl = lower ? dl + HALF : dl - HALF;
-    u32x4 par = *reinterpret_cast<const u32x4*>(vec + pl);
-    float pf[8];
-    unpack8(par, pf);
-    const int tl = lower ? dl : dl - HALF;
+__device__ __forceinline__ RawRow load_raw_row(const uint16_t* vec, int dl, bool with_partner) {
+  constexpr int HALF = D / 2;
+  RawRow r;
+  r.own = *reinterpret_cast<const u32x4*>(vec + dl);
+  r.par = with_partner ? *reinterpret_cast<const u32x4*>(vec + (dl < HALF ? dl + HALF : dl - HALF)) : r.own;
+  return r;
+}
+template <int D>
+__device__ __forceinline__ TrigRow load_trig_row(const float* cos_row, const float* sin_row, int dl) {
+  constexpr int HALF = D / 2;
+  const int tl = dl < HALF ? dl : dl - HALF;
+  TrigRow t;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float c = cos_row[tl + i], s = sin_row[tl + i];
-      const float y = lower ? rope_lo(out[i], pf[i], c, s) : rope_hi(pf[i], out[i], c, s);
-      out[i] = round_bf16(y);
-    }
+  for (int i = 0; i < 8; ++i) { t.c[i] = cos_row[tl + i]; t.s[i] = sin_row[tl + i]; }
+  return t;
+}
+
+// This lane's 8 channels of a [D] bf16 vector rotated with the position's cos/sin row (pairs
+// (i, i + D/2)) and rounded to bf16 like the reference does after RoPE, as floats.
+template <int D>
+__device__ __forceinline__ void rot_row(const RawRow& r, const TrigRow& t, int dl, float* out) {
+  const bool lower = dl < D / 2;
+  float pf[8];
+  unpack8(r.own, out);
+  unpack8(r.par, pf);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float y = lower ? rope_lo(out[i], pf[i], t.c[i], t.s[i]) : rope_hi(pf[i], out[i], t.c[i], t.s[i]);
+    out[i] = round_bf16(y);
   }
 }
 
@@ -92,15 +106,12 @@ __device__ __forceinline__ void load_vec_rot(const uint16_t* vec, int dl, const 
 // rounded to bf16 like the norm's output tensor, then the rotation, rounded again: the arithmetic
 // and the roundings of qkv_prep_kernel for one row.
 template <int D>
-__device__ __forceinline__ void norm_rot(const uint16_t* vec, int dl, const float* cos_row, const float* sin_row,
-                                         float eps, float* out) {
-  constexpr int LPR = D / 8, HALF = D / 2;
-  const bool lower = dl < HALF;
-  const int pl = lower ? dl + HALF : dl - HALF;
-  const int tl = lower ? dl : dl - HALF;
+__device__ __forceinline__ void norm_rot_row(const RawRow& r, const TrigRow& t, int dl, float eps, float* out) {
+  constexpr int LPR = D / 8;
+  const bool lower = dl < D / 2;
   float own[8], par[8];
-  unpack8(*reinterpret_cast<const u32x4*>(vec + dl), own);
-  unpack8(*reinterpret_cast<const u32x4*>(vec + pl), par);
+  unpack8(r.own, own);
+  unpack8(r.par, par);
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) ss += own[i] * own[i];
@@ -109,19 +120,18 @@ __device__ __forceinline__ void norm_rot(const uint16_t* vec, int dl, const floa
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float a = round_bf16(own[i] * rstd), b = round_bf16(par[i] * rstd);
-    const float c = cos_row[tl + i], sn = sin_row[tl + i];
-    out[i] = round_bf16(lower ? rope_lo(a, b, c, sn) : rope_hi(b, a, c, sn));
+    out[i] = round_bf16(lower ? rope_lo(a, b, t.c[i], t.s[i]) : rope_hi(b, a, t.c[i], t.s[i]));
   }
 }
 
 // RMS norm of a value row and, when a second row is given, gate * v + (1 - gate) * ve with every
 // product and the sum rounded to bf16 (the roundings of a bf16 tensor library).
 template <int D>
-__device__ __forceinline__ void norm_mix(const uint16_t* vec, const uint16_t* ve, const float* gate, int dl,
-                                         float eps, float* out) {
+__device__ __forceinline__ void norm_mix_row(const u32x4& v_raw, bool with_ve, const u32x4& ve_raw, float g, float eps,
+                                             float* out) {
   constexpr int LPR = D / 8;
   float own[8];
-  unpack8(*reinterpret_cast<const u32x4*>(vec + dl), own);
+  unpack8(v_raw, own);
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) ss += own[i] * own[i];
@@ -129,10 +139,9 @@ __device__ __forceinline__ void norm_mix(const uint16_t* vec, const uint16_t* ve
   const float rstd = rsqrtf(ss / (float)D + eps);
 #pragma unroll
   for (int i = 0; i < 8; ++i) out[i] = round_bf16(own[i] * rstd);
-  if (ve != nullptr) {
+  if (with_ve) {
     float e[8];
-    unpack8(*reinterpret_cast<const u32x4*>(ve + dl), e);
-    const float g = gate[0];
+    unpack8(ve_raw, e);
     const float og = round_bf16(1.0f - g);
 #pragma unroll
     for (int i = 0; i < 8; ++i) out[i] = round_bf16(round_bf16(g * out[i]) + round_bf16(og * e[i]));
@@ -185,76 +194,75 @@ __device__ __forceinline__ void merge_state(SoftmaxState& a, const SoftmaxState&
 // PREP: q, k_new and v_new are rows of the QKV projection output; the kernel normalises, rotates
 // and mixes them itself (every workgroup of a (batch, head) redoes these few hundred flops).
 // F16C: the cache rows are fp16 (the new rows are converted on their way in).
+//
+// Order of the memory instructions: the new token's rows and the table rows (raw), then the first two
+// sets of cache rows, and only then the arithmetic on the new rows; inside the loop a register set is
+// loaded again as soon as it has been used.  A wavefront so keeps 2 * kDecodeUnroll KiB of cache rows
+// in flight from its first instructions to its last row: with a few hundred workgroups on the chip
+// (one sequence, a dozen heads) the launch is a handful of memory round trips long, and every trip
+// spent with nothing in flight shows.
 template <int D, bool PREP, bool F16C = false>
 __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) {
   constexpr int LPR = D / 8;        // lanes per cache row
   constexpr int RPW = 64 / LPR;     // rows per wavefront load
   constexpr int U = kDecodeUnroll;
-  constexpr int RB = RPW * U;       // rows per wavefront iteration
+  constexpr int RB = RPW * U;       // rows of one register set
+  constexpr int STRIDE = kDecodeWaves * RB;   // rows the four wavefronts cover with one set each
 
   const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int sub = lane / LPR;
   const int dl = (lane % LPR) * 8;
 
-  float qf[8], knf[8];
-  u32x4 vn_packed;
+  const DecodeRange rg = decode_range(p);
+  const int new_idx = rg.new_idx;
+  const int r0 = split * rg.rows_per_split;
+  const int r1 = min(r0 + rg.rows_per_split, rg.n_rows);
+  // Only the split that holds the new token's slot needs the new key and value rows.
+  const bool holds_new = new_idx >= r0 && new_idx < r0 + rg.rows_per_split;
+  uint16_t* kbase = p.kc + b * p.kc_sb + h * p.kc_sh + dl;
+  uint16_t* vbase = p.vc + b * p.vc_sb + h * p.vc_sh + dl;
+  const uint16_t* q_row = p.q + b * p.q_sb + h * p.q_sh;
+  const uint16_t* kn_row = p.k_new + b * p.kn_sb + h * p.kn_sh;
+  const uint16_t* vn_row = p.v_new + b * p.vn_sb + h * p.vn_sh;
+
+  // Raw rows of the new token.
+  RawRow q_raw, kn_raw;
+  TrigRow trig;
+  u32x4 vn_raw, ve_raw = {0u, 0u, 0u, 0u};
+  float gate = 0.f;
+  bool past_tables = false, rotate = true;
   if constexpr (PREP) {
     const int t = p.pos_dev != nullptr ? max(p.pos_dev[0], 0) : p.pos_host;
     // A position past the rotation tables (possible only when it comes from device memory) reads the
     // last table row, to stay inside the allocation, and is reported: the status word gets its bit and
     // the outputs of the step are NaN, so that the step cannot pass for a valid one.
-    const bool past_tables = t >= p.table_rows;
+    past_tables = t >= p.table_rows;
     const int64_t trow = (int64_t)min(t, p.table_rows - 1) * (D / 2);
-    norm_rot<D>(p.q + b * p.q_sb + h * p.q_sh, dl, p.cos_tab + trow, p.sin_tab + trow, p.eps, qf);
-    if (past_tables) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) qf[i] = __builtin_nanf("");
-      if (p.status != nullptr && tid == 0 && split == 0 && h == 0 && b == 0)
-        __hip_atomic_fetch_or(p.status, DAISY_STATUS_POSITION_PAST_TABLES, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    trig = load_trig_row<D>(p.cos_tab + trow, p.sin_tab + trow, dl);
+    q_raw = load_raw_row<D>(q_row, dl, true);
+    kn_raw = load_raw_row<D>(holds_new ? kn_row : q_row, dl, true);
+    vn_raw = *reinterpret_cast<const u32x4*>((holds_new ? vn_row : q_row) + dl);
+    if (p.ve != nullptr) {
+      ve_raw = *reinterpret_cast<const u32x4*>((holds_new ? p.ve + b * p.ve_sb + h * p.ve_sh : q_row) + dl);
+      gate = p.gate[0];
     }
-    // Only the split that holds the new token's slot needs the new key and value rows.
-    const DecodeRange own = decode_range(p);
-    const int own0 = split * own.rows_per_split;
-    float vnf[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { knf[i] = 0.f; vnf[i] = 0.f; }
-    if (own.new_idx >= own0 && own.new_idx < own0 + own.rows_per_split) {
-      norm_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_tab + trow, p.sin_tab + trow, p.eps, knf);
-      norm_mix<D>(p.v_new + b * p.vn_sb + h * p.vn_sh, p.ve ? p.ve + b * p.ve_sb + h * p.ve_sh : nullptr, p.gate, dl, p.eps, vnf);
-    }
-    vn_packed = F16C ? pack8_f16(vnf) : pack8(vnf);
   } else {
     static_assert(!F16C, "fp16 cache rows come with the kernel-side preparation only");
-    load_vec_rot<D>(p.q + b * p.q_sb + h * p.q_sh, dl, p.cos_row, p.sin_row, qf);
-    load_vec_rot<D>(p.k_new + b * p.kn_sb + h * p.kn_sh, dl, p.cos_row, p.sin_row, knf);
-    vn_packed = *reinterpret_cast<const u32x4*>(p.v_new + b * p.vn_sb + h * p.vn_sh + dl);
+    rotate = p.cos_row != nullptr;
+    if (rotate) trig = load_trig_row<D>(p.cos_row, p.sin_row, dl);
+    q_raw = load_raw_row<D>(q_row, dl, rotate);
+    kn_raw = load_raw_row<D>(kn_row, dl, rotate);
+    vn_raw = *reinterpret_cast<const u32x4*>(vn_row + dl);
   }
-  const u32x4 kn_packed = F16C ? pack8_f16(knf) : pack8(knf);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) qf[i] *= p.scale_log2e;
-
-  const DecodeRange rg = decode_range(p);
-  const int new_idx = rg.new_idx;
-  const int r0 = split * rg.rows_per_split;
-  const int r1 = min(r0 + rg.rows_per_split, rg.n_rows);
-  uint16_t* kbase = p.kc + b * p.kc_sb + h * p.kc_sh + dl;
-  uint16_t* vbase = p.vc + b * p.vc_sb + h * p.vc_sh + dl;
-
-  SoftmaxState st;
-  st.m = -INFINITY;
-  st.l = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) st.acc[i] = 0.f;
 
   // Lanes whose row is past the range, or is the new token's slot, load a row
   // that is always readable instead (and are masked / overwritten below).
   const int safe_row = (r0 != new_idx) ? r0 : r0 + 1;
-  const uint16_t* k_safe = (safe_row < r1) ? kbase + (int64_t)safe_row * p.kc_sr : p.k_new + b * p.kn_sb + h * p.kn_sh + dl;
-  const uint16_t* v_safe = (safe_row < r1) ? vbase + (int64_t)safe_row * p.vc_sr : p.v_new + b * p.vn_sb + h * p.vn_sh + dl;
+  const uint16_t* k_safe = (safe_row < r1) ? kbase + (int64_t)safe_row * p.kc_sr : kn_row + dl;
+  const uint16_t* v_safe = (safe_row < r1) ? vbase + (int64_t)safe_row * p.vc_sr : vn_row + dl;
 
-  for (int base = r0 + wave * RB; base < r1; base += kDecodeWaves * RB) {
-    u32x4 kr[U], vr[U];
+  auto load_set = [&](int base, u32x4* kr, u32x4* vr) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int row = base + u * RPW + sub;
@@ -267,7 +275,55 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
       const uint16_t* a = (row < r1 && row != new_idx) ? vbase + (int64_t)row * p.vc_sr : v_safe;
       vr[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a));
     }
+  };
 
+  // Two register sets; a set past the end of the range loads the safe row (one cache line) and is not used.
+  u32x4 kA[U], vA[U], kB[U], vB[U];
+  int base = r0 + wave * RB;
+  __builtin_amdgcn_sched_barrier(0);
+  load_set(base, kA, vA);
+  load_set(base + STRIDE, kB, vB);
+  __builtin_amdgcn_sched_barrier(0);
+
+  float qf[8], knf[8];
+  u32x4 vn_packed;
+  if constexpr (PREP) {
+    norm_rot_row<D>(q_raw, trig, dl, p.eps, qf);
+    if (past_tables) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qf[i] = __builtin_nanf("");
+      if (p.status != nullptr && tid == 0 && split == 0 && h == 0 && b == 0)
+        __hip_atomic_fetch_or(p.status, DAISY_STATUS_POSITION_PAST_TABLES, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    float vnf[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { knf[i] = 0.f; vnf[i] = 0.f; }
+    if (holds_new) {
+      norm_rot_row<D>(kn_raw, trig, dl, p.eps, knf);
+      norm_mix_row<D>(vn_raw, p.ve != nullptr, ve_raw, gate, p.eps, vnf);
+    }
+    vn_packed = F16C ? pack8_f16(vnf) : pack8(vnf);
+  } else {
+    if (rotate) {
+      rot_row<D>(q_raw, trig, dl, qf);
+      rot_row<D>(kn_raw, trig, dl, knf);
+    } else {
+      unpack8(q_raw.own, qf);
+      unpack8(kn_raw.own, knf);
+    }
+    vn_packed = vn_raw;
+  }
+  const u32x4 kn_packed = F16C ? pack8_f16(knf) : pack8(knf);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) qf[i] *= p.scale_log2e;
+
+  SoftmaxState st;
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) st.acc[i] = 0.f;
+
+  auto consume = [&](int base, u32x4* kr, u32x4* vr) {
     float s[U];
     float mblk = -INFINITY;
 #pragma unroll
@@ -307,6 +363,13 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
 #pragma unroll
       for (int i = 0; i < 8; ++i) st.acc[i] = fmaf(pu, vf[i], st.acc[i]);
     }
+  };
+
+  for (; base < r1; base += 2 * STRIDE) {
+    consume(base, kA, vA);
+    load_set(base + 2 * STRIDE, kA, vA);
+    if (base + STRIDE < r1) consume(base + STRIDE, kB, vB);
+    load_set(base + 3 * STRIDE, kB, vB);
   }
 
   // Merge the row groups of this wavefront (lanes that differ above bit log2(LPR)).
@@ -360,40 +423,67 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_kernel(DecodeParams p) 
   }
 }
 
-// Combines the per-split partials of one (batch, head); one thread per channel.  The partials of
-// eight splits are fetched together (independent loads, one memory round trip per eight splits).
+// Combines the per-split partials of one (batch, head).  The workgroup is 1 to kCombineThreads / D groups of D
+// threads (one group per eight splits), a thread per channel; group g takes the splits g, g + groups, ... (at most
+// kCombineUnroll of them) and fetches all of its partials with independent loads -- one memory round trip
+// whatever the split count -- and the groups are merged through LDS.
+constexpr int kCombineThreads = 512;
+constexpr int kCombineUnroll = 16;
+constexpr int kMaxSplits = kCombineUnroll * (kCombineThreads / 128);   // 64, for D = 64 and 128 alike
+static int combine_threads(int D, int nsplit) {
+  const int groups = (nsplit + 7) / 8 < kCombineThreads / D ? (nsplit + 7) / 8 : kCombineThreads / D;
+  return groups * D;
+}
 template <int D>
-__global__ __launch_bounds__(D) void decode_combine_kernel(DecodeParams p) {
-  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+__global__ __launch_bounds__(kCombineThreads) void decode_combine_kernel(DecodeParams p) {
+  constexpr int GMAX = kCombineThreads / D;
+  constexpr int U = kCombineUnroll;
+  const int G = blockDim.x / D;            // split groups of this launch; g is the same for all lanes of a wavefront
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x % D, g = threadIdx.x / D;
   const float* part = p.partials + ((int64_t)b * p.H + h) * p.nsplit * (D + 2);
-  constexpr int U = 8;
-  float m = -INFINITY, l = 0.f, acc = 0.f;
-  for (int s0 = 0; s0 < p.nsplit; s0 += U) {
-    float ms[U], ls[U], as[U];
+  float ms[U], ls[U], as[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int s = min(s0 + u, p.nsplit - 1);   // surplus slots re-read the last split and are ignored
+  for (int u = 0; u < U; ++u) {
+    const int s = g + u * G;
+    ms[u] = -INFINITY;
+    ls[u] = 0.f;
+    as[u] = 0.f;
+    if (s < p.nsplit) {
       ms[u] = part[s * (D + 2)];
       ls[u] = part[s * (D + 2) + 1];
       as[u] = part[s * (D + 2) + 2 + d];
     }
-    float mb = m;
+  }
+  float m = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (s0 + u < p.nsplit) mb = fmaxf(mb, ms[u]);
-    const float mu = (mb == -INFINITY) ? 0.f : mb;
-    const float keep = fast_exp2(m - mu);
-    l *= keep;
-    acc *= keep;
+  for (int u = 0; u < U; ++u) m = fmaxf(m, ms[u]);
+  const float mu = (m == -INFINITY) ? 0.f : m;
+  float l = 0.f, acc = 0.f;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (s0 + u < p.nsplit) {
-        const float w = fast_exp2(ms[u] - mu);
-        l = fmaf(ls[u], w, l);
-        acc = fmaf(as[u], w, acc);
-      }
+  for (int u = 0; u < U; ++u) {
+    const float w = fast_exp2(ms[u] - mu);   // an absent split has m = -inf: weight 0
+    l = fmaf(ls[u], w, l);
+    acc = fmaf(as[u], w, acc);
+  }
+  __shared__ float sm_m[GMAX], sm_l[GMAX], sm_acc[GMAX][D];
+  if (G > 1) {
+    if (d == 0) {
+      sm_m[g] = m;
+      sm_l[g] = l;
     }
-    m = mb;
+    sm_acc[g][d] = acc;
+    __syncthreads();
+    if (g != 0) return;
+    m = sm_m[0];
+    for (int i = 1; i < G; ++i) m = fmaxf(m, sm_m[i]);
+    const float mut = (m == -INFINITY) ? 0.f : m;
+    l = 0.f;
+    acc = 0.f;
+    for (int i = 0; i < G; ++i) {
+      const float w = fast_exp2(sm_m[i] - mut);
+      l = fmaf(sm_l[i], w, l);
+      acc = fmaf(sm_acc[i][d], w, acc);
+    }
   }
   const float r = acc / l;
   p.o[b * p.o_sb + h * p.o_sh + d] = (uint16_t)(pack_bf16x2(r, 0.f) & 0xffffu);
@@ -414,12 +504,13 @@ static int choose_nsplit(int B, int H, int n_rows) {
     ns = by_rows < fill ? by_rows : fill;
   }
   if (ns < 1) ns = 1;
-  if (ns > 64) ns = 64;
+  if (ns > kMaxSplits) ns = kMaxSplits;
   return ns;
 }
 
 static int resolve_nsplit(int B, int H, int n_rows, int nsplit) {
   if (nsplit <= 0) nsplit = choose_nsplit(B, H, n_rows);
+  if (nsplit > kMaxSplits) nsplit = kMaxSplits;   // what the combine kernel takes
   if (nsplit > n_rows) nsplit = n_rows;
   if (nsplit < 1) nsplit = 1;
   const int rps = (n_rows + nsplit - 1) / nsplit;
@@ -608,7 +699,7 @@ static int decode_launch(const void* q, const int64_t* q_strides,
     else hipLaunchKernelGGL((decode_kernel<128, false>), grid, dim3(kDecodeThreads), 0, s, p);
     DAISY_CHECK_LAUNCH("decode_kernel");
     if (p.nsplit > 1) {
-      hipLaunchKernelGGL(decode_combine_kernel<128>, dim3(H, B), dim3(128), 0, s, p);
+      hipLaunchKernelGGL(decode_combine_kernel<128>, dim3(H, B), dim3(combine_threads(128, p.nsplit)), 0, s, p);
       DAISY_CHECK_LAUNCH("decode_combine_kernel");
     }
   } else {
@@ -617,7 +708,7 @@ static int decode_launch(const void* q, const int64_t* q_strides,
     else hipLaunchKernelGGL((decode_kernel<64, false>), grid, dim3(kDecodeThreads), 0, s, p);
     DAISY_CHECK_LAUNCH("decode_kernel");
     if (p.nsplit > 1) {
-      hipLaunchKernelGGL(decode_combine_kernel<64>, dim3(H, B), dim3(64), 0, s, p);
+      hipLaunchKernelGGL(decode_combine_kernel<64>, dim3(H, B), dim3(combine_threads(64, p.nsplit)), 0, s, p);
       DAISY_CHECK_LAUNCH("decode_combine_kernel");
     }
   }

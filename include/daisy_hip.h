@@ -127,7 +127,7 @@ int daisy_prefill_fwd_f32(const float* q, const int64_t* q_strides,
  *                      (applied to q and k_new), or both NULL.
  * workspace          : >= daisy_decode_workspace_bytes(...) bytes, 256-byte
  *                      aligned; may be NULL when that function returns 0.
- * nsplit             : number of sequence splits per (b, h); 0 = choose.
+ * nsplit             : number of sequence splits per (b, h); 0 = choose; values above 64 are taken as 64.
  * D is 64 or 128 for the streaming kernel; any other even D <= 256 runs a
  * one-wavefront-per-(batch, head) kernel meant for small test shapes (no splits).
  */

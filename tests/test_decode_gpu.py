@@ -28,6 +28,11 @@ def _ref_decode(q, k_rows, v_rows, scale=0.12):
     (1, 12, 128, 8192, 8292, 0),   # one sequence, 12 heads, ring of 8192 (model_specs/daisy_milli.yml; the generator's batch of one)
     (1, 12, 128, 8192, 8292, 16),
     (1, 12, 128, 8192, 300, 0),    # the same ring early in a generation: 301 live rows
+    (1, 12, 128, 8192, 8292, 64),  # the largest split count: every combine thread takes its full share of partials
+    (1, 12, 128, 8192, 8292, 100), # more than that is taken as 64
+    (1, 3, 64, 4096, 5000, 37),    # odd counts: combine groups with unequal numbers of splits
+    (2, 2, 128, 2048, 3000, 9),
+    (2, 2, 64, 2048, 3000, 5),     # fewer splits than combine groups at D = 64
 ])
 def test_decode_ring_matches_oracle(B, H, D, W, t, nsplit):
     say(f"decode ring case B{B} H{H} D{D} W{W} t{t} nsplit{nsplit}")

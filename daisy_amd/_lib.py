@@ -16,7 +16,8 @@ import torch
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libdaisy_hip.so")
 _lib: Optional[ctypes.CDLL] = None
 
-ABI_VERSION = 3
+ABI_VERSION = 4
+LINEAR_MAX_ROWS = 8
 STATUS_POSITION_PAST_TABLES = 1
 DECODE_STATIC_SCRATCH_BYTES = 4 << 20
 
@@ -126,6 +127,8 @@ SIGNATURES = {
         c_void_p, c_int, c_void_p,                              # cu_seqlens (device int32), n_seq, cache_in
         c_void_p, c_int64, c_void_p,                            # y, y row stride, cache_out
         c_int, c_int, c_int, c_int, c_void_p]),                 # T, C, K, apply_silu, stream
+    "daisy_linear_rows_fwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,   # x, w, y (+ row strides)
+                                       c_int, c_int, c_int, c_void_p]),                          # M, N, K, stream
     "daisy_qkv_prep_fwd": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q, k, v (+ strides)
         c_void_p, _I64P, c_void_p,                               # ve, ve strides, gate

@@ -509,6 +509,47 @@ def kda_gate_fwd(g: torch.Tensor, A_log: torch.Tensor, head_k_dim: int,
     return out
 
 
+def linear_rows_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether ``linear_rows`` takes this pair: bf16 on a GPU, at most ``_lib.LINEAR_MAX_ROWS`` rows of ``x``,
+    rows of both starting on 16-byte boundaries."""
+    if not (x.is_cuda and weight.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16):
+        return False
+    if weight.dim() != 2 or x.dim() < 1 or x.shape[-1] != weight.shape[1] or weight.shape[1] % 8 != 0:
+        return False
+    rows = x.numel() // x.shape[-1] if x.shape[-1] else 0
+    if not 1 <= rows <= _lib.LINEAR_MAX_ROWS:
+        return False
+    return weight.stride(1) == 1 and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0
+
+
+def linear_rows(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``F.linear(x, weight)`` for the few activation rows of a decode step (``daisy_linear_rows_fwd``):
+    ``x [..., K]`` bf16 with at most ``_lib.LINEAR_MAX_ROWS`` rows in all, ``weight [N, K]`` bf16 (rows may be
+    strided); returns ``[..., N]`` bf16.  Reads the weights once; fp32 accumulation, one rounding."""
+    dev = _lib.require_gpu(x, weight, out)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise TypeError(f"linear_rows: x and weight must be bf16, got {x.dtype}, {weight.dtype}")
+    if weight.dim() != 2 or x.dim() < 1 or x.shape[-1] != weight.shape[1]:
+        raise ValueError(f"linear_rows: x [..., K] and weight [N, K] do not fit: {tuple(x.shape)}, {tuple(weight.shape)}")
+    if weight.stride(1) != 1:
+        raise ValueError("linear_rows: the weight's last dim must be contiguous")
+    N, K = weight.shape
+    x2 = x.reshape(-1, K)
+    if x2.stride(1) != 1 or (x2.size(0) > 1 and x2.stride(0) % 8 != 0) or x2.data_ptr() % 16 != 0:
+        x2 = x2.contiguous()
+    M = x2.size(0)
+    if out is None:
+        out = torch.empty(*x.shape[:-1], N, dtype=torch.bfloat16, device=dev)
+    elif out.dtype != torch.bfloat16 or out.shape != (*x.shape[:-1], N) or not out.is_contiguous():
+        raise ValueError(f"linear_rows: out must be a contiguous bf16 {(*x.shape[:-1], N)} tensor")
+    lib = _lib.load()
+    with _lib.on_device(dev):
+        rc = lib.daisy_linear_rows_fwd(x2.data_ptr(), x2.stride(0) if M > 1 else K, weight.data_ptr(), weight.stride(0),
+                                       out.data_ptr(), N, M, N, K, _lib.current_stream(dev))
+    _lib.check(rc, "daisy_linear_rows_fwd")
+    return out
+
+
 def qkv_prep(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, eps: float,
              cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
              pos0: Union[int, torch.Tensor] = 0,

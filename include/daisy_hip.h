@@ -377,6 +377,21 @@ int daisy_qkv_prep_fwd_at(const void* q, const int64_t* q_strides,
                           int B, int T, int H, int D, float eps, void* stream);
 
 /* ---------------------------------------------------------------------------
+ * The two projections of a decode step, F.linear(x, qkvo_w[:3].flatten(end_dim=1)) and
+ * F.linear(y, qkvo_w[3]) (models/daisy/attention.py:119-120 and :201), for the one activation row per
+ * sequence that a step has:
+ *     y[m, n] = sum_k x[m, k] * w[n, k]        m < M <= 8
+ * bf16 in and out, fp32 accumulation, one rounding at the end.  The call reads the weights once
+ * (N * K * 2 bytes: bound by HBM bandwidth); more rows than 8 belong to a library GEMM
+ * (DAISY_ERR_UNSUPPORTED).
+ * x : [M, K] bf16, row stride x_row_stride elements;  w : [N, K] bf16 (the layout of a Linear weight),
+ *     row stride w_row_stride;  y : [M, N] bf16, row stride y_row_stride.  K a multiple of 8; x, w and
+ *     their row strides such that every row starts on a 16-byte boundary.
+ */
+int daisy_linear_rows_fwd(const void* x, int64_t x_row_stride, const void* w, int64_t w_row_stride,
+                          void* y, int64_t y_row_stride, int M, int N, int K, void* stream);
+
+/* ---------------------------------------------------------------------------
  * The KDA layer's elementwise neighbours (models/daisy/attention_kimi.py:155-158: three
  * ShortConvolution modules in front of chunk_kda; :136-137: the gated RMS norm behind it; both
  * modules come from a package absent from the reference checkout and are restated from their

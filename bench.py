@@ -583,14 +583,14 @@ def bench_decode_b1(steps, warmup):
             cache.t = t_before
             return core.step(model, tok, cache)
 
-        ms_eager = time_gpu(step_eager, max(steps, 32), max(warmup, 8))
+        ms_eager = time_gpu(step_eager, max(steps, 4), max(warmup, 4))
         recorded = core.GraphedStep(model, cache)
 
         def step_recorded():
             cache.t = t_before
             return recorded(tok)
 
-        ms_graph = time_gpu(step_recorded, max(4 * steps, 128), max(warmup, 8))
+        ms_graph = time_gpu(step_recorded, max(4 * steps, 16), max(warmup, 8))
         # the attention launches alone: the one-launch step (norm, RoPE, append, attention) on each layer's ring
         cos, sin = model.blocks[0].attn.rotary.cos, model.blocks[0].attn.rotary.sin
         raw = torch.randn(1, 3 * H, D, generator=g, device=dev).bfloat16()
@@ -610,12 +610,38 @@ def bench_decode_b1(steps, warmup):
             torch.cuda.synchronize()
             with torch.cuda.graph(graph):
                 attn_layers()
-            variants["library_choice" if nsplit == 0 else f"nsplit{nsplit}"] = time_gpu(graph.replay, max(4 * steps, 128), 8)
+            variants["library_choice" if nsplit == 0 else f"nsplit{nsplit}"] = time_gpu(graph.replay, max(4 * steps, 16), 8)
             del graph
+        # the step's two projections, one activation row against each layer's own matrices (12 different matrices per
+        # replay: 226 MB, nothing stays in the caches), through the few-rows kernel and through the library's GEMM
+        x_row = torch.randn(1, 1, dim, generator=g, device=dev).bfloat16()
+        projections = {}
+        for label, weights in (("qkv_4608x1536", [b.attn.qkvo_w[:3].flatten(end_dim=1) for b in model.blocks]),
+                               ("out_1536x1536", [b.attn.qkvo_w[3] for b in model.blocks])):
+            outs = [torch.empty(1, 1, w.shape[0], dtype=torch.bfloat16, device=dev) for w in weights]
+            per = {}
+            for name, fn in (("linear_rows", lambda w, y: ops.linear_rows(x_row, w, out=y)),
+                             ("library_gemm", lambda w, y: torch.nn.functional.linear(x_row, w))):
+                def all_layers():
+                    for w, y in zip(weights, outs):
+                        fn(w, y)
+                graph = torch.cuda.CUDAGraph()
+                all_layers()
+                torch.cuda.synchronize()
+                with torch.cuda.graph(graph):
+                    all_layers()
+                per[name] = time_gpu(graph.replay, max(4 * steps, 16), 8) / L
+                del graph
+            wbytes = weights[0].numel() * 2
+            projections[label] = {"weight_bytes": wbytes, "us_per_call": per["linear_rows"] * 1e3,
+                                  "gbs": wbytes / per["linear_rows"] / 1e6,
+                                  "frac_of_hbm_peak": wbytes / per["linear_rows"] / 1e6 / PEAK_HBM_GBS,
+                                  "us_per_call_library_gemm": per["library_gemm"] * 1e3}
     nbytes = L * 2 * W * H * D * 2
     row = lambda ms: {"ms_per_token": ms, "gbs": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBS}
     out.update({"kv_bytes_per_token": nbytes, "model_step_eager": row(ms_eager), "model_step_recorded_graph": row(ms_graph),
                 "attention_launches_only_recorded_graph": {k: row(v) for k, v in variants.items()},
+                "projections_one_row_recorded_graph": projections,
                 "what": "model step = embed, 12 x (norm, QKV projection, one-launch attention step, output projection, residual), "
                         "final norm, vocabulary projection; attention launches only = the 12 decode launches (+ their split "
                         "combines) replayed as one graph"})

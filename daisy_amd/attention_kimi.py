@@ -32,6 +32,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from . import ops
+from .attention import _step_linear
 from .kda import chunk_kda, fused_kda_gate, fused_recurrent_kda
 
 
@@ -75,6 +76,13 @@ class GatedRMSNorm(nn.Module):
 
     def forward(self, x: Tensor, gate: Tensor) -> Tensor:
         return ops.gated_rmsnorm(x, gate, self.weight, self.eps)
+
+
+def _project(lin: nn.Linear, x: Tensor) -> Tensor:
+    """``lin(x)``; a bias-free projection of a decode step's few rows reads its weights through the few-rows kernel."""
+    if lin.bias is None:
+        return _step_linear(x, lin.weight)
+    return lin(x)
 
 
 class KimiLinearSelfAttention(nn.Module):
@@ -196,19 +204,19 @@ class KimiLinearSelfAttention(nn.Module):
             # a decode step shifts its windows in place (same tensors, same addresses, every step)
             shift = (use_cache and T == 1 and cu_seqlens is None
                      and all(c is not None and c.dtype == torch.bfloat16 and c.is_contiguous() for c in convs))
-            q, cq = self.q_conv1d(self.q_proj(x), convs[0], use_cache, cu_seqlens, shift)
-            k, ck = self.k_conv1d(self.k_proj(x), convs[1], use_cache, cu_seqlens, shift)
-            v, cv = self.v_conv1d(self.v_proj(x), convs[2], use_cache, cu_seqlens, shift)
+            q, cq = self.q_conv1d(_project(self.q_proj, x), convs[0], use_cache, cu_seqlens, shift)
+            k, ck = self.k_conv1d(_project(self.k_proj, x), convs[1], use_cache, cu_seqlens, shift)
+            v, cv = self.v_conv1d(_project(self.v_proj, x), convs[2], use_cache, cu_seqlens, shift)
         else:
-            q, k, v = F.silu(self.q_proj(x)), F.silu(self.k_proj(x)), F.silu(self.v_proj(x))
+            q, k, v = F.silu(_project(self.q_proj, x)), F.silu(_project(self.k_proj, x)), F.silu(_project(self.v_proj, x))
             cq = ck = cv = None
         q, k, v = q.view(B, T, H, Dk), k.view(B, T, H, Dk), v.view(B, T, H, Dv)
         if self.receives_ve:
             torch._assert(ve is not None, "ve must be provided when receives_ve=True")
             g_x = torch.sigmoid(self.g_ve).to(v.dtype)
             v = g_x * v + (1.0 - g_x) * ve.view_as(v).to(v.dtype)
-        g = fused_kda_gate(self.f_proj(x), self.A_log, Dk, self.dt_bias)
-        beta = torch.sigmoid(self.b_proj(x)).to(torch.float32)
+        g = fused_kda_gate(_project(self.f_proj[1], _project(self.f_proj[0], x)), self.A_log, Dk, self.dt_bias)
+        beta = torch.sigmoid(_project(self.b_proj, x)).to(torch.float32)
         if use_cache and T == 1 and state is not None and cu_seqlens is None:
             o, state = fused_recurrent_kda(q, k, v, g, beta, initial_state=state, use_qk_l2norm_in_kernel=True,
                                            inplace_state=True)
@@ -221,9 +229,9 @@ class KimiLinearSelfAttention(nn.Module):
             self._conv_state = tuple(self._store(h, c) for h, c in zip(homes[1:], (cq, ck, cv)))
             self._state_homes[state.shape[0]] = (self._recurrent_state,) + self._conv_state
             self._seen += T
-        gate = self.g_proj(x).view(B, T, H, Dv)
+        gate = self.g_proj[1](_project(self.g_proj[0], x)).view(B, T, H, Dv)
         o = self.o_norm(o.to(gate.dtype), gate)
-        y = self.o_proj(o.reshape(B, T, H * Dv))
+        y = _project(self.o_proj, o.reshape(B, T, H * Dv))
         if indices is not None:   # back to the padded layout, zeros where the mask was 0
             padded = y.new_zeros(B0 * S0, y.size(-1))
             padded[indices] = y[0]

@@ -29,14 +29,12 @@ __device__ __forceinline__ float wave_sum(float x) {
   return x + __shfl_xor(x, 32);
 }
 
-// M activation rows, R weight rows per wavefront, P 16-byte pieces of every row in flight per lane;
-// workgroups of WAVES wavefronts.
-template <int M, int R, int P, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void linear_rows_kernel(LinearParams p) {
-  const int lane = threadIdx.x & 63;
-  const int wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
-  const int row0 = wave * R;
-  if (row0 >= p.N) return;   // whole wavefronts only
+// M activation rows, R weight rows per wavefront, P 16-byte pieces of every row in flight per lane; one wavefront
+// per workgroup.
+template <int M, int R, int P>
+__global__ __launch_bounds__(64) void linear_rows_kernel(LinearParams p) {
+  const int lane = threadIdx.x;
+  const int row0 = blockIdx.x * R;
   const int pieces = p.K / 8;
 
   const uint16_t* wr[R];
@@ -96,10 +94,9 @@ __global__ __launch_bounds__(64 * WAVES) void linear_rows_kernel(LinearParams p)
   }
 }
 
-template <int M, int R, int P, int WAVES>
+template <int M, int R, int P>
 static void launch_linear(const LinearParams& p, hipStream_t s) {
-  const int waves = (p.N + R - 1) / R;
-  hipLaunchKernelGGL((linear_rows_kernel<M, R, P, WAVES>), dim3((waves + WAVES - 1) / WAVES), dim3(64 * WAVES), 0, s, p);
+  hipLaunchKernelGGL((linear_rows_kernel<M, R, P>), dim3((p.N + R - 1) / R), dim3(64), 0, s, p);
 }
 
 // Rows per wavefront from a sweep (M = 1, 2, 4; N = 768 ... 50304; K = 768 ... 6144): one row -- as many
@@ -108,9 +105,9 @@ static void launch_linear(const LinearParams& p, hipStream_t s) {
 template <int M>
 static void launch_linear_rows(const LinearParams& p, hipStream_t s) {
   constexpr int P = M <= 2 ? 4 : 2;
-  if (M >= 3 && p.N >= 16384) launch_linear<M, 4, P, 1>(p, s);
-  else if ((M == 2 && p.N >= 16384) || (M >= 3 && p.N >= 4096)) launch_linear<M, 2, P, 1>(p, s);
-  else launch_linear<M, 1, P, 1>(p, s);
+  if (M >= 3 && p.N >= 16384) launch_linear<M, 4, P>(p, s);
+  else if ((M == 2 && p.N >= 16384) || (M >= 3 && p.N >= 4096)) launch_linear<M, 2, P>(p, s);
+  else launch_linear<M, 1, P>(p, s);
 }
 
 }  // namespace daisy

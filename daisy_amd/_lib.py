@@ -16,7 +16,7 @@ import torch
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc", "libdaisy_hip.so")
 _lib: Optional[ctypes.CDLL] = None
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 LINEAR_MAX_ROWS = 8
 STATUS_POSITION_PAST_TABLES = 1
 DECODE_STATIC_SCRATCH_BYTES = 4 << 20
@@ -129,6 +129,17 @@ SIGNATURES = {
         c_int, c_int, c_int, c_int, c_void_p]),                 # T, C, K, apply_silu, stream
     "daisy_linear_rows_fwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,   # x, w, y (+ row strides)
                                        c_int, c_int, c_int, c_void_p]),                          # M, N, K, stream
+    "daisy_attn_layer_step_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "daisy_attn_layer_step_fwd": (c_int, [
+        c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,   # x, w_qkv, w_out (+ row strides)
+        c_void_p, _I64P, c_void_p,                               # ve, ve strides, gate
+        c_void_p, c_void_p, c_int,                              # cos, sin, table_rows
+        c_int, c_void_p, c_void_p, c_float,                     # pos, pos_dev, status, eps
+        c_void_p, _I64P, c_void_p, _I64P, c_int,                # k_ring, v_ring (+strides), ring is fp16
+        c_void_p, c_int64,                                      # y (+ row stride)
+        c_int, c_int, c_int, c_int, c_int,                      # B, H, D, dim, ring_rows
+        c_float, c_int,                                         # scale, nsplit
+        c_void_p, c_size_t, c_void_p]),                         # workspace, bytes, stream
     "daisy_qkv_prep_fwd": (c_int, [
         c_void_p, _I64P, c_void_p, _I64P, c_void_p, _I64P,         # q, k, v (+ strides)
         c_void_p, _I64P, c_void_p,                               # ve, ve strides, gate

@@ -560,17 +560,26 @@ class CausalSelfAttention(nn.Module):
         ``ops.attn_step``.  Returns the new rows as views of the ring, or ``None, None`` when only
         the device knows the position."""
         B, H, D = x.size(0), self.num_heads, self.head_dim
-        qkv = _step_linear(x.to(self.qkvo_w.dtype), self.qkvo_w[:3].flatten(end_dim=1)).view(B, 3 * H, D)
+        x = x.to(self.qkvo_w.dtype)
         ve_rows = gate = None
         if self.receives_ve:
             torch._assert(ve is not None, "ve must be provided when receives_ve=True")
             ve_rows = ve.to(torch.bfloat16).view(B, H, D)
             gate = torch.sigmoid(self.g_ve.detach()).to(torch.bfloat16).float().reshape(1)
-        o = ops.attn_step(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], ring.k, ring.v, pos,
-                          cos=self.rotary.cos, sin=self.rotary.sin, eps=NORM_EPS_BF16, ve=ve_rows, gate=gate,
-                          scale=self.attn_scale, status=ring.status if isinstance(pos, Tensor) else None)
-        ring.mark_written()
-        y = _step_linear(o.reshape(B, 1, self.m_dim), self.qkvo_w[3])
+        status = ring.status if isinstance(pos, Tensor) else None
+        w_qkv, w_out = self.qkvo_w[:3].flatten(end_dim=1), self.qkvo_w[3]
+        if B <= STEP_ROWS_KERNEL_MAX and x.is_contiguous() and H * D == self.m_dim and ops.linear_rows_ok(x, w_qkv):
+            # a few sequences: both projections and the attention step go out in one call
+            y = ops.attn_layer_step(x, w_qkv, w_out, ring.k, ring.v, pos, cos=self.rotary.cos, sin=self.rotary.sin,
+                                    eps=NORM_EPS_BF16, ve=ve_rows, gate=gate, scale=self.attn_scale, status=status)
+            ring.mark_written()
+        else:
+            qkv = _step_linear(x, w_qkv).view(B, 3 * H, D)
+            o = ops.attn_step(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], ring.k, ring.v, pos,
+                              cos=self.rotary.cos, sin=self.rotary.sin, eps=NORM_EPS_BF16, ve=ve_rows, gate=gate,
+                              scale=self.attn_scale, status=status)
+            ring.mark_written()
+            y = _step_linear(o.reshape(B, 1, self.m_dim), w_out)
         if isinstance(pos, Tensor):
             return y, None, None
         slot = pos % ring.W

@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_NAME = "libdaisy_hip.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
-SOURCES = ["abi.hip", "decode.hip", "prefill.hip", "kda.hip", "kda_step.hip", "prep.hip", "kimi.hip", "linear.hip"]
+SOURCES = ["abi.hip", "decode.hip", "prefill.hip", "kda.hip", "kda_step.hip", "prep.hip", "kimi.hip", "linear.hip", "layer_step.hip"]
 # Diagnostic kernels of the benchmark (matrix-pipe and read-stream ceilings): not part of the product.  Their source
 # sits next to bench.py at the repository root and is built into a library of its own there, which only bench.py loads.
 ROOT = os.path.dirname(os.path.dirname(CSRC))

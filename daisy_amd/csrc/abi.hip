@@ -16,4 +16,4 @@ void set_error(const char* fmt, ...) {
 
 extern "C" const char* daisy_last_error(void) { return daisy::g_err; }
 
-extern "C" int daisy_abi_version(void) { return 4; }
+extern "C" int daisy_abi_version(void) { return 5; }

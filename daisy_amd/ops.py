@@ -346,6 +346,66 @@ def attn_step(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, k_ring: torch.T
     return out
 
 
+def attn_layer_step(x: torch.Tensor, w_qkv: torch.Tensor, w_out: torch.Tensor, k_ring: torch.Tensor,
+                    v_ring: torch.Tensor, pos: Union[int, torch.Tensor], *, cos: torch.Tensor, sin: torch.Tensor,
+                    eps: float, ve: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                    scale: float = ATTN_SCALE, nsplit: int = 0, status: Optional[torch.Tensor] = None,
+                    workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One decode step of an attention layer in one call (``daisy_attn_layer_step_fwd``): QKV projection of
+    ``x [B, dim]`` (or ``[B, 1, dim]``) with ``w_qkv [3*H*D, dim]``, the one-launch attention step of ``attn_step`` on
+    the rings ``[B, H, W, D]``, output projection with ``w_out [dim, H*D]``.  bf16 throughout (the rings may be fp16),
+    ``B`` at most ``_lib.LINEAR_MAX_ROWS``.  Returns ``y`` shaped like ``x``.  Same results as ``linear_rows``,
+    ``attn_step``, ``linear_rows`` one after the other; what it saves is the host's time between the launches."""
+    pos_dev = pos if isinstance(pos, torch.Tensor) else None
+    dev = _lib.require_gpu(x, w_qkv, w_out, k_ring, v_ring, cos, sin, ve, gate, pos_dev, status, workspace)
+    _check_status(status)
+    if x.dtype != torch.bfloat16 or w_qkv.dtype != torch.bfloat16 or w_out.dtype != torch.bfloat16:
+        raise TypeError("attn_layer_step: x, w_qkv and w_out must be bf16")
+    if k_ring.dtype != v_ring.dtype or k_ring.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"attn_layer_step: the rings must both be bf16 or both fp16, got {k_ring.dtype}, {v_ring.dtype}")
+    if k_ring.dim() != 4 or v_ring.shape != k_ring.shape or k_ring.stride(3) != 1 or v_ring.stride(3) != 1:
+        raise ValueError("attn_layer_step: k_ring, v_ring must be [B, H, W, D] with a contiguous last dim")
+    B, H, W, D = k_ring.shape
+    dim = x.shape[-1]
+    if x.numel() != B * dim or w_qkv.shape != (3 * H * D, dim) or w_out.shape != (dim, H * D):
+        raise ValueError(f"attn_layer_step: x {tuple(x.shape)}, w_qkv {tuple(w_qkv.shape)}, w_out {tuple(w_out.shape)} do not "
+                         f"fit rings of {B} x {H} x {D}")
+    if not (x.is_contiguous() and w_qkv.stride(1) == 1 and w_out.stride(1) == 1):
+        raise ValueError("attn_layer_step: x must be contiguous and the weights' last dims contiguous")
+    for name, t in (("cos", cos), ("sin", sin)):
+        if t.dtype != torch.float32 or t.dim() != 2 or t.shape[1] != D // 2 or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous fp32 [rows, {D // 2}] table, got {tuple(t.shape)} {t.dtype}")
+    if pos_dev is not None:
+        if pos_dev.dtype != torch.int32 or pos_dev.numel() != 1:
+            raise ValueError("a device position must be a one-element int32 tensor")
+    else:
+        torch._assert(0 <= pos < cos.shape[0], f"Rotary buffers too small {cos.shape[0]} < {pos + 1}")
+    if (ve is None) != (gate is None):
+        raise ValueError("ve and gate must be given together")
+    ve_strides = None
+    if ve is not None:
+        if ve.dtype != torch.bfloat16 or ve.shape != (B, H, D) or ve.stride(2) != 1:
+            raise ValueError(f"ve must be bf16 [{B}, {H}, {D}] with a contiguous last dim, got {tuple(ve.shape)} {ve.dtype}")
+        if gate.dtype != torch.float32 or gate.numel() != 1:
+            raise ValueError("gate must be a one-element fp32 tensor")
+        ve_strides = _lib.strides(ve, (0, 1))
+    lib = _lib.load()
+    need = int(lib.daisy_attn_layer_step_workspace_bytes(B, H, D, W, nsplit))
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    y = torch.empty_like(x)
+    with _lib.on_device(dev):
+        rc = lib.daisy_attn_layer_step_fwd(
+            x.data_ptr(), dim, w_qkv.data_ptr(), w_qkv.stride(0), w_out.data_ptr(), w_out.stride(0),
+            _lib.ptr(ve), ve_strides, _lib.ptr(gate), cos.data_ptr(), sin.data_ptr(), int(cos.shape[0]),
+            0 if pos_dev is not None else int(pos), _lib.ptr(pos_dev), _lib.ptr(status), float(eps),
+            k_ring.data_ptr(), _lib.strides(k_ring, (0, 1, 2)), v_ring.data_ptr(), _lib.strides(v_ring, (0, 1, 2)),
+            1 if k_ring.dtype == torch.float16 else 0, y.data_ptr(), dim, B, H, D, dim, W, float(scale), int(nsplit),
+            workspace.data_ptr(), workspace.numel() * workspace.element_size(), _lib.current_stream(dev))
+    _lib.check(rc, "daisy_attn_layer_step_fwd")
+    return y
+
+
 def _check_status(status: Optional[torch.Tensor]) -> None:
     if status is not None and (status.dtype != torch.int32 or status.numel() != 1):
         raise ValueError("status must be a one-element int32 tensor")

@@ -391,6 +391,32 @@ int daisy_qkv_prep_fwd_at(const void* q, const int64_t* q_strides,
 int daisy_linear_rows_fwd(const void* x, int64_t x_row_stride, const void* w, int64_t w_row_stride,
                           void* y, int64_t y_row_stride, int M, int N, int K, void* stream);
 
+/* One decode step of an attention layer in one call: CausalSelfAttention.step
+ * (models/daisy/attention.py:181-202) from its input rows to its output rows,
+ *     qkv = x W_qkv^T  (daisy_linear_rows_fwd);   o = daisy_attn_step_fwd on the three thirds of qkv;
+ *     y = o W_out^T    (daisy_linear_rows_fwd),
+ * as three launches (four with split partials) on `stream`.  Results are those of the three calls.
+ * x      : bf16 [B, dim], row stride x_row_stride;  y : bf16 [B, dim], row stride y_row_stride;  B <= 8.
+ * w_qkv  : bf16 [3*H*D, dim] (qkvo_w[:3] flattened: q rows, then k rows, then v rows);  w_out : bf16 [dim, H*D].
+ * ve, gate, cos, sin, table_rows, pos, pos_dev, status, eps, the ring cache, cache_is_f16, ring_rows,
+ * scale, nsplit : as for daisy_attn_step_fwd (ve: bf16 [B, H, D] with {batch, head} strides).
+ * workspace : >= daisy_attn_layer_step_workspace_bytes(B, H, D, ring_rows, nsplit) bytes, 256-byte aligned
+ *          (the projected rows, the attention output and the split partials; sized for the whole ring).
+ */
+size_t daisy_attn_layer_step_workspace_bytes(int B, int H, int D, int ring_rows, int nsplit);
+int daisy_attn_layer_step_fwd(const void* x, int64_t x_row_stride,
+                              const void* w_qkv, int64_t w_qkv_row_stride,
+                              const void* w_out, int64_t w_out_row_stride,
+                              const void* ve, const int64_t* ve_strides, const float* gate,
+                              const float* cos, const float* sin, int table_rows,
+                              int pos, const int32_t* pos_dev, int32_t* status, float eps,
+                              void* k_cache, const int64_t* k_cache_strides,
+                              void* v_cache, const int64_t* v_cache_strides, int cache_is_f16,
+                              void* y, int64_t y_row_stride,
+                              int B, int H, int D, int dim, int ring_rows,
+                              float scale, int nsplit,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------
  * The KDA layer's elementwise neighbours (models/daisy/attention_kimi.py:155-158: three
  * ShortConvolution modules in front of chunk_kda; :136-137: the gated RMS norm behind it; both

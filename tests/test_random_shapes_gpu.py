@@ -57,15 +57,15 @@ def test_prefill_random_shapes(seed):
             assert_close_bf16(k_rot, kr, f"rotated keys (case {it})")
 
 
-@pytest.mark.parametrize("seed", [21])
+@pytest.mark.parametrize("seed", [21, 22])
 def test_decode_random_rings(seed):
     rng = random.Random(seed)
     pos = torch.zeros(1, dtype=torch.int32, device="cuda")
     for it in range(80):
         B, H, D = rng.choice([1, 2, 5]), rng.choice([1, 3, 4]), rng.choice([128, 128, 64])
-        W = rng.choice([1, 2, 7, 31, 32, 33, 64, 200, 255, 256, 257, 511, 512, 513, 1024, 1500, 2048])
+        W = rng.choice([1, 2, 7, 31, 32, 33, 63, 64, 65, 127, 128, 129, 200, 255, 256, 257, 511, 512, 513, 1024, 1500, 2048, 4096, 5000])
         t = rng.choice([0, 1, W - 1, W, W + 1, 2 * W, rng.randrange(0, 3 * W + 1), rng.randrange(0, W + 1)])
-        nsplit, on_device = rng.choice([0, 0, 1, 2, 3, 7]), rng.random() < 0.5
+        nsplit, on_device = rng.choice([0, 0, 1, 2, 3, 7, 16, 40, 64]), rng.random() < 0.5
         say(f"decode sweep case {it}: B{B} H{H} D{D} W{W} t{t} nsplit{nsplit} position on device {on_device}")
         g = torch.Generator().manual_seed(seed * 7919 + it)
         kc, vc = (torch.randn(B, H, W, D, generator=g).bfloat16() for _ in range(2))

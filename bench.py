@@ -804,8 +804,18 @@ def bench_next_rows(steps, warmup):
         with torch.cuda.graph(graph):
             layer.step(x1, None, None, 64, None, None)
         ms_step_graph = time_gpu(graph.replay, 32, 4)
+        del graph
+        # one sequence (the generator's regime): the layer's bias-free projections read their weights through the few-rows kernel
+        layer.reset_history()
+        layer.prefill(xs[:1], None)
+        ms_step_b1 = time_gpu(lambda: layer.step(x1[:1], None, None, 64, None, None), 64, 16)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            layer.step(x1[:1], None, None, 64, None, None)
+        ms_step_b1_graph = time_gpu(graph.replay, 64, 8)
     out["kimi_layer_dim2048_H16"] = {"forward_ms_B4_T8192": ms_layer, "forward_ms_first_steps_from_idle": ms_layer_first, "step_ms_B64": ms_step,
-                                     "step_ms_B64_recorded_graph": ms_step_graph}
+                                     "step_ms_B64_recorded_graph": ms_step_graph, "step_ms_B1": ms_step_b1,
+                                     "step_ms_B1_recorded_graph": ms_step_b1_graph}
     del graph
     return out
 

@@ -109,6 +109,7 @@ class Generator:
         self.vocab_size = model.embed.num_embeddings
         self.eos_token_id = torch.tensor(eos, device=self.device)
         self.rep_p_t = torch.tensor(repetition_penalty, device=self.device, dtype=dtype)
+        self._rep_p_host = float(repetition_penalty)
         self._one = torch.tensor(1, device=self.device, dtype=dtype)
         self.sample = sample_token
         self.apply_repetition_penalty = penalise_repeats
@@ -170,6 +171,7 @@ class Generator:
 
     def set_repetition_penalty(self, repetition_penalty: float):
         self.rep_p_t = torch.tensor(repetition_penalty, device=self.rep_p_t.device, dtype=self.rep_p_t.dtype)
+        self._rep_p_host = float(repetition_penalty)
         return self
 
     def reset_history(self):
@@ -183,6 +185,14 @@ class Generator:
 
     def _trim(self, logits: Tensor) -> Tensor:
         return logits.to(self.dtype)[..., :self.vocab_size]
+
+    def _penalised(self, logits: Tensor, recent: Tensor) -> Tensor:
+        """The repetition penalty on ``logits``.  A strength of exactly 1 leaves every logit as it is (``x * 1``,
+        ``x / 1``), so the dozen small launches of the stock routine are skipped then; a routine put in its place
+        (``apply_repetition_penalty`` is an attribute, as in the reference) is always called."""
+        if self._rep_p_host == 1.0 and self.apply_repetition_penalty is penalise_repeats:
+            return logits
+        return self.apply_repetition_penalty(logits, recent, self.rep_p_t, self._one)
 
     # -- model calls -----------------------------------------------------------------------
     def _prefill(self, prompt_ids: Tensor) -> Tensor:
@@ -253,7 +263,7 @@ class Generator:
         self._sync()
         t_prompt = time.perf_counter()
         for produced in range(1, max_new_tokens + 1):
-            scores = self.apply_repetition_penalty(logits[-1], self.history[-_PENALTY_LOOKBACK:], self.rep_p_t, self._one)
+            scores = self._penalised(logits[-1], self.history[-_PENALTY_LOOKBACK:])
             token = self.sample(scores, self.temperature, self.top_k, self.top_p)
             if token == self.eos_token_id:
                 break
@@ -302,7 +312,7 @@ class Generator:
         done = torch.zeros(B, dtype=torch.bool, device=self.device)
         for produced in range(1, max_new_tokens + 1):
             scores = self._trim(logits)
-            scores = self.apply_repetition_penalty(scores, seen[:, max(n_seen - _PENALTY_LOOKBACK, 0):n_seen], self.rep_p_t, self._one)
+            scores = self._penalised(scores, seen[:, max(n_seen - _PENALTY_LOOKBACK, 0):n_seen])
             token = self.sample(scores, self.temperature, self.top_k, self.top_p)
             token = torch.where(done, eos, token)
             done |= token == eos

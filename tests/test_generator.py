@@ -146,3 +146,26 @@ def test_sampling_helpers():
     l2 = torch.tensor([0.95, 0.94, 0.93, 0.0, 0.0, 0.0, 0.0, 0.0])
     pen = gen.apply_repetition_penalty(l2, gen.history[-128:], gen.rep_p_t.float(), gen._one)
     assert int(torch.argmax(pen)) == 0                                   # tokens 1 and 2 were seen, 0 was not
+
+
+def test_a_penalty_of_one_is_the_identity_and_skipped():
+    """A repetition penalty of exactly 1 changes no logit (inference/generate.py:47-58: scale = 1 ** count), so the
+    generator does not launch the routine for it -- unless a caller has put a routine of their own in its place."""
+    from daisy_amd.generate import penalise_repeats
+    model = OneHotModel(8, layers=1)
+    gen = Generator(model, window=4, seed=1, device=torch.device("cpu"), dtype=torch.bfloat16)
+    recent = torch.tensor([1, 2, 3, 2, 1])
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
+        logits = torch.tensor([0.1, -0.9, 0.5, -1.0, 3.0, 0.0, -7.5, 2.25], dtype=dt)
+        assert torch.equal(penalise_repeats(logits, recent, torch.tensor(1.0, dtype=dt)), logits)
+        assert gen._penalised(logits, recent) is logits
+    calls = []
+    gen.apply_repetition_penalty = lambda lg, prev, strength, one: (calls.append(float(strength)), lg + 1)[1]
+    out = gen._penalised(torch.zeros(8), recent)
+    assert calls == [1.0] and torch.equal(out, torch.ones(8))
+    gen.apply_repetition_penalty = penalise_repeats
+    gen.set_repetition_penalty(1.3)
+    want = penalise_repeats(torch.ones(8, dtype=torch.bfloat16), recent, gen.rep_p_t, gen._one)
+    assert torch.equal(gen._penalised(torch.ones(8, dtype=torch.bfloat16), recent), want) and not torch.equal(want, torch.ones(8, dtype=torch.bfloat16))
+    gen.set_repetition_penalty(1.0)
+    assert gen._penalised(want, recent) is want

@@ -312,7 +312,7 @@ class Rotary(nn.Module):
 STEP_ROWS_KERNEL_MAX = 4
 
 
-def _step_linear(x: Tensor, w: Tensor) -> Tensor:
+def step_linear(x: Tensor, w: Tensor) -> Tensor:
     """``F.linear(x, w)`` for the activations of a decode step (models/daisy/attention.py:119-120, :201)."""
     if x.numel() <= STEP_ROWS_KERNEL_MAX * x.shape[-1] and ops.linear_rows_ok(x, w):
         return ops.linear_rows(x, w)
@@ -361,7 +361,7 @@ class CausalSelfAttention(nn.Module):
         """QKV projection + RMS norm of q, k and v (no RoPE); ``[B, T, H, D]`` views."""
         B, T = x.size(0), x.size(1)
         x = x.to(self.qkvo_w.dtype)
-        qkv = _step_linear(x, self.qkvo_w[:3].flatten(end_dim=1)).view(B, T, 3 * self.num_heads, self.head_dim)
+        qkv = step_linear(x, self.qkvo_w[:3].flatten(end_dim=1)).view(B, T, 3 * self.num_heads, self.head_dim)
         q, k, v = qkv.chunk(3, dim=-2)
         return norm(q), norm(k), norm(v)
 
@@ -386,7 +386,7 @@ class CausalSelfAttention(nn.Module):
         ``k_out`` / ``v_out``: strided ``[B, T, H, D]`` views that receive k and v (e.g. slots of a ring cache)."""
         B, T = x.size(0), x.size(1)
         x = x.to(self.qkvo_w.dtype)
-        qkv = _step_linear(x, self.qkvo_w[:3].flatten(end_dim=1)).view(B, T, 3 * self.num_heads, self.head_dim)
+        qkv = step_linear(x, self.qkvo_w[:3].flatten(end_dim=1)).view(B, T, 3 * self.num_heads, self.head_dim)
         q, k, v = qkv.chunk(3, dim=-2)
         gate = None
         if self.receives_ve:
@@ -533,7 +533,7 @@ class CausalSelfAttention(nn.Module):
                                      write_back=False, scale=self.attn_scale)
             k_new, v_new = k_new.to(dtype), v_new.to(dtype)
         y = o.reshape(B, 1, self.m_dim).to(dtype)
-        y = _step_linear(y, self.qkvo_w[3])
+        y = step_linear(y, self.qkvo_w[3])
         return y, k_new, v_new
 
     def _step_f32(self, q, k, v, k_ctx, v_ctx, pos, window, cos_row, sin_row):
@@ -574,12 +574,12 @@ class CausalSelfAttention(nn.Module):
                                     eps=NORM_EPS_BF16, ve=ve_rows, gate=gate, scale=self.attn_scale, status=status)
             ring.mark_written()
         else:
-            qkv = _step_linear(x, w_qkv).view(B, 3 * H, D)
+            qkv = step_linear(x, w_qkv).view(B, 3 * H, D)
             o = ops.attn_step(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], ring.k, ring.v, pos,
                               cos=self.rotary.cos, sin=self.rotary.sin, eps=NORM_EPS_BF16, ve=ve_rows, gate=gate,
                               scale=self.attn_scale, status=status)
             ring.mark_written()
-            y = _step_linear(o.reshape(B, 1, self.m_dim), w_out)
+            y = step_linear(o.reshape(B, 1, self.m_dim), w_out)
         if isinstance(pos, Tensor):
             return y, None, None
         slot = pos % ring.W

@@ -32,7 +32,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from . import ops
-from .attention import _step_linear
+from .attention import step_linear
 from .kda import chunk_kda, fused_kda_gate, fused_recurrent_kda
 
 
@@ -81,7 +81,7 @@ class GatedRMSNorm(nn.Module):
 def _project(lin: nn.Linear, x: Tensor) -> Tensor:
     """``lin(x)``; a bias-free projection of a decode step's few rows reads its weights through the few-rows kernel."""
     if lin.bias is None:
-        return _step_linear(x, lin.weight)
+        return step_linear(x, lin.weight)
     return lin(x)
 
 

@@ -26,7 +26,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor
 
-from .attention import CausalSelfAttention, WindowMask, _step_linear, build_window_mask
+from .attention import CausalSelfAttention, WindowMask, step_linear, build_window_mask
 from .functional import norm
 from .kv_cache import KVCache
 
@@ -157,7 +157,7 @@ def _walk_step(model, token_ids: Tensor, cache: KVCache, pos, status: Optional[T
             torch._assert(not on_device, "a recorded step needs attention layers that write the ring themselves")
             cache.write(i, k_new.to(cache.dtype), v_new.to(cache.dtype))
     x = norm(x)
-    return _step_linear(x.flatten(end_dim=1).bfloat16(), model.lm_head_w.bfloat16()).float()
+    return step_linear(x.flatten(end_dim=1).bfloat16(), model.lm_head_w.bfloat16()).float()
 
 
 class GraphedStep:

@@ -313,8 +313,10 @@ STEP_ROWS_KERNEL_MAX = 4
 
 
 def step_linear(x: Tensor, w: Tensor) -> Tensor:
-    """``F.linear(x, w)`` for the activations of a decode step (models/daisy/attention.py:119-120, :201)."""
-    if x.numel() <= STEP_ROWS_KERNEL_MAX * x.shape[-1] and ops.linear_rows_ok(x, w):
+    """``F.linear(x, w)`` for the activations of a decode step (models/daisy/attention.py:119-120, :201).
+    The kernel has no backward: where autograd would record the product, the library op stays."""
+    if (x.numel() <= STEP_ROWS_KERNEL_MAX * x.shape[-1] and ops.linear_rows_ok(x, w)
+            and not (torch.is_grad_enabled() and (x.requires_grad or w.requires_grad))):
         return ops.linear_rows(x, w)
     return F.linear(x, w)
 
@@ -568,7 +570,8 @@ class CausalSelfAttention(nn.Module):
             gate = torch.sigmoid(self.g_ve.detach()).to(torch.bfloat16).float().reshape(1)
         status = ring.status if isinstance(pos, Tensor) else None
         w_qkv, w_out = self.qkvo_w[:3].flatten(end_dim=1), self.qkvo_w[3]
-        if B <= STEP_ROWS_KERNEL_MAX and x.is_contiguous() and H * D == self.m_dim and ops.linear_rows_ok(x, w_qkv):
+        if (B <= STEP_ROWS_KERNEL_MAX and x.is_contiguous() and H * D == self.m_dim and ops.linear_rows_ok(x, w_qkv)
+                and not (torch.is_grad_enabled() and (x.requires_grad or w_qkv.requires_grad))):
             # a few sequences: both projections and the attention step go out in one call
             y = ops.attn_layer_step(x, w_qkv, w_out, ring.k, ring.v, pos, cos=self.rotary.cos, sin=self.rotary.sin,
                                     eps=NORM_EPS_BF16, ve=ve_rows, gate=gate, scale=self.attn_scale, status=status)

@@ -197,7 +197,7 @@ __device__ __forceinline__ void merge_state(SoftmaxState& a, const SoftmaxState&
 //
 // Order of the memory instructions: the new token's rows and the table rows (raw), then the first two
 // sets of cache rows, and only then the arithmetic on the new rows; inside the loop a register set is
-// loaded again as soon as it has been used.  A wavefront so keeps 2 * kDecodeUnroll KiB of cache rows
+// loaded again as soon as it has been used.  A wavefront so keeps 2 to 4 * kDecodeUnroll KiB of cache rows
 // in flight from its first instructions to its last row: with a few hundred workgroups on the chip
 // (one sequence, a dozen heads) the launch is a handful of memory round trips long, and every trip
 // spent with nothing in flight shows.

@@ -32,6 +32,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from . import ops
+from . import attention as _attention
 from .attention import step_linear
 from .kda import chunk_kda, fused_kda_gate, fused_recurrent_kda
 
@@ -147,6 +148,38 @@ class KimiLinearSelfAttention(nn.Module):
         # and writes stay the same for the life of the module, also when calls of different batch
         # sizes alternate (a recorded step checks the addresses before every replay all the same).
         self._state_homes: dict = {}
+        # The six projections that read the layer's input, stacked into one matrix for decode steps (see
+        # _input_projections); rebuilt when one of the weights moves or changes.
+        self._stacked_w: Optional[Tensor] = None
+        self._stacked_key = None
+
+    def _input_projections(self, x: Tensor):
+        """``q_proj(x), k_proj(x), v_proj(x), f_proj[0](x), g_proj[0](x), b_proj(x)``.  For the few rows of a decode
+        step (no autograd, bf16 on the GPU) the six weight matrices are kept stacked and read by ONE launch of the
+        few-rows kernel instead of six; its rows are computed one by one, so every output equals the separate call's
+        bit for bit.  The stack (as large as the six weights) is made outside stream capture and follows the
+        parameters' addresses and versions."""
+        lins = (self.q_proj, self.k_proj, self.v_proj, self.f_proj[0], self.g_proj[0], self.b_proj)
+        rows = x.numel() // x.shape[-1]
+        fused = (rows <= _attention.STEP_ROWS_KERNEL_MAX and x.is_cuda and x.dtype == torch.bfloat16
+                 and not (torch.is_grad_enabled() and (x.requires_grad or any(l.weight.requires_grad for l in lins)))
+                 and all(l.bias is None and l.weight.dtype == torch.bfloat16 for l in lins))
+        if fused:
+            key = tuple((l.weight.data_ptr(), l.weight._version) for l in lins)
+            if key != self._stacked_key:
+                if torch.cuda.is_current_stream_capturing():
+                    fused = False          # not the moment to build it: the separate launches are recorded
+                else:
+                    with torch.no_grad():
+                        w = torch.cat([l.weight for l in lins], 0)
+                        if w.shape[0] % 8:  # whole 16-byte pieces per output row of a batch
+                            w = torch.cat([w, w.new_zeros(8 - w.shape[0] % 8, w.shape[1])], 0)
+                    self._stacked_w, self._stacked_key = w.contiguous(), key
+        if fused and ops.linear_rows_ok(x, self._stacked_w):
+            sizes = [l.weight.shape[0] for l in lins]
+            y = ops.linear_rows(x, self._stacked_w)
+            return y[..., :sum(sizes)].split(sizes, dim=-1)
+        return tuple(_project(l, x) for l in lins)
 
     def _apply(self, fn, recurse=True):
         # The decay parameters stay fp32 under module-wide casts, as the reference creates them.
@@ -200,23 +233,24 @@ class KimiLinearSelfAttention(nn.Module):
         B, T, _ = x.shape
         state = self._recurrent_state if use_cache else None
         convs = self._conv_state if (use_cache and self._conv_state is not None) else (None, None, None)
+        q_lin, k_lin, v_lin, f_low, g_low, b_lin = self._input_projections(x)
         if self.use_short_conv:
             # a decode step shifts its windows in place (same tensors, same addresses, every step)
             shift = (use_cache and T == 1 and cu_seqlens is None
                      and all(c is not None and c.dtype == torch.bfloat16 and c.is_contiguous() for c in convs))
-            q, cq = self.q_conv1d(_project(self.q_proj, x), convs[0], use_cache, cu_seqlens, shift)
-            k, ck = self.k_conv1d(_project(self.k_proj, x), convs[1], use_cache, cu_seqlens, shift)
-            v, cv = self.v_conv1d(_project(self.v_proj, x), convs[2], use_cache, cu_seqlens, shift)
+            q, cq = self.q_conv1d(q_lin, convs[0], use_cache, cu_seqlens, shift)
+            k, ck = self.k_conv1d(k_lin, convs[1], use_cache, cu_seqlens, shift)
+            v, cv = self.v_conv1d(v_lin, convs[2], use_cache, cu_seqlens, shift)
         else:
-            q, k, v = F.silu(_project(self.q_proj, x)), F.silu(_project(self.k_proj, x)), F.silu(_project(self.v_proj, x))
+            q, k, v = F.silu(q_lin), F.silu(k_lin), F.silu(v_lin)
             cq = ck = cv = None
         q, k, v = q.view(B, T, H, Dk), k.view(B, T, H, Dk), v.view(B, T, H, Dv)
         if self.receives_ve:
             torch._assert(ve is not None, "ve must be provided when receives_ve=True")
             g_x = torch.sigmoid(self.g_ve).to(v.dtype)
             v = g_x * v + (1.0 - g_x) * ve.view_as(v).to(v.dtype)
-        g = fused_kda_gate(_project(self.f_proj[1], _project(self.f_proj[0], x)), self.A_log, Dk, self.dt_bias)
-        beta = torch.sigmoid(_project(self.b_proj, x)).to(torch.float32)
+        g = fused_kda_gate(_project(self.f_proj[1], f_low), self.A_log, Dk, self.dt_bias)
+        beta = torch.sigmoid(b_lin).to(torch.float32)
         if use_cache and T == 1 and state is not None and cu_seqlens is None:
             o, state = fused_recurrent_kda(q, k, v, g, beta, initial_state=state, use_qk_l2norm_in_kernel=True,
                                            inplace_state=True)
@@ -229,7 +263,8 @@ class KimiLinearSelfAttention(nn.Module):
             self._conv_state = tuple(self._store(h, c) for h, c in zip(homes[1:], (cq, ck, cv)))
             self._state_homes[state.shape[0]] = (self._recurrent_state,) + self._conv_state
             self._seen += T
-        gate = self.g_proj[1](_project(self.g_proj[0], x)).view(B, T, H, Dv)
+        # (contiguous rows: the library adds the bias inside the product then, as it does for the reference's tensors)
+        gate = self.g_proj[1](g_low.contiguous()).view(B, T, H, Dv)
         o = self.o_norm(o.to(gate.dtype), gate)
         y = _project(self.o_proj, o.reshape(B, T, H * Dv))
         if indices is not None:   # back to the padded layout, zeros where the mask was 0

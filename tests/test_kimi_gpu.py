@@ -375,3 +375,57 @@ def test_bounds_outside_the_token_range_are_clamped_the_same_way_by_every_packed
     # looked at; for the convolution the point is that the launch completes (run_all synchronises).
     for name in ("chunk", "recurrent"):
         assert bool(torch.isfinite(c[name][1].float()).all()), f"{name}: state with out-of-order bounds"
+
+
+@pytest.mark.parametrize("B", [1, 3])
+def test_stacked_input_projections_equal_the_separate_ones(B):
+    """A decode step of a few sequences reads the six projections of the layer's input through one stacked matrix
+    (models/daisy/attention_kimi.py:99-118 are six separate Linear modules): every output equals the separate
+    launch's bit for bit, the stack follows a weight that changes, and a stale stack is not rebuilt under capture."""
+    from daisy_amd.attention_kimi import _project
+    with torch.no_grad():
+        m = _layer(seed=11).to(DEV)
+        g = torch.Generator().manual_seed(12)
+        x = torch.randn(B, 1, 256, generator=g).bfloat16().to(DEV)
+        lins = (m.q_proj, m.k_proj, m.v_proj, m.f_proj[0], m.g_proj[0], m.b_proj)
+
+        def separate():
+            return tuple(_project(l, x) for l in lins)
+
+        got = m._input_projections(x)
+        assert m._stacked_w is not None and m._stacked_w.shape[0] % 8 == 0
+        assert m._stacked_w.shape[0] >= sum(l.weight.shape[0] for l in lins)
+        for a, b in zip(got, separate()):
+            assert a.shape == b.shape and torch.equal(a, b)
+        m.k_proj.weight.mul_(1.5)                        # in place: same address, new version
+        for a, b in zip(m._input_projections(x), separate()):
+            assert torch.equal(a, b)
+        # the whole step through the stacked matrix equals the step through the separate launches
+        xs = torch.randn(B, 6, 256, generator=g).bfloat16().to(DEV)
+        m.reset_history()
+        m.prefill(xs[:, :3], None, attn_mask=None)
+        y_stacked = [m.step(xs[:, t:t + 1], None, None, t, None, window=None)[0] for t in range(3, 6)]
+        m.reset_history()
+        m._input_projections = lambda inp: tuple(_project(l, inp) for l in lins)
+        m.prefill(xs[:, :3], None, attn_mask=None)
+        y_separate = [m.step(xs[:, t:t + 1], None, None, t, None, window=None)[0] for t in range(3, 6)]
+        del m._input_projections
+        for a, b in zip(y_stacked, y_separate):
+            assert torch.equal(a, b)
+        # more rows than the few-rows kernel is used for: the separate library products
+        wide = torch.randn(8, 1, 256, generator=g).bfloat16().to(DEV)
+        for a, l in zip(m._input_projections(wide), lins):
+            assert torch.equal(a, l(wide))
+        # a stack that has gone stale while the stream is capturing is left alone
+        m.v_proj.weight.mul_(0.5)
+        key_before = m._stacked_key
+        graph = torch.cuda.CUDAGraph()
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            with torch.cuda.graph(graph, stream=s):
+                captured = m._input_projections(x)
+        assert m._stacked_key == key_before
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(captured, separate()):
+            assert torch.equal(a, b)

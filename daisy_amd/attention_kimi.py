@@ -153,6 +153,13 @@ class KimiLinearSelfAttention(nn.Module):
         self._stacked_w: Optional[Tensor] = None
         self._stacked_key = None
 
+    def replay_guard(self) -> tuple:
+        """What a recorded decode step of this layer depends on besides the tensors it updates in place: the stacked
+        copy of the input projections is a snapshot, so a recording is good for as long as the six weights keep their
+        addresses and versions (``core.GraphedStep`` compares this before every replay and records again otherwise)."""
+        lins = (self.q_proj, self.k_proj, self.v_proj, self.f_proj[0], self.g_proj[0], self.b_proj)
+        return tuple((l.weight.data_ptr(), l.weight._version) for l in lins)
+
     def _input_projections(self, x: Tensor):
         """``q_proj(x), k_proj(x), v_proj(x), f_proj[0](x), g_proj[0](x), b_proj(x)``.  For the few rows of a decode
         step (no autograd, bf16 on the GPU) the six weight matrices are kept stacked and read by ONE launch of the
@@ -165,7 +172,7 @@ class KimiLinearSelfAttention(nn.Module):
                  and not (torch.is_grad_enabled() and (x.requires_grad or any(l.weight.requires_grad for l in lins)))
                  and all(l.bias is None and l.weight.dtype == torch.bfloat16 for l in lins))
         if fused:
-            key = tuple((l.weight.data_ptr(), l.weight._version) for l in lins)
+            key = self.replay_guard()
             if key != self._stacked_key:
                 if torch.cuda.is_current_stream_capturing():
                     fused = False          # not the moment to build it: the separate launches are recorded

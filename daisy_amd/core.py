@@ -196,8 +196,10 @@ class GraphedStep:
                 for t in blk.attn.state_tensors()]
 
     def _addresses(self) -> tuple:
-        """Every address the recorded launches carry besides the parameters: the ring and the layers' own state."""
-        return (self.cache.k.data_ptr(), self.cache.v.data_ptr()) + tuple(t.data_ptr() for t in self._stateful_tensors())
+        """Every address the recorded launches carry besides the parameters: the ring and the layers' own state; and
+        what layers that read a snapshot of their parameters say the snapshot depends on (``replay_guard``)."""
+        guards = tuple(blk.attn.replay_guard() for blk in self.model.blocks if hasattr(getattr(blk, "attn", None), "replay_guard"))
+        return (self.cache.k.data_ptr(), self.cache.v.data_ptr()) + tuple(t.data_ptr() for t in self._stateful_tensors()) + guards
 
     def check(self) -> None:
         """Raises what the kernels of the replayed steps reported (a position past the rotary tables).

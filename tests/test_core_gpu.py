@@ -303,6 +303,34 @@ def test_recorded_step_with_a_kda_layer():
         assert torch.equal(want, got)
 
 
+def test_recorded_step_follows_a_weight_that_changes_in_place():
+    """The KDA layer's decode step reads a stacked snapshot of six of its weights; a recording made before one of
+    them changed in place (a state dict loaded into the same model) must not go on replaying the old snapshot."""
+    import copy
+    from daisy_amd import KimiLinearSelfAttention
+    with torch.no_grad():
+        model = _Core(window=48, max_seq_len=512)
+        torch.manual_seed(2)
+        model.blocks[0].attn = KimiLinearSelfAttention(256, 2, 512, 128).bfloat16()
+        model = model.to(DEV)
+        twin = copy.deepcopy(model)
+        B, T = 1, 20
+        ids = torch.randint(2, 96, (B, T + 12), generator=torch.Generator().manual_seed(4)).to(DEV)
+        eager = KVCache(4, B, 2, 48, 128, DEV, torch.bfloat16)
+        replayed = KVCache(4, B, 2, 48, 128, DEV, torch.bfloat16)
+        core.prefill(model, ids[:, :T], eager)
+        core.prefill(twin, ids[:, :T], replayed)
+        graphed = core.GraphedStep(twin, replayed)
+        for s in range(4):
+            _close(graphed(ids[:, T + s]), core.step(model, ids[:, T + s], eager), f"replay {s}", tol=1e-2)
+        first_graph = graphed._graph
+        for m in (model, twin):                      # the same in-place change on both
+            m.blocks[0].attn.v_proj.weight.mul_(-1.0)
+        for s in range(4, 8):
+            _close(graphed(ids[:, T + s]), core.step(model, ids[:, T + s], eager), f"replay {s} after the change", tol=1e-2)
+        assert graphed._graph is not first_graph, "the step was recorded again"
+
+
 def test_generator_single_sequence_with_recorded_steps():
     """Generator.generate (the reference's one-sequence loop) with record_steps and direct_prefill: the
     same tokens as through model.prefill + bulk_write_packed and steps launched kernel by kernel, for
